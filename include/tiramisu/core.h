@@ -1,0 +1,436 @@
+// Front-end of the Tiramisu embedded compiler, re-provided without Halide on top of isl:
+// function / buffer / computation / input / constant, the scheduling commands, the GPU
+// mapping commands and codegen().  Interface follows include/tiramisu/core.h of the
+// reference (function :189, buffer :1424, computation :1863, input :4952,
+// constant :5212); the implementation is new and lowers to HIP for gfx950.
+#ifndef TIRAMISU_AMD_CORE_H
+#define TIRAMISU_AMD_CORE_H
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <tuple>
+#include <unordered_map>
+#include <vector>
+
+#include <tiramisu/debug.h>
+#include <tiramisu/expr.h>
+#include <tiramisu/type.h>
+
+struct isl_ctx;
+struct isl_set;
+struct isl_map;
+struct isl_ast_node;
+
+namespace tiramisu {
+
+class function;
+class computation;
+class buffer;
+class constant;
+class input;
+class block;
+namespace lir { struct program; }
+
+/** Start a new implicit function called \p name (reference: tiramisu_core.cpp:60-70). */
+void init(std::string name);
+void init();
+
+/** Generate code for the implicit function.  \p arguments are the buffers of the generated
+  * function's signature, in order.  \p gen_gpu true selects the GPU back-end (HIP, gfx950);
+  * false selects the CPU back-end, which must be linked separately (it lives with the
+  * parity oracle and is not part of the GPU product library).
+  * Reference: tiramisu_core.cpp:88-98, tiramisu_function.cpp:2540-2602. */
+void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+             const bool gen_gpu = false);
+void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+             const hardware_architecture_t gen_architecture_flag);
+
+/** GPU memory spaces of a buffer (reference: cuda_ast.h:180-188). */
+enum class memory_location { host, global, shared, local, constant, reg };
+
+/** A code-generation back-end: turns the lowered loop program of a function into an
+  * artefact on disk.  Back-ends register themselves by architecture. */
+class backend {
+public:
+    virtual ~backend() {}
+    virtual void generate(function &f, lir::program &prog, const std::string &obj_filename) = 0;
+    static void register_backend(hardware_architecture_t arch, backend *b);
+    static backend *find(hardware_architecture_t arch);
+};
+
+class function {
+    friend class computation;
+    friend class buffer;
+    friend class constant;
+    friend class input;
+
+    std::string name;
+    isl_ctx *ctx = nullptr;
+    std::vector<computation *> body;          // in declaration order
+    std::vector<computation *> invariants;    // function-wide constants
+    std::map<std::string, buffer *> buffers_list;
+    std::vector<buffer *> function_arguments;
+    isl_set *context_set = nullptr;
+    isl_ast_node *ast = nullptr;
+    std::unique_ptr<lir::program> lowered;
+    std::vector<std::string> iterator_names;
+
+public:
+    // (computation name, level) tags
+    std::set<std::pair<std::string, int>> parallel_dimensions;
+    std::map<std::pair<std::string, int>, int> vector_dimensions;   // -> vector length
+    std::map<std::pair<std::string, int>, int> unroll_dimensions;   // -> factor (0 = full)
+    std::set<std::pair<std::string, int>> distributed_dimensions;
+    /** (computation name, (l0,l1,l2)) with -1 for unused levels, outermost first
+      * (reference: core.h:340-346). */
+    std::vector<std::pair<std::string, std::tuple<int, int, int>>> gpu_block_dimensions;
+    std::vector<std::pair<std::string, std::tuple<int, int, int>>> gpu_thread_dimensions;
+
+    /** Ordering graph: sched_graph[a][b] = level means "b right after a, fused down to level". */
+    std::unordered_map<computation *, std::unordered_map<computation *, int>> sched_graph;
+    std::unordered_map<computation *, std::unordered_map<computation *, int>> sched_graph_reversed;
+    std::set<computation *> starting_computations;
+    bool use_low_level_scheduling_commands = false;
+
+    explicit function(std::string name);
+    ~function();
+
+    const std::string &get_name() const { return name; }
+    isl_ctx *get_isl_ctx() const { return ctx; }
+    const std::vector<computation *> &get_computations() const { return body; }
+    std::vector<computation *> get_computation_by_name(std::string nm) const;
+    const std::vector<computation *> &get_invariants() const { return invariants; }
+    std::vector<std::string> get_invariant_names() const;
+    const std::map<std::string, buffer *> &get_buffers() const { return buffers_list; }
+    const std::vector<buffer *> &get_arguments() const { return function_arguments; }
+    void add_computation(computation *c);
+    void add_invariant(constant *c);
+    void add_buffer(std::pair<std::string, buffer *> b);
+    void add_context_constraints(std::string constraints);
+    void set_context_set(const std::string &s) { add_context_constraints(s); }
+    isl_set *get_program_context() const { return context_set; }
+    void set_iterator_names(const std::vector<std::string> &names) { iterator_names = names; }
+    const std::vector<std::string> &get_iterator_names() const { return iterator_names; }
+
+    void add_parallel_dimension(std::string comp, int level);
+    void add_vector_dimension(std::string comp, int level, int length);
+    void add_unroll_dimension(std::string comp, int level, int factor);
+    void add_gpu_block_dimensions(std::string comp, int l0, int l1 = -1, int l2 = -1);
+    void add_gpu_thread_dimensions(std::string comp, int l0, int l1 = -1, int l2 = -1);
+    bool should_parallelize(const std::string &comp, int level) const;
+    int vector_length(const std::string &comp, int level) const;     // 0 if untagged
+    bool should_unroll(const std::string &comp, int level) const;
+    /** 0..2 = block z..x / thread index position in its tuple, -1 if the level is not mapped. */
+    int gpu_block_position(const std::string &comp, int level) const;
+    int gpu_thread_position(const std::string &comp, int level) const;
+
+    // ---- the code generation pipeline (reference: tiramisu_function.cpp:2540-2562) ----
+    void set_arguments(const std::vector<buffer *> &buffer_vec);
+    /** Turn the ordering graph into static schedule dimensions (reference :2231-2295). */
+    void gen_ordering_schedules();
+    /** Pad all schedules to the same number of dimensions (reference :1774-1794). */
+    void align_schedules();
+    void gen_time_space_domain();
+    /** Build the isl AST and lower it to the loop program shared by all back-ends. */
+    void gen_isl_ast();
+    isl_ast_node *get_isl_ast() const { return ast; }
+    lir::program &get_lowered_program();
+    /** Stages of the reference pipeline that existing programs call by hand; in this build
+      * gen_cuda_stmt selects the GPU back-end and gen_halide_obj runs it. */
+    void gen_cuda_stmt() { hand_driven_gpu = true; }
+    void gen_halide_stmt() {}
+    void gen_halide_obj(const std::string &obj_file_name);
+    void gen_c_code() const;
+    void dump_halide_stmt() const {}
+    void dump(bool exhaustive = false) const;
+    void dump_schedule() const;
+    void dump_sched_graph();
+    void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+                 const hardware_architecture_t arch);
+    void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+                 const bool gen_gpu = false);
+    int get_max_schedules_range_dim() const;
+    std::string generate_new_name(const std::string &prefix);
+    const std::vector<std::string> &get_codegen_log() const { return codegen_log; }
+    void log(const std::string &s) { codegen_log.push_back(s); }
+
+private:
+    bool hand_driven_gpu = false;
+    int name_counter = 0;
+    std::vector<std::string> codegen_log;
+};
+
+class buffer {
+    friend class computation;
+    friend class function;
+    std::string name;
+    std::vector<expr> dim_sizes;  // outermost first; last dimension is contiguous
+    primitive_t type;
+    argument_t argtype;
+    function *fct;
+    bool allocated = false;
+    bool auto_allocate = true;
+    bool auto_deallocate = true;
+
+public:
+    memory_location location = memory_location::host;
+
+    /** Reference: tiramisu_core.cpp:6762-6781. */
+    buffer(std::string name, std::vector<expr> dim_sizes, primitive_t type, argument_t argt,
+           function *fct = global::get_implicit_function(), std::string corr = "");
+
+    const std::string &get_name() const { return name; }
+    int get_n_dims() const { return (int)dim_sizes.size(); }
+    primitive_t get_elements_type() const { return type; }
+    const std::vector<expr> &get_dim_sizes() const { return dim_sizes; }
+    argument_t get_argument_type() const { return argtype; }
+    void set_argument_type(argument_t t) { argtype = t; }
+    memory_location get_location() const { return location; }
+    bool get_auto_allocate() const { return auto_allocate; }
+    bool get_auto_deallocate() const { return auto_deallocate; }
+    void set_auto_allocate(bool v) { auto_allocate = v; }
+    void set_auto_deallocate(bool v) { auto_deallocate = v; }
+    bool has_constant_extents() const;
+    function *get_function() const { return fct; }
+
+    /** Memory-space tags (reference: tiramisu_core.cpp:8913-8936). */
+    void tag_gpu_global() { location = memory_location::global; }
+    void tag_gpu_shared() { location = memory_location::shared; auto_allocate = false; }
+    void tag_gpu_local() { location = memory_location::local; auto_allocate = false; }
+    void tag_gpu_register();
+    void tag_gpu_constant() { location = memory_location::constant; }
+
+    /** Allocate (resp. free) this buffer right before (after) \p C at loop level \p level
+      * (reference: tiramisu_core.cpp:1479-1631). */
+    computation *allocate_at(computation &C, var level);
+    computation *allocate_at(computation &C, int level);
+    computation *deallocate_at(computation &C, var level);
+    computation *deallocate_at(computation &C, int level);
+    void dump(bool exhaustive) const;
+};
+
+class computation {
+    friend class function;
+    friend class buffer;
+    friend class input;
+    friend class constant;
+    friend class block;
+
+protected:
+    std::string name;
+    function *fct = nullptr;
+    isl_ctx *ctx = nullptr;
+    isl_set *iteration_domain = nullptr;
+    isl_map *schedule = nullptr;          // domain -> [dup, s0, d0, s1, ..., d(n-1), sn]
+    isl_map *access = nullptr;            // domain -> buffer
+    isl_set *time_space_domain = nullptr;
+    std::vector<std::string> level_names; // names of the dynamic dimensions, outermost first
+    std::vector<std::string> iterator_names_;  // names of the iteration-domain dimensions
+    expr expression;
+    expr predicate;
+    primitive_t data_type = p_none;
+    bool schedule_this = true;
+    bool is_let = false;
+    bool inline_ = false;
+    buffer *automatically_allocated_buffer = nullptr;
+    std::vector<std::pair<std::string, expr>> associated_let_stmts;
+    std::vector<var> declared_vars;
+
+    computation() {}
+    void init_computation(std::string iteration_space_str, function *f, const expr &e,
+                          bool schedule_this_computation, primitive_t t);
+    std::string construct_iteration_domain(const std::string &nm, const std::vector<var> &vars);
+    void set_identity_schedule();
+    int dynamic_pos(int level) const { return 2 * level + 2; }
+    int static_pos(int level_plus_one) const { return 2 * level_plus_one + 1; }
+    void apply_on_range(const std::string &transformation);
+    void assert_names_not_assigned(const std::vector<std::string> &names) const;
+    void separate_and_split(int level, int factor, const std::string &outer,
+                            const std::string &inner, bool &split_applied);
+
+public:
+    static const var root;
+    static constexpr int root_dimension = -1;
+
+    /** Low-level constructor from an isl set string such as
+      * "[N]->{S[i,j]: 0<=i<N and 0<=j<N}" (reference: core.h:3148-3152). */
+    computation(std::string iteration_domain, expr e, bool schedule_this_computation,
+                primitive_t t, function *fct);
+    computation(std::string name, std::vector<var> iterator_variables, expr e,
+                bool schedule_this_computation);
+    computation(std::vector<var> iterator_variables, expr e);
+    computation(std::string name, std::vector<var> iterator_variables, expr e);
+    computation(std::vector<var> iterator_variables, expr predicate, expr e);
+    computation(std::string name, std::vector<var> iterator_variables, expr predicate, expr e);
+    computation(std::vector<var> iterator_variables, expr e, bool schedule_this_computation);
+    computation(std::string name, std::vector<var> iterator_variables, primitive_t t)
+        : computation(name, iterator_variables, expr(t)) {}
+    computation(std::vector<var> iterator_variables, primitive_t t)
+        : computation(iterator_variables, expr(t)) {}
+    virtual ~computation();
+
+    // ---- queries ----
+    const std::string &get_name() const { return name; }
+    function *get_function() const { return fct; }
+    isl_ctx *get_ctx() const { return ctx; }
+    isl_set *get_iteration_domain() const { return iteration_domain; }
+    isl_map *get_schedule() const { return schedule; }
+    isl_map *get_access_relation() const { return access; }
+    isl_set *get_time_space_domain() const { return time_space_domain; }
+    const expr &get_expr() const { return expression; }
+    const expr &get_predicate() const { return predicate; }
+    primitive_t get_data_type() const { return data_type; }
+    int get_iteration_domain_dimensions_number() const;
+    int get_loop_levels_number() const { return (int)level_names.size(); }
+    const std::vector<std::string> &get_loop_level_names() const { return level_names; }
+    const std::vector<std::string> &get_iteration_domain_dimension_names() const { return iterator_names_; }
+    bool should_schedule_this_computation() const { return schedule_this; }
+    bool is_let_stmt() const { return is_let; }
+    bool is_inline_computation() const { return inline_; }
+    bool has_accesses() const;
+    buffer *get_buffer() const;
+    buffer *get_automatically_allocated_buffer() const { return automatically_allocated_buffer; }
+    buffer *auto_buffer() const { return automatically_allocated_buffer; }
+    const std::vector<std::pair<std::string, expr>> &get_associated_let_stmts() const { return associated_let_stmts; }
+    int get_loop_level_number_from_dimension_name(std::string dim_name) const {
+        return get_loop_level_numbers_from_dimension_names({dim_name})[0];
+    }
+    /** Look dimension names up in the schedule range; "root" gives -1
+      * (reference: tiramisu_core.cpp:2725-2770). */
+    std::vector<int> get_loop_level_numbers_from_dimension_names(const std::vector<std::string> &names) const;
+    void dump_iteration_domain() const;
+    void dump_schedule() const;
+    void dump() const;
+
+    // ---- definition ----
+    void set_expression(const expr &e);
+    void add_predicate(expr p) { predicate = p; }
+    void add_associated_let_stmt(std::string nm, expr e) { associated_let_stmts.push_back({nm, e}); }
+    void set_inline(bool is_inline = true) { inline_ = is_inline; }
+    void set_access(std::string access_str);
+    void set_access(isl_map *acc);
+    void store_in(buffer *buff);
+    void store_in(buffer *buff, std::vector<expr> iterators);
+    void store_in(std::vector<expr> mapping, std::vector<expr> sizes);
+    void allocate_and_map_buffer_automatically(argument_t type = a_temporary);
+    void unschedule_this_computation() { schedule_this = false; }
+
+    template <typename... Args> expr operator()(Args... args) {
+        std::vector<expr> idx{expr(args)...};
+        return make_access(idx);
+    }
+    expr make_access(const std::vector<expr> &idx);
+    operator expr();
+
+    // ---- ordering (reference: tiramisu_core.cpp:2352-2496) ----
+    void after(computation &comp, var iterator);
+    void after(computation &comp, int level);
+    void after_low_level(computation &comp, int level);
+    void before(computation &consumer, var L);
+    void before(computation &consumer, int L);
+    void between(computation &before_comp, var before_l, computation &after_comp, var after_l);
+    void between(computation &before_comp, int before_l, computation &after_comp, int after_l);
+    computation &then(computation &next_computation, var L = computation::root);
+    computation &then(computation &next_computation, int L);
+    void fuse_after(var lev, computation &comp) { after(comp, lev); }
+    computation *get_predecessor();
+
+    // ---- loop transformations ----
+    virtual void split(var L0, int sizeX);
+    virtual void split(var L0, int sizeX, var L0_outer, var L0_inner);
+    virtual void split(int L0, int sizeX);
+    virtual void tile(var L0, var L1, int sizeX, int sizeY);
+    virtual void tile(var L0, var L1, int sizeX, int sizeY, var L0_outer, var L1_outer,
+                      var L0_inner, var L1_inner);
+    virtual void tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ);
+    virtual void tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ, var L0_outer,
+                      var L1_outer, var L2_outer, var L0_inner, var L1_inner, var L2_inner);
+    virtual void tile(int L0, int L1, int sizeX, int sizeY);
+    virtual void tile(int L0, int L1, int L2, int sizeX, int sizeY, int sizeZ);
+    virtual void interchange(var L0, var L1);
+    virtual void interchange(int L0, int L1);
+    virtual void shift(var L0, int n);
+    virtual void shift(int L0, int n);
+    virtual void skew(var i, var j, int factor, var ni, var nj);
+    virtual void skew(var i, var j, int factor);
+    virtual void skew(int i, int j, int factor);
+    virtual void loop_reversal(var old_var, var new_var);
+    virtual void loop_reversal(int i);
+    virtual void parallelize(var L);
+    virtual void vectorize(var L, int v);
+    virtual void vectorize(var L, int v, var L_outer, var L_inner);
+    virtual void unroll(var L, int fac);
+    virtual void unroll(var L, int fac, var L_outer, var L_inner);
+    void tag_parallel_level(var L);
+    void tag_parallel_level(int L);
+    void tag_vector_level(var L, int len);
+    void tag_vector_level(int L, int len);
+    void tag_unroll_level(var L);
+    void tag_unroll_level(var L, int F);
+    void tag_unroll_level(int L);
+    void tag_unroll_level(int L, int F);
+    void set_low_level_schedule(std::string map_str);
+    void apply_transformation_on_schedule(std::string map_str);
+    void set_loop_level_names(std::vector<std::string> names);
+    void set_loop_level_names(std::vector<int> loop_levels, std::vector<std::string> names);
+    void add_schedule_constraint(std::string domain_constraints, std::string range_constraints);
+    int compute_maximal_AST_depth();
+
+    // ---- GPU mapping (reference: tiramisu_core.cpp:358-566, :2498-2580) ----
+    virtual void gpu_tile(var L0, var L1, int sizeX, int sizeY);
+    virtual void gpu_tile(var L0, var L1, int sizeX, int sizeY, var L0_outer, var L1_outer,
+                          var L0_inner, var L1_inner);
+    virtual void gpu_tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ);
+    virtual void gpu_tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ, var L0_outer,
+                          var L1_outer, var L2_outer, var L0_inner, var L1_inner, var L2_inner);
+    void tag_gpu_level(var L0, var L1);
+    void tag_gpu_level(var L0, var L1, var L2, var L3);
+    void tag_gpu_level(var L0, var L1, var L2, var L3, var L4, var L5);
+    void tag_gpu_level(int L0, int L1);
+    void tag_gpu_level(int L0, int L1, int L2, int L3);
+    void tag_gpu_level(int L0, int L1, int L2, int L3, int L4, int L5);
+    void tag_gpu_block_level(int L0);
+    void tag_gpu_block_level(int L0, int L1);
+    void tag_gpu_block_level(int L0, int L1, int L2);
+    void tag_gpu_thread_level(int L0);
+    void tag_gpu_thread_level(int L0, int L1);
+    void tag_gpu_thread_level(int L0, int L1, int L2);
+    /** Stage the part of \p inp that one thread block reads in LDS: a cooperative copy
+      * at loop level \p level of a tile of \p buffer_shape elements starting at
+      * \p copy_offsets, bracketed by barriers (reference: tiramisu_core.cpp:9297-9534). */
+    computation *cache_shared(computation &inp, const var &level, const std::vector<int> buffer_shape,
+                              const std::vector<expr> copy_offsets, bool pad_buffer = false);
+    std::vector<int> thread_block_shape;
+
+    void gen_time_space_domain();
+};
+
+class input : public computation {
+public:
+    input(std::string name, std::vector<var> iterator_variables, primitive_t t);
+    input(std::vector<var> iterator_variables, primitive_t t);
+    input(std::string name, std::vector<std::string> dimension_names,
+          std::vector<expr> dimension_sizes, primitive_t t);
+};
+
+class Input : public input {
+public:
+    Input(std::string name, std::vector<expr> sizes, primitive_t t);
+    std::vector<var> iterators_from_size_expressions(std::vector<expr> sizes);
+};
+
+class constant : public computation {
+public:
+    /** Function-wide constant (an invariant): becomes a parameter of every iteration domain
+      * declared afterwards and a const scalar at function entry
+      * (reference: tiramisu_core.cpp:8178-8283). */
+    constant(std::string param_name, const expr &param_expr);
+    constant(std::string param_name, const expr &param_expr, primitive_t t, function *func);
+    constant(std::string param_name, const expr &param_expr, primitive_t t, bool function_wide,
+             computation *with_computation, int at_loop_level, function *func);
+    operator expr();
+};
+
+}  // namespace tiramisu
+#endif

@@ -1,0 +1,1094 @@
+// function / buffer / computation: declaration of iteration domains, the schedule algebra
+// and the GPU mapping commands.  Schedules are isl maps from the iteration domain to a
+// time-space vector [dup, s0, d0, s1, d1, ..., d(n-1), sn] (static ordering dimensions s_k
+// interleaved with dynamic loop dimensions d_k), as in the reference
+// (src/tiramisu_core.cpp:2041-2081, :7640-7662); every command is a rewrite of the range.
+#include <tiramisu/block.h>
+#include <tiramisu/core.h>
+
+#include <algorithm>
+#include <cassert>
+#include <queue>
+#include <sstream>
+
+#include "isl_api.h"
+#include "lir.h"
+#include "util.h"
+
+namespace tiramisu {
+
+const var computation::root = var("root");
+
+// ------------------------------------------------------------------ helpers
+
+std::string expr_to_isl_str(const expr &e, bool &ok) {
+    if (!e.is_defined()) { ok = false; return ""; }
+    switch (e.get_expr_type()) {
+    case e_val:
+        if (is_float_type(e.get_data_type())) { ok = false; return ""; }
+        return std::to_string(e.get_int_val());
+    case e_var: return e.get_name();
+    case e_op: {
+        auto sub = [&](int i) { return expr_to_isl_str(e.get_operand(i), ok); };
+        switch (e.get_op_type()) {
+        case o_add: return "(" + sub(0) + " + " + sub(1) + ")";
+        case o_sub: return "(" + sub(0) + " - " + sub(1) + ")";
+        case o_minus: return "(-" + sub(0) + ")";
+        case o_mul:
+            if (!e.get_operand(0).is_integer_literal() && !e.get_operand(1).is_integer_literal()) ok = false;
+            return "(" + sub(0) + " * " + sub(1) + ")";
+        case o_div:
+            if (!e.get_operand(1).is_integer_literal()) ok = false;
+            return "floor(" + sub(0) + " / " + sub(1) + ")";
+        case o_mod:
+            if (!e.get_operand(1).is_integer_literal()) ok = false;
+            return "(" + sub(0) + " mod " + sub(1) + ")";
+        case o_max: return "max(" + sub(0) + ", " + sub(1) + ")";
+        case o_min: return "min(" + sub(0) + ", " + sub(1) + ")";
+        case o_cast:
+            if (is_float_type(e.get_data_type())) ok = false;
+            return sub(0);
+        default: ok = false; return "";
+        }
+    }
+    default: ok = false; return "";
+    }
+}
+
+static std::string params_prefix(const std::vector<std::string> &params) {
+    if (params.empty()) return "";
+    return "[" + join(params, ", ") + "] -> ";
+}
+
+// ------------------------------------------------------------------ init / codegen
+
+void init(std::string name) {
+    function *f = new function(name);
+    global::set_implicit_function(f);
+}
+
+void init() { init("foo"); }
+
+void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename, const bool gen_gpu) {
+    global::get_implicit_function()->codegen(arguments, obj_filename, gen_gpu);
+}
+
+void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+             const hardware_architecture_t arch) {
+    global::get_implicit_function()->codegen(arguments, obj_filename, arch);
+}
+
+static std::map<hardware_architecture_t, backend *> &backend_table() {
+    static std::map<hardware_architecture_t, backend *> t;
+    return t;
+}
+void backend::register_backend(hardware_architecture_t arch, backend *b) { backend_table()[arch] = b; }
+backend *backend::find(hardware_architecture_t arch) {
+    auto it = backend_table().find(arch);
+    return it == backend_table().end() ? nullptr : it->second;
+}
+
+// ------------------------------------------------------------------ function
+
+function::function(std::string nm) : name(nm) {
+    ctx = isl_ctx_alloc();
+    if (nm.empty()) ERROR("a function needs a name", true);
+}
+
+function::~function() {}
+
+std::vector<computation *> function::get_computation_by_name(std::string nm) const {
+    std::vector<computation *> r;
+    for (auto c : body)
+        if (c->get_name() == nm) r.push_back(c);
+    return r;
+}
+
+std::vector<std::string> function::get_invariant_names() const {
+    std::vector<std::string> r;
+    for (auto c : invariants) r.push_back(c->get_name());
+    return r;
+}
+
+void function::add_computation(computation *c) {
+    body.push_back(c);
+    if (c->should_schedule_this_computation()) starting_computations.insert(c);
+}
+
+void function::add_invariant(constant *c) { invariants.push_back(c); }
+
+void function::add_buffer(std::pair<std::string, buffer *> b) {
+    if (buffers_list.count(b.first)) ERROR("buffer " + b.first + " declared twice", true);
+    buffers_list[b.first] = b.second;
+}
+
+void function::add_context_constraints(std::string s) {
+    isl_set *c = isl_set_read_from_str(ctx, s.c_str());
+    if (!c) ERROR("cannot parse context " + s, true);
+    context_set = context_set ? isl_set_intersect(context_set, c) : c;
+}
+
+std::string function::generate_new_name(const std::string &prefix) {
+    return prefix + std::to_string(name_counter++);
+}
+
+void function::add_parallel_dimension(std::string comp, int level) { parallel_dimensions.insert({comp, level}); }
+void function::add_vector_dimension(std::string comp, int level, int length) { vector_dimensions[{comp, level}] = length; }
+void function::add_unroll_dimension(std::string comp, int level, int factor) { unroll_dimensions[{comp, level}] = factor; }
+
+void function::add_gpu_block_dimensions(std::string comp, int l0, int l1, int l2) {
+    for (auto &p : gpu_block_dimensions)
+        if (p.first == comp) { p.second = std::make_tuple(l0, l1, l2); return; }
+    gpu_block_dimensions.push_back({comp, std::make_tuple(l0, l1, l2)});
+}
+void function::add_gpu_thread_dimensions(std::string comp, int l0, int l1, int l2) {
+    for (auto &p : gpu_thread_dimensions)
+        if (p.first == comp) { p.second = std::make_tuple(l0, l1, l2); return; }
+    gpu_thread_dimensions.push_back({comp, std::make_tuple(l0, l1, l2)});
+}
+
+bool function::should_parallelize(const std::string &comp, int level) const {
+    return parallel_dimensions.count({comp, level}) > 0;
+}
+int function::vector_length(const std::string &comp, int level) const {
+    auto it = vector_dimensions.find({comp, level});
+    return it == vector_dimensions.end() ? 0 : it->second;
+}
+bool function::should_unroll(const std::string &comp, int level) const {
+    return unroll_dimensions.count({comp, level}) > 0;
+}
+
+// x/y/z are given to the tagged levels from the innermost outwards, so that the
+// fastest-varying tagged loop becomes the x index (reference: tiramisu_codegen_cuda.cpp:560-617).
+static int position_in(const std::tuple<int, int, int> &t, int level) {
+    int lv[3] = {std::get<2>(t), std::get<1>(t), std::get<0>(t)};
+    int pos = 0;
+    for (int i = 0; i < 3; i++) {
+        if (lv[i] == -1) continue;
+        if (lv[i] == level) return pos;
+        pos++;
+    }
+    return -1;
+}
+int function::gpu_block_position(const std::string &comp, int level) const {
+    for (auto &p : gpu_block_dimensions)
+        if (p.first == comp) return position_in(p.second, level);
+    return -1;
+}
+int function::gpu_thread_position(const std::string &comp, int level) const {
+    for (auto &p : gpu_thread_dimensions)
+        if (p.first == comp) return position_in(p.second, level);
+    return -1;
+}
+
+void function::set_arguments(const std::vector<buffer *> &buffer_vec) {
+    function_arguments = buffer_vec;
+    for (auto b : buffer_vec) {
+        if (!b) ERROR("null buffer passed as a function argument", true);
+        if (b->location != memory_location::host && b->location != memory_location::global)
+            ERROR("argument buffer " + b->get_name() + " must live in host or GPU global memory", true);
+    }
+}
+
+int function::get_max_schedules_range_dim() const {
+    int m = 0;
+    for (auto c : body)
+        if (c->schedule) m = std::max(m, (int)isl_map_dim(c->schedule, isl_dim_out));
+    return m;
+}
+
+void function::align_schedules() {
+    int m = get_max_schedules_range_dim();
+    for (auto c : body) {
+        if (!c->schedule) continue;
+        int r = isl_map_dim(c->schedule, isl_dim_out);
+        if (r == m) continue;
+        std::vector<std::string> in, out;
+        for (int i = 0; i < r; i++) { in.push_back("x" + std::to_string(i)); out.push_back(in.back()); }
+        for (int i = r; i < m; i++) out.push_back("0");
+        c->apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+    }
+}
+
+void function::gen_ordering_schedules() {
+    if (use_low_level_scheduling_commands) return;
+    // Scheduled computations without a predecessor, in declaration order.
+    std::vector<computation *> roots;
+    for (auto c : body)
+        if (c->should_schedule_this_computation() && starting_computations.count(c)) roots.push_back(c);
+    computation *last = nullptr;
+    for (auto start : roots) {
+        if (last) start->after_low_level(*last, computation::root_dimension);
+        // Walk the tree, always descending into the deepest pending fuse level first
+        // (reference: tiramisu_function.cpp:2249-2287).
+        std::priority_queue<int> level_to_check;
+        std::map<int, std::deque<computation *>> level_queue;
+        computation *current = start;
+        while (true) {
+            // deterministic order: successors sorted by declaration order
+            std::vector<std::pair<computation *, int>> edges(sched_graph[current].begin(), sched_graph[current].end());
+            std::sort(edges.begin(), edges.end(), [&](auto &a, auto &b) {
+                return std::find(body.begin(), body.end(), a.first) < std::find(body.begin(), body.end(), b.first);
+            });
+            for (auto &e : edges) {
+                if (level_queue[e.second].empty()) level_to_check.push(e.second);
+                level_queue[e.second].push_back(e.first);
+            }
+            if (level_to_check.empty()) break;
+            int fuse_level = level_to_check.top();
+            computation *next = level_queue[fuse_level].front();
+            level_queue[fuse_level].pop_front();
+            next->after_low_level(*current, fuse_level);
+            current = next;
+            if (level_queue[fuse_level].empty()) level_to_check.pop();
+        }
+        last = current;
+    }
+}
+
+void function::gen_time_space_domain() {
+    gen_ordering_schedules();
+    align_schedules();
+    for (auto c : body) c->gen_time_space_domain();
+}
+
+void function::dump_sched_graph() {
+    for (auto &a : sched_graph)
+        for (auto &b : a.second)
+            std::cout << a.first->get_name() << " => " << b.first->get_name() << " [" << b.second << "]\n";
+}
+
+void function::dump_schedule() const {
+    for (auto c : body) c->dump_schedule();
+}
+
+void function::dump(bool) const {
+    std::cout << "function " << name << "\n";
+    for (auto c : body) c->dump();
+}
+
+void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename, const bool gen_gpu) {
+    codegen(arguments, obj_filename,
+            gen_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu);
+}
+
+void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+                       hardware_architecture_t arch) {
+    if (arch == hardware_architecture_t::arch_nvidia_gpu) arch = hardware_architecture_t::arch_amd_gpu;
+    backend *b = backend::find(arch);
+    if (!b) {
+        if (arch == hardware_architecture_t::arch_cpu)
+            ERROR("no CPU back-end is linked into this program: the GPU library generates HIP only; "
+                  "link the oracle's CPU emitter to generate host code", true);
+        ERROR("no back-end registered for the requested architecture", true);
+    }
+    set_arguments(arguments);
+    gen_time_space_domain();
+    gen_isl_ast();
+    b->generate(*this, get_lowered_program(), obj_filename);
+}
+
+void function::gen_halide_obj(const std::string &obj_file_name) {
+    hardware_architecture_t arch =
+        hand_driven_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu;
+    backend *b = backend::find(arch);
+    if (!b) ERROR("no back-end registered for the requested architecture", true);
+    if (!ast) gen_isl_ast();
+    b->generate(*this, get_lowered_program(), obj_file_name);
+}
+
+lir::program &function::get_lowered_program() {
+    if (!lowered) ERROR("gen_isl_ast() has not been run", true);
+    return *lowered;
+}
+
+// ------------------------------------------------------------------ buffer
+
+buffer::buffer(std::string nm, std::vector<expr> sizes, primitive_t t, argument_t argt, function *f,
+               std::string)
+    : name(nm), dim_sizes(std::move(sizes)), type(t), argtype(argt), fct(f) {
+    if (!fct) ERROR("declare a function (tiramisu::init) before declaring buffers", true);
+    if (name.empty()) ERROR("a buffer needs a name", true);
+    for (auto &e : dim_sizes)
+        if (!e.is_defined()) ERROR("undefined size expression for buffer " + name, true);
+    fct->add_buffer({name, this});
+}
+
+bool buffer::has_constant_extents() const {
+    for (auto &e : dim_sizes)
+        if (!lir::simplify(e).is_integer_literal()) return false;
+    return true;
+}
+
+void buffer::tag_gpu_register() {
+    bool one = dim_sizes.size() == 1 && lir::simplify(dim_sizes[0]).is_integer_literal() &&
+               lir::simplify(dim_sizes[0]).get_int_val() == 1;
+    if (!one) ERROR("a register buffer must have the shape {1}: " + name, true);
+    location = memory_location::reg;
+    auto_allocate = false;
+}
+
+void buffer::dump(bool) const {
+    std::cout << "buffer " << name << " [";
+    for (size_t i = 0; i < dim_sizes.size(); i++) std::cout << (i ? ", " : "") << dim_sizes[i].to_str();
+    std::cout << "] " << str_from_tiramisu_type_primitive(type) << "\n";
+}
+
+// Allocation / release computations live on the first level+1 dimensions of C's iteration
+// domain; the program orders them itself with then()/after()
+// (reference: tiramisu_core.cpp:1479-1631).
+static computation *make_alloc_like(buffer *b, computation &C, int level, bool is_alloc, function *fct) {
+    isl_set *dom = isl_set_copy(C.get_iteration_domain());
+    int n = isl_set_dim(dom, isl_dim_set);
+    if (level + 1 > n) ERROR("allocate_at/deallocate_at: level out of range", true);
+    if (level + 1 == 0) {
+        isl_set_free(dom);
+        dom = isl_set_read_from_str(C.get_ctx(), "{ [0] }");
+    } else {
+        dom = isl_set_project_out(dom, isl_dim_set, level + 1, n - (level + 1));
+    }
+    std::string nm = std::string(is_alloc ? "_allocation_" : "_deallocation_") + C.get_name();
+    dom = isl_set_set_tuple_name(dom, nm.c_str());
+    char *s = isl_set_to_str(dom);
+    std::string dom_str(s);
+    free(s);
+    isl_set_free(dom);
+    expr e = is_alloc ? expr(o_allocate, b->get_name()) : expr(o_free, b->get_name());
+    computation *a = new computation(dom_str, e, true, p_none, fct);
+    std::vector<std::string> names(C.get_loop_level_names().begin(), C.get_loop_level_names().begin() + level + 1);
+    a->set_loop_level_names(names);
+    return a;
+}
+
+computation *buffer::allocate_at(computation &C, int level) {
+    set_auto_allocate(false);
+    return make_alloc_like(this, C, level, true, fct);
+}
+computation *buffer::allocate_at(computation &C, var level) {
+    return allocate_at(C, C.get_loop_level_number_from_dimension_name(level.get_name()));
+}
+computation *buffer::deallocate_at(computation &C, int level) {
+    set_auto_deallocate(false);
+    return make_alloc_like(this, C, level, false, fct);
+}
+computation *buffer::deallocate_at(computation &C, var level) {
+    return deallocate_at(C, C.get_loop_level_number_from_dimension_name(level.get_name()));
+}
+
+// ------------------------------------------------------------------ computation: construction
+
+computation::~computation() {}
+
+std::string computation::construct_iteration_domain(const std::string &nm, const std::vector<var> &vars) {
+    std::vector<std::string> params = fct->get_invariant_names();
+    std::ostringstream os;
+    os << params_prefix(params) << "{ " << nm << "[";
+    if (vars.empty()) {
+        os << "0] }";
+        return os.str();
+    }
+    for (size_t i = 0; i < vars.size(); i++) os << (i ? ", " : "") << vars[i].get_name();
+    os << "] : ";
+    for (size_t i = 0; i < vars.size(); i++) {
+        bool ok = true;
+        if (!vars[i].get_lower().is_defined() || !vars[i].get_upper().is_defined())
+            ERROR("iterator " + vars[i].get_name() + " of " + nm + " has no bounds", true);
+        std::string lo = expr_to_isl_str(vars[i].get_lower(), ok);
+        std::string up = expr_to_isl_str(vars[i].get_upper(), ok);
+        if (!ok) ERROR("bounds of iterator " + vars[i].get_name() + " are not affine", true);
+        os << (i ? " and " : "") << lo << " <= " << vars[i].get_name() << " < " << up;
+    }
+    os << " }";
+    return os.str();
+}
+
+void computation::init_computation(std::string iteration_space_str, function *f, const expr &e,
+                                   bool schedule_this_computation, primitive_t t) {
+    fct = f;
+    if (!fct) ERROR("declare a function (tiramisu::init) before declaring computations", true);
+    ctx = fct->get_isl_ctx();
+    iteration_domain = isl_set_read_from_str(ctx, iteration_space_str.c_str());
+    if (!iteration_domain) ERROR("cannot parse iteration domain: " + iteration_space_str, true);
+    const char *tn = isl_set_get_tuple_name(iteration_domain);
+    if (!tn) ERROR("iteration domain without a name: " + iteration_space_str, true);
+    name = tn;
+    int n = isl_set_dim(iteration_domain, isl_dim_set);
+    iterator_names_.clear();
+    for (int i = 0; i < n; i++) {
+        const char *dn = isl_set_get_dim_name(iteration_domain, isl_dim_set, i);
+        iterator_names_.push_back(dn ? dn : ("_i" + std::to_string(i)));
+    }
+    level_names = iterator_names_;
+    expression = e;
+    data_type = t;
+    schedule_this = schedule_this_computation;
+    set_identity_schedule();
+    fct->add_computation(this);
+}
+
+void computation::set_identity_schedule() {
+    int n = (int)iterator_names_.size();
+    std::vector<std::string> in, out{"0", "0"};
+    for (int i = 0; i < n; i++) {
+        in.push_back("t" + std::to_string(i));
+        out.push_back(in.back());
+        out.push_back("0");
+    }
+    std::string s = "{ " + name + "[" + join(in, ",") + "] -> [" + join(out, ",") + "] }";
+    schedule = isl_map_read_from_str(ctx, s.c_str());
+}
+
+computation::computation(std::string iteration_domain_str, expr e, bool schedule_this_computation,
+                         primitive_t t, function *f) {
+    init_computation(iteration_domain_str, f, e, schedule_this_computation, t);
+}
+
+computation::computation(std::string nm, std::vector<var> iterator_variables, expr e,
+                         bool schedule_this_computation) {
+    fct = global::get_implicit_function();
+    if (!fct) ERROR("call tiramisu::init() first", true);
+    declared_vars = iterator_variables;
+    init_computation(construct_iteration_domain(nm, iterator_variables), fct, e, schedule_this_computation,
+                     e.get_data_type());
+    if (iterator_variables.empty()) { iterator_names_ = {"_zero"}; level_names = iterator_names_; }
+    if (global::is_auto_data_mapping_set() && has_accesses()) allocate_and_map_buffer_automatically(a_temporary);
+}
+
+static std::string fresh_computation_name() {
+    static int n = 0;
+    return "_comp" + std::to_string(n++);
+}
+
+computation::computation(std::vector<var> iterator_variables, expr e)
+    : computation(fresh_computation_name(), iterator_variables, e, true) {}
+computation::computation(std::string nm, std::vector<var> iterator_variables, expr e)
+    : computation(nm, iterator_variables, e, true) {}
+computation::computation(std::vector<var> iterator_variables, expr p, expr e)
+    : computation(fresh_computation_name(), iterator_variables, e, true) { add_predicate(p); }
+computation::computation(std::string nm, std::vector<var> iterator_variables, expr p, expr e)
+    : computation(nm, iterator_variables, e, true) { add_predicate(p); }
+computation::computation(std::vector<var> iterator_variables, expr e, bool schedule_this_computation)
+    : computation(fresh_computation_name(), iterator_variables, e, schedule_this_computation) {}
+
+bool computation::has_accesses() const {
+    // Leaves that only act (barrier, copy, allocation, library call) store nothing
+    // (reference: tiramisu_core.cpp:7797-7813).
+    if (expression.get_expr_type() == e_sync) return false;
+    if (expression.get_expr_type() == e_op) {
+        op_t o = expression.get_op_type();
+        if (o == o_memcpy || o == o_allocate || o == o_free) return false;
+    }
+    if (is_let) return false;
+    return true;
+}
+
+int computation::get_iteration_domain_dimensions_number() const {
+    return isl_set_dim(iteration_domain, isl_dim_set);
+}
+
+void computation::allocate_and_map_buffer_automatically(argument_t type) {
+    std::vector<expr> sizes;
+    if (declared_vars.empty()) {
+        sizes.push_back(expr((int32_t)1));
+    } else {
+        for (auto &v : declared_vars) {
+            if (!v.get_upper().is_defined()) return;  // unbounded: the user maps it by hand
+            sizes.push_back(lir::simplify(v.get_upper() - v.get_lower()));
+        }
+    }
+    std::string bname = "_" + name + "_" + fct->generate_new_name("b");
+    automatically_allocated_buffer = new buffer(bname, sizes, data_type, type, fct);
+    store_in(automatically_allocated_buffer);
+}
+
+buffer *computation::get_buffer() const {
+    if (!access) return nullptr;
+    const char *bn = isl_map_get_tuple_name(access, isl_dim_out);
+    if (!bn) return nullptr;
+    auto it = fct->get_buffers().find(bn);
+    return it == fct->get_buffers().end() ? nullptr : it->second;
+}
+
+void computation::set_expression(const expr &e) {
+    expression = e;
+    if (data_type == p_none) data_type = e.get_data_type();
+}
+
+void computation::set_access(std::string access_str) {
+    isl_map *m = isl_map_read_from_str(ctx, access_str.c_str());
+    if (!m) ERROR("cannot parse access relation " + access_str, true);
+    set_access(m);
+}
+
+void computation::set_access(isl_map *acc) {
+    if (access) isl_map_free(access);
+    access = acc;
+}
+
+void computation::store_in(buffer *buff) {
+    std::vector<expr> idx;
+    int n = (int)iterator_names_.size();
+    // A buffer with fewer dimensions than the domain takes the innermost iterators.
+    int nb = buff->get_n_dims();
+    for (int i = std::max(0, n - nb); i < n; i++) idx.push_back(var(iterator_names_[i]));
+    if (declared_vars.empty() && n == 1) idx = {expr((int32_t)0)};
+    store_in(buff, idx);
+}
+
+void computation::store_in(buffer *buff, std::vector<expr> iterators) {
+    std::vector<std::string> out;
+    for (auto &e : iterators) {
+        bool ok = true;
+        out.push_back(expr_to_isl_str(e, ok));
+        if (!ok) ERROR("store_in of " + name + ": index " + e.to_str() + " is not affine", true);
+    }
+    std::vector<std::string> in = iterator_names_;
+    if (declared_vars.empty() && in.size() == 1) in = {"_zero"};
+    std::string s = params_prefix(fct->get_invariant_names()) + "{ " + name + "[" + join(in, ", ") + "] -> " +
+                    buff->get_name() + "[" + join(out, ", ") + "] }";
+    set_access(s);
+}
+
+void computation::store_in(std::vector<expr> mapping, std::vector<expr> sizes) {
+    std::string bname = "_" + name + "_" + fct->generate_new_name("b");
+    buffer *b = new buffer(bname, sizes, data_type, a_temporary, fct);
+    automatically_allocated_buffer = b;
+    store_in(b, mapping);
+}
+
+expr computation::make_access(const std::vector<expr> &idx) {
+    if ((int)idx.size() != (int)iterator_names_.size() && !(declared_vars.empty() && idx.empty())) {
+        std::string s = "Error - Incorrect access: " + name + "(";
+        for (size_t i = 0; i < idx.size(); i++) s += (i ? ", " : "") + idx[i].to_str();
+        ERROR(s + "). The number of access dimensions does not match the declaration of " + name, true);
+    }
+    if (inline_) {
+        std::map<std::string, expr> subs;
+        for (size_t i = 0; i < idx.size(); i++) subs[iterator_names_[i]] = idx[i];
+        return expression.substitute(subs);
+    }
+    return expr(o_access, name, idx, data_type);
+}
+
+computation::operator expr() {
+    std::vector<expr> idx;
+    for (auto &n : iterator_names_) idx.push_back(var(n));
+    return make_access(idx);
+}
+
+void computation::dump_iteration_domain() const {
+    char *s = isl_set_to_str(iteration_domain);
+    std::cout << s << std::endl;
+    free(s);
+}
+void computation::dump_schedule() const {
+    char *s = isl_map_to_str(schedule);
+    std::cout << name << ": " << s << "   levels: " << join(level_names, ",") << std::endl;
+    free(s);
+}
+void computation::dump() const {
+    dump_iteration_domain();
+    dump_schedule();
+    std::cout << "  expr: " << expression.to_str() << std::endl;
+    if (access) {
+        char *s = isl_map_to_str(access);
+        std::cout << "  access: " << s << std::endl;
+        free(s);
+    }
+}
+
+// ------------------------------------------------------------------ computation: names and levels
+
+std::vector<int> computation::get_loop_level_numbers_from_dimension_names(const std::vector<std::string> &names) const {
+    std::vector<int> r;
+    for (auto &n : names) {
+        if (n == "root") { r.push_back(root_dimension); continue; }
+        auto it = std::find(level_names.begin(), level_names.end(), n);
+        if (it == level_names.end())
+            ERROR("dimension " + n + " not found in the schedule of " + name + " (levels: " + join(level_names, ",") + ")", true);
+        r.push_back((int)(it - level_names.begin()));
+    }
+    return r;
+}
+
+void computation::set_loop_level_names(std::vector<std::string> names) {
+    for (size_t i = 0; i < names.size() && i < level_names.size(); i++) level_names[i] = names[i];
+}
+void computation::set_loop_level_names(std::vector<int> loop_levels, std::vector<std::string> names) {
+    for (size_t i = 0; i < loop_levels.size(); i++) level_names.at(loop_levels[i]) = names[i];
+}
+
+void computation::assert_names_not_assigned(const std::vector<std::string> &names) const {
+    for (auto &n : names)
+        if (std::find(level_names.begin(), level_names.end(), n) != level_names.end())
+            ERROR("dimension name " + n + " is already used in the schedule of " + name, true);
+}
+
+void computation::apply_on_range(const std::string &t) {
+    isl_map *m = isl_map_read_from_str(ctx, t.c_str());
+    if (!m) ERROR("cannot parse schedule transformation " + t, true);
+    schedule = isl_map_apply_range(schedule, m);
+}
+
+void computation::apply_transformation_on_schedule(std::string map_str) { apply_on_range(map_str); }
+
+void computation::set_low_level_schedule(std::string map_str) {
+    isl_map *m = isl_map_read_from_str(ctx, map_str.c_str());
+    if (!m) ERROR("cannot parse schedule " + map_str, true);
+    if (schedule) isl_map_free(schedule);
+    schedule = m;
+    fct->use_low_level_scheduling_commands = true;
+}
+
+void computation::add_schedule_constraint(std::string domain_constraints, std::string range_constraints) {
+    if (!domain_constraints.empty()) {
+        isl_set *d = isl_set_read_from_str(ctx, domain_constraints.c_str());
+        schedule = isl_map_intersect_domain(schedule, d);
+    }
+    if (!range_constraints.empty()) {
+        isl_set *r = isl_set_read_from_str(ctx, range_constraints.c_str());
+        schedule = isl_map_intersect_range(schedule, r);
+    }
+}
+
+// Range variable lists for a transformation of a schedule with n levels.
+static void range_vars(int n, std::vector<std::string> &v) {
+    v.clear();
+    for (int i = 0; i < 2 * n + 2; i++) v.push_back("x" + std::to_string(i));
+}
+
+// ------------------------------------------------------------------ loop transformations
+
+void computation::split(int L0, int sizeX) {
+    int n = (int)level_names.size();
+    if (L0 < 0 || L0 >= n) ERROR("split: level out of range for " + name, true);
+    if (sizeX < 1) ERROR("split: factor must be positive", true);
+    std::vector<std::string> in, out;
+    range_vars(n, in);
+    int p = dynamic_pos(L0);
+    for (int i = 0; i < (int)in.size(); i++) {
+        if (i == p) { out.push_back("o"); out.push_back("0"); out.push_back("r"); }
+        else out.push_back(in[i]);
+    }
+    std::string s = std::to_string(sizeX);
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] : o = floor(" + in[p] + "/" + s +
+                   ") and r = " + in[p] + " - " + s + "*o }");
+    std::string base = level_names[L0];
+    level_names[L0] = base + "_outer";
+    level_names.insert(level_names.begin() + L0 + 1, base + "_inner");
+}
+
+void computation::split(var L0, int sizeX, var L0_outer, var L0_inner) {
+    int l = get_loop_level_number_from_dimension_name(L0.get_name());
+    assert_names_not_assigned({L0_outer.get_name(), L0_inner.get_name()});
+    split(l, sizeX);
+    level_names[l] = L0_outer.get_name();
+    level_names[l + 1] = L0_inner.get_name();
+}
+
+void computation::split(var L0, int sizeX) {
+    split(L0, sizeX, var(fct->generate_new_name(L0.get_name() + "_o")), var(fct->generate_new_name(L0.get_name() + "_i")));
+}
+
+void computation::interchange(int L0, int L1) {
+    int n = (int)level_names.size();
+    if (L0 < 0 || L1 < 0 || L0 >= n || L1 >= n) ERROR("interchange: level out of range for " + name, true);
+    std::vector<std::string> in, out;
+    range_vars(n, in);
+    out = in;
+    std::swap(out[dynamic_pos(L0)], out[dynamic_pos(L1)]);
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+    std::swap(level_names[L0], level_names[L1]);
+}
+
+void computation::interchange(var L0, var L1) {
+    auto l = get_loop_level_numbers_from_dimension_names({L0.get_name(), L1.get_name()});
+    interchange(l[0], l[1]);
+}
+
+// tile = split both loops, then move the first inner loop below the second outer loop
+// (reference: tiramisu_core.cpp:2705-2723).
+void computation::tile(int L0, int L1, int sizeX, int sizeY) {
+    if (L1 != L0 + 1) ERROR("tile: the two levels must be consecutive", true);
+    split(L0, sizeX);
+    split(L1 + 1, sizeY);
+    interchange(L0 + 1, L1 + 1);
+}
+
+void computation::tile(var L0, var L1, int sizeX, int sizeY, var L0_outer, var L1_outer, var L0_inner,
+                       var L1_inner) {
+    auto l = get_loop_level_numbers_from_dimension_names({L0.get_name(), L1.get_name()});
+    assert_names_not_assigned({L0_outer.get_name(), L1_outer.get_name(), L0_inner.get_name(), L1_inner.get_name()});
+    tile(l[0], l[1], sizeX, sizeY);
+    level_names[l[0]] = L0_outer.get_name();
+    level_names[l[0] + 1] = L1_outer.get_name();
+    level_names[l[0] + 2] = L0_inner.get_name();
+    level_names[l[0] + 3] = L1_inner.get_name();
+}
+
+void computation::tile(var L0, var L1, int sizeX, int sizeY) {
+    tile(L0, L1, sizeX, sizeY, var(fct->generate_new_name(L0.get_name() + "_o")),
+         var(fct->generate_new_name(L1.get_name() + "_o")), var(fct->generate_new_name(L0.get_name() + "_i")),
+         var(fct->generate_new_name(L1.get_name() + "_i")));
+}
+
+// 3-D tile: order becomes L0o, L1o, L2o, L0i, L1i, L2i (reference: tiramisu_core.cpp:2971-3062).
+void computation::tile(int L0, int L1, int L2, int sizeX, int sizeY, int sizeZ) {
+    if (L1 != L0 + 1 || L2 != L1 + 1) ERROR("tile: the three levels must be consecutive", true);
+    split(L0, sizeX);       // L0o L0i L1 L2
+    split(L0 + 2, sizeY);   // L0o L0i L1o L1i L2
+    split(L0 + 4, sizeZ);   // L0o L0i L1o L1i L2o L2i
+    interchange(L0 + 1, L0 + 2);  // L0o L1o L0i L1i L2o L2i
+    interchange(L0 + 2, L0 + 4);  // L0o L1o L2o L1i L0i L2i
+    interchange(L0 + 3, L0 + 4);  // L0o L1o L2o L0i L1i L2i
+}
+
+void computation::tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ, var L0_outer, var L1_outer,
+                       var L2_outer, var L0_inner, var L1_inner, var L2_inner) {
+    auto l = get_loop_level_numbers_from_dimension_names({L0.get_name(), L1.get_name(), L2.get_name()});
+    tile(l[0], l[1], l[2], sizeX, sizeY, sizeZ);
+    std::string nm[6] = {L0_outer.get_name(), L1_outer.get_name(), L2_outer.get_name(),
+                         L0_inner.get_name(), L1_inner.get_name(), L2_inner.get_name()};
+    for (int i = 0; i < 6; i++) level_names[l[0] + i] = nm[i];
+}
+
+void computation::tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ) {
+    auto g = [&](const var &v, const char *s) { return var(fct->generate_new_name(v.get_name() + s)); };
+    tile(L0, L1, L2, sizeX, sizeY, sizeZ, g(L0, "_o"), g(L1, "_o"), g(L2, "_o"), g(L0, "_i"), g(L1, "_i"), g(L2, "_i"));
+}
+
+void computation::shift(int L0, int n) {
+    std::vector<std::string> in, out;
+    range_vars((int)level_names.size(), in);
+    out = in;
+    out[dynamic_pos(L0)] = in[dynamic_pos(L0)] + " + " + std::to_string(n);
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+}
+void computation::shift(var L0, int n) { shift(get_loop_level_number_from_dimension_name(L0.get_name()), n); }
+
+// skew(i, j, f): j' = f*i + j (reference: core.h "skew" documentation).
+void computation::skew(int i, int j, int factor) {
+    std::vector<std::string> in, out;
+    range_vars((int)level_names.size(), in);
+    out = in;
+    out[dynamic_pos(j)] = std::to_string(factor) + "*" + in[dynamic_pos(i)] + " + " + in[dynamic_pos(j)];
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+}
+void computation::skew(var i, var j, int factor) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name()});
+    skew(l[0], l[1], factor);
+}
+void computation::skew(var i, var j, int factor, var ni, var nj) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name()});
+    skew(l[0], l[1], factor);
+    level_names[l[0]] = ni.get_name();
+    level_names[l[1]] = nj.get_name();
+}
+
+void computation::loop_reversal(int i) {
+    std::vector<std::string> in, out;
+    range_vars((int)level_names.size(), in);
+    out = in;
+    out[dynamic_pos(i)] = "-" + in[dynamic_pos(i)];
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+}
+void computation::loop_reversal(var old_var, var new_var) {
+    int l = get_loop_level_number_from_dimension_name(old_var.get_name());
+    loop_reversal(l);
+    level_names[l] = new_var.get_name();
+}
+
+void computation::tag_parallel_level(int L) { fct->add_parallel_dimension(name, L); }
+void computation::tag_parallel_level(var L) { tag_parallel_level(get_loop_level_number_from_dimension_name(L.get_name())); }
+void computation::parallelize(var L) { tag_parallel_level(L); }
+void computation::tag_vector_level(int L, int len) { fct->add_vector_dimension(name, L, len); }
+void computation::tag_vector_level(var L, int len) { tag_vector_level(get_loop_level_number_from_dimension_name(L.get_name()), len); }
+void computation::tag_unroll_level(int L) { fct->add_unroll_dimension(name, L, 0); }
+void computation::tag_unroll_level(int L, int F) { fct->add_unroll_dimension(name, L, F); }
+void computation::tag_unroll_level(var L) { tag_unroll_level(get_loop_level_number_from_dimension_name(L.get_name())); }
+void computation::tag_unroll_level(var L, int F) { tag_unroll_level(get_loop_level_number_from_dimension_name(L.get_name()), F); }
+
+// vectorize/unroll: split by the factor and tag the inner loop.  The reference first
+// separates a remainder computation when the extent is not a multiple of the factor
+// (tiramisu_core.cpp:1238-1370); here the inner loop simply keeps a min() bound on the last
+// tile, which executes the same iterations in the same order.
+void computation::separate_and_split(int level, int factor, const std::string &outer, const std::string &inner,
+                                     bool &split_applied) {
+    isl_set *ts = isl_set_apply(isl_set_copy(iteration_domain), isl_map_copy(schedule));
+    int p = dynamic_pos(level);
+    isl_val *mx = isl_set_dim_max_val(isl_set_copy(ts), p);
+    isl_val *mn = isl_set_dim_min_val(ts, p);
+    long extent = -1;
+    if (mx && mn && isl_val_is_int(mx) == isl_bool_true && isl_val_is_int(mn) == isl_bool_true)
+        extent = isl_val_get_num_si(mx) - isl_val_get_num_si(mn) + 1;
+    isl_val_free(mx);
+    isl_val_free(mn);
+    split_applied = !(extent > 0 && extent <= factor);
+    if (split_applied) {
+        split(level, factor);
+        level_names[level] = outer;
+        level_names[level + 1] = inner;
+    }
+}
+
+void computation::vectorize(var L, int v, var L_outer, var L_inner) {
+    int l = get_loop_level_number_from_dimension_name(L.get_name());
+    bool applied;
+    separate_and_split(l, v, L_outer.get_name(), L_inner.get_name(), applied);
+    tag_vector_level(applied ? l + 1 : l, v);
+}
+void computation::vectorize(var L, int v) {
+    vectorize(L, v, var(fct->generate_new_name(L.get_name() + "_vo")), var(fct->generate_new_name(L.get_name() + "_vi")));
+}
+void computation::unroll(var L, int fac, var L_outer, var L_inner) {
+    int l = get_loop_level_number_from_dimension_name(L.get_name());
+    bool applied;
+    separate_and_split(l, fac, L_outer.get_name(), L_inner.get_name(), applied);
+    tag_unroll_level(applied ? l + 1 : l, fac);
+}
+void computation::unroll(var L, int fac) {
+    unroll(L, fac, var(fct->generate_new_name(L.get_name() + "_uo")), var(fct->generate_new_name(L.get_name() + "_ui")));
+}
+
+int computation::compute_maximal_AST_depth() { return (int)level_names.size(); }
+
+// ------------------------------------------------------------------ ordering
+
+void computation::after(computation &comp, int level) {
+    auto &edges = fct->sched_graph[&comp];
+    auto it = edges.find(this);
+    if (it != edges.end() && it->second > level) level = it->second;
+    edges[this] = level;
+    fct->starting_computations.erase(this);
+    fct->sched_graph_reversed[this][&comp] = level;
+    if (fct->sched_graph_reversed[this].size() > 1)
+        ERROR("computation " + name + " has more than one predecessor in the ordering graph", true);
+}
+
+void computation::after(computation &comp, var level) {
+    after(comp, get_loop_level_number_from_dimension_name(level.get_name()));
+}
+void computation::before(computation &consumer, var L) { consumer.after(*this, L); }
+void computation::before(computation &consumer, int L) { consumer.after(*this, L); }
+
+void computation::between(computation &before_c, int before_l, computation &after_c, int after_l) {
+    auto &g = fct->sched_graph;
+    if (g[&before_c].count(&after_c)) {
+        g[&before_c].erase(&after_c);
+        fct->sched_graph_reversed[&after_c].erase(&before_c);
+    }
+    after(before_c, before_l);
+    after_c.after(*this, after_l);
+}
+void computation::between(computation &before_c, var before_l, computation &after_c, var after_l) {
+    int bl = get_loop_level_number_from_dimension_name(before_l.get_name());
+    int al = after_c.get_loop_level_number_from_dimension_name(after_l.get_name());
+    between(before_c, bl, after_c, al);
+}
+
+computation &computation::then(computation &next, var L) { next.after(*this, L); return next; }
+computation &computation::then(computation &next, int L) { next.after(*this, L); return next; }
+
+computation *computation::get_predecessor() {
+    auto &r = fct->sched_graph_reversed[this];
+    return r.empty() ? nullptr : r.begin()->first;
+}
+
+// Static dimensions before the fuse level are copied from the predecessor; the one right
+// after the fuse level becomes the predecessor's + 10 (reference: tiramisu_core.cpp:2126-2185).
+void computation::after_low_level(computation &comp, int level) {
+    fct->align_schedules();
+    int r = isl_map_dim(schedule, isl_dim_out);
+    int last_static = static_pos(level + 1);
+    if (last_static >= r) ERROR("after: level " + std::to_string(level) + " is deeper than the schedule of " + name, true);
+    for (int pos = 1; pos <= last_static; pos += 2) {
+        isl_val *v = isl_map_plain_get_val_if_fixed(comp.schedule, isl_dim_out, pos);
+        long order = (v && isl_val_is_int(v) == isl_bool_true) ? isl_val_get_num_si(v) : 0;
+        isl_val_free(v);
+        if (pos == last_static) order += 10;
+        // Replace the constant at this position.
+        std::vector<std::string> in, out;
+        for (int i = 0; i < r; i++) { in.push_back("x" + std::to_string(i)); out.push_back(in.back()); }
+        out[pos] = std::to_string(order);
+        apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+    }
+}
+
+// ------------------------------------------------------------------ GPU mapping
+
+void computation::tag_gpu_block_level(int L0) { fct->add_gpu_block_dimensions(name, L0); }
+void computation::tag_gpu_block_level(int L0, int L1) { fct->add_gpu_block_dimensions(name, L0, L1); }
+void computation::tag_gpu_block_level(int L0, int L1, int L2) { fct->add_gpu_block_dimensions(name, L0, L1, L2); }
+void computation::tag_gpu_thread_level(int L0) { fct->add_gpu_thread_dimensions(name, L0); }
+void computation::tag_gpu_thread_level(int L0, int L1) { fct->add_gpu_thread_dimensions(name, L0, L1); }
+void computation::tag_gpu_thread_level(int L0, int L1, int L2) { fct->add_gpu_thread_dimensions(name, L0, L1, L2); }
+
+void computation::tag_gpu_level(int L0, int L1) { tag_gpu_block_level(L0); tag_gpu_thread_level(L1); }
+void computation::tag_gpu_level(int L0, int L1, int L2, int L3) { tag_gpu_block_level(L0, L1); tag_gpu_thread_level(L2, L3); }
+void computation::tag_gpu_level(int L0, int L1, int L2, int L3, int L4, int L5) {
+    tag_gpu_block_level(L0, L1, L2);
+    tag_gpu_thread_level(L3, L4, L5);
+}
+void computation::tag_gpu_level(var L0, var L1) {
+    auto l = get_loop_level_numbers_from_dimension_names({L0.get_name(), L1.get_name()});
+    tag_gpu_level(l[0], l[1]);
+}
+void computation::tag_gpu_level(var L0, var L1, var L2, var L3) {
+    auto l = get_loop_level_numbers_from_dimension_names({L0.get_name(), L1.get_name(), L2.get_name(), L3.get_name()});
+    tag_gpu_level(l[0], l[1], l[2], l[3]);
+}
+void computation::tag_gpu_level(var L0, var L1, var L2, var L3, var L4, var L5) {
+    auto l = get_loop_level_numbers_from_dimension_names(
+        {L0.get_name(), L1.get_name(), L2.get_name(), L3.get_name(), L4.get_name(), L5.get_name()});
+    tag_gpu_level(l[0], l[1], l[2], l[3], l[4], l[5]);
+}
+
+void computation::gpu_tile(var L0, var L1, int sizeX, int sizeY, var L0_outer, var L1_outer, var L0_inner,
+                           var L1_inner) {
+    tile(L0, L1, sizeX, sizeY, L0_outer, L1_outer, L0_inner, L1_inner);
+    tag_gpu_level(L0_outer, L1_outer, L0_inner, L1_inner);
+    thread_block_shape = {sizeX, sizeY};
+}
+void computation::gpu_tile(var L0, var L1, int sizeX, int sizeY) {
+    auto g = [&](const var &v, const char *s) { return var(fct->generate_new_name(v.get_name() + s)); };
+    gpu_tile(L0, L1, sizeX, sizeY, g(L0, "_b"), g(L1, "_b"), g(L0, "_t"), g(L1, "_t"));
+}
+void computation::gpu_tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ, var L0_outer, var L1_outer,
+                           var L2_outer, var L0_inner, var L1_inner, var L2_inner) {
+    tile(L0, L1, L2, sizeX, sizeY, sizeZ, L0_outer, L1_outer, L2_outer, L0_inner, L1_inner, L2_inner);
+    tag_gpu_level(L0_outer, L1_outer, L2_outer, L0_inner, L1_inner, L2_inner);
+    thread_block_shape = {sizeX, sizeY, sizeZ};
+}
+void computation::gpu_tile(var L0, var L1, var L2, int sizeX, int sizeY, int sizeZ) {
+    auto g = [&](const var &v, const char *s) { return var(fct->generate_new_name(v.get_name() + s)); };
+    gpu_tile(L0, L1, L2, sizeX, sizeY, sizeZ, g(L0, "_b"), g(L1, "_b"), g(L2, "_b"), g(L0, "_t"), g(L1, "_t"), g(L2, "_t"));
+}
+
+void computation::gen_time_space_domain() {
+    if (time_space_domain) isl_set_free(time_space_domain);
+    isl_set *d = isl_set_copy(iteration_domain);
+    if (fct->get_program_context())
+        d = isl_set_intersect_params(d, isl_set_copy(fct->get_program_context()));
+    time_space_domain = isl_set_apply(d, isl_map_copy(schedule));
+}
+
+// ------------------------------------------------------------------ input / constant
+
+static std::string fresh_input_name() {
+    static int n = 0;
+    return "_input" + std::to_string(n++);
+}
+
+input::input(std::string nm, std::vector<var> iterator_variables, primitive_t t) {
+    fct = global::get_implicit_function();
+    if (!fct) ERROR("call tiramisu::init() first", true);
+    declared_vars = iterator_variables;
+    init_computation(construct_iteration_domain(nm, iterator_variables), fct, expr(), false, t);
+    if (global::is_auto_data_mapping_set()) allocate_and_map_buffer_automatically(a_input);
+}
+
+input::input(std::vector<var> iterator_variables, primitive_t t) : input(fresh_input_name(), iterator_variables, t) {}
+
+static std::vector<var> vars_from_names_sizes(const std::vector<std::string> &names, const std::vector<expr> &sizes) {
+    if (names.size() != sizes.size()) ERROR("input: as many dimension names as sizes are needed", true);
+    std::vector<var> v;
+    for (size_t i = 0; i < names.size(); i++) v.push_back(var(names[i], expr((int32_t)0), sizes[i]));
+    return v;
+}
+
+input::input(std::string nm, std::vector<std::string> dimension_names, std::vector<expr> dimension_sizes, primitive_t t)
+    : input(nm, vars_from_names_sizes(dimension_names, dimension_sizes), t) {}
+
+std::vector<var> Input::iterators_from_size_expressions(std::vector<expr> sizes) {
+    std::vector<var> v;
+    for (size_t i = 0; i < sizes.size(); i++) v.push_back(var("_in" + std::to_string(i), expr((int32_t)0), sizes[i]));
+    return v;
+}
+Input::Input(std::string nm, std::vector<expr> sizes, primitive_t t) : input(nm, iterators_from_size_expressions(sizes), t) {}
+
+constant::constant(std::string param_name, const expr &param_expr, primitive_t t, bool function_wide,
+                   computation *, int, function *func) {
+    if (!function_wide)
+        ERROR("constant " + param_name + ": only function-wide constants are provided by this build", true);
+    fct = func;
+    if (!fct) ERROR("call tiramisu::init() first", true);
+    ctx = fct->get_isl_ctx();
+    name = param_name;
+    expression = param_expr;
+    data_type = t;
+    is_let = true;
+    schedule_this = false;
+    iteration_domain = isl_set_read_from_str(ctx, ("{ " + param_name + "[0] }").c_str());
+    iterator_names_ = {"_zero"};
+    level_names = iterator_names_;
+    set_identity_schedule();
+    fct->add_invariant(this);
+}
+
+constant::constant(std::string param_name, const expr &param_expr)
+    : constant(param_name, param_expr, param_expr.get_data_type(), true, nullptr, 0, global::get_implicit_function()) {}
+constant::constant(std::string param_name, const expr &param_expr, primitive_t t, function *func)
+    : constant(param_name, param_expr, t, true, nullptr, 0, func) {}
+
+constant::operator expr() { return var(data_type, name); }
+
+// ------------------------------------------------------------------ block
+
+block::block(const std::vector<computation *> c) : children(c) {}
+
+#define FORALL(call) do { for (auto c : children) c->call; } while (0)
+void block::gpu_tile(var L0, var L1, int X, int Y) {
+    // All children must get the same generated names.
+    function *f = children.empty() ? nullptr : children[0]->get_function();
+    auto g = [&](const var &v, const char *s) { return var(f->generate_new_name(v.get_name() + s)); };
+    gpu_tile(L0, L1, X, Y, g(L0, "_b"), g(L1, "_b"), g(L0, "_t"), g(L1, "_t"));
+}
+void block::gpu_tile(var L0, var L1, int X, int Y, var a, var b, var c_, var d) { FORALL(gpu_tile(L0, L1, X, Y, a, b, c_, d)); }
+void block::gpu_tile(var L0, var L1, var L2, int X, int Y, int Z) {
+    function *f = children.empty() ? nullptr : children[0]->get_function();
+    auto g = [&](const var &v, const char *s) { return var(f->generate_new_name(v.get_name() + s)); };
+    gpu_tile(L0, L1, L2, X, Y, Z, g(L0, "_b"), g(L1, "_b"), g(L2, "_b"), g(L0, "_t"), g(L1, "_t"), g(L2, "_t"));
+}
+void block::gpu_tile(var L0, var L1, var L2, int X, int Y, int Z, var a, var b, var c_, var d, var e, var f) {
+    FORALL(gpu_tile(L0, L1, L2, X, Y, Z, a, b, c_, d, e, f));
+}
+void block::interchange(var L0, var L1) { FORALL(interchange(L0, L1)); }
+void block::interchange(int L0, int L1) { FORALL(interchange(L0, L1)); }
+void block::parallelize(var L) { FORALL(parallelize(L)); }
+void block::shift(var L0, int n) { FORALL(shift(L0, n)); }
+void block::skew(var i, var j, int f, var ni, var nj) { FORALL(skew(i, j, f, ni, nj)); }
+void block::split(var L0, int X) {
+    function *f = children[0]->get_function();
+    split(L0, X, var(f->generate_new_name(L0.get_name() + "_o")), var(f->generate_new_name(L0.get_name() + "_i")));
+}
+void block::split(var L0, int X, var o, var i) { FORALL(split(L0, X, o, i)); }
+void block::split(int L0, int X) { FORALL(split(L0, X)); }
+void block::tile(var L0, var L1, int X, int Y) {
+    function *f = children[0]->get_function();
+    auto g = [&](const var &v, const char *s) { return var(f->generate_new_name(v.get_name() + s)); };
+    tile(L0, L1, X, Y, g(L0, "_o"), g(L1, "_o"), g(L0, "_i"), g(L1, "_i"));
+}
+void block::tile(var L0, var L1, int X, int Y, var a, var b, var c_, var d) { FORALL(tile(L0, L1, X, Y, a, b, c_, d)); }
+void block::tile(var L0, var L1, var L2, int X, int Y, int Z) {
+    function *f = children[0]->get_function();
+    auto g = [&](const var &v, const char *s) { return var(f->generate_new_name(v.get_name() + s)); };
+    tile(L0, L1, L2, X, Y, Z, g(L0, "_o"), g(L1, "_o"), g(L2, "_o"), g(L0, "_i"), g(L1, "_i"), g(L2, "_i"));
+}
+void block::tile(var L0, var L1, var L2, int X, int Y, int Z, var a, var b, var c_, var d, var e, var f) {
+    FORALL(tile(L0, L1, L2, X, Y, Z, a, b, c_, d, e, f));
+}
+void block::tile(int L0, int L1, int X, int Y) { FORALL(tile(L0, L1, X, Y)); }
+void block::tile(int L0, int L1, int L2, int X, int Y, int Z) { FORALL(tile(L0, L1, L2, X, Y, Z)); }
+void block::unroll(var L, int fac) {
+    function *f = children[0]->get_function();
+    unroll(L, fac, var(f->generate_new_name(L.get_name() + "_uo")), var(f->generate_new_name(L.get_name() + "_ui")));
+}
+void block::unroll(var L, int fac, var o, var i) { FORALL(unroll(L, fac, o, i)); }
+void block::vectorize(var L, int v) {
+    function *f = children[0]->get_function();
+    vectorize(L, v, var(f->generate_new_name(L.get_name() + "_vo")), var(f->generate_new_name(L.get_name() + "_vi")));
+}
+void block::vectorize(var L, int v, var o, var i) { FORALL(vectorize(L, v, o, i)); }
+#undef FORALL
+
+}  // namespace tiramisu

@@ -1,0 +1,29 @@
+// Small string helpers shared by the compiler sources.
+#ifndef TIRAMISU_AMD_UTIL_H
+#define TIRAMISU_AMD_UTIL_H
+#include <string>
+#include <vector>
+
+namespace tiramisu {
+
+inline std::string join(const std::vector<std::string> &v, const std::string &sep) {
+    std::string r;
+    for (size_t i = 0; i < v.size(); i++) r += (i ? sep : std::string()) + v[i];
+    return r;
+}
+
+inline std::string replace_all(std::string s, const std::string &from, const std::string &to) {
+    size_t pos = 0;
+    while ((pos = s.find(from, pos)) != std::string::npos) {
+        s.replace(pos, from.size(), to);
+        pos += to.size();
+    }
+    return s;
+}
+
+class expr;
+/** isl syntax for an integer (quasi-)affine expression; sets \p ok to false otherwise. */
+std::string expr_to_isl_str(const expr &e, bool &ok);
+
+}  // namespace tiramisu
+#endif
