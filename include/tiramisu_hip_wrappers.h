@@ -1,0 +1,83 @@
+/* C ABI of the runtime layer that generated Tiramisu host code calls to reach the GPU.
+ *
+ * This is the drop-in boundary of the HIP back-end: plain pointers and sizes, no C++ or
+ * framework types.  Each entry point names the reference interface it replaces
+ * (src/tiramisu_cuda_wrappers.cpp of the reference tree).  Failure model of the
+ * reference is kept: a failing HIP call prints "Error at <function>: <reason>" on
+ * stderr and ends the process with status 1, so successful calls return 0.
+ *
+ * Stream model: every call works on the calling thread's *current stream*.  It starts as
+ * HIP's per-thread default stream (the reference compiles with
+ * --default-stream per-thread, tiramisu_codegen_cuda.cpp:1745) and can be replaced
+ * with tiramisu_hip_set_stream() by callers that time or overlap work.
+ */
+#ifndef TIRAMISU_HIP_WRAPPERS_H
+#define TIRAMISU_HIP_WRAPPERS_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- memory (replaces tiramisu_cuda_malloc / tiramisu_cuda_free,
+ *      tiramisu_cuda_wrappers.cpp:55-68) ---- */
+void *tiramisu_hip_malloc(uint64_t size);
+int tiramisu_hip_free(void *ptr);
+
+/* ---- copies (replace tiramisu_cuda_memcpy_to_device / _to_host / _to_symbol,
+ *      tiramisu_cuda_wrappers.cpp:34-53).  Issued with hipMemcpyAsync on the current
+ *      stream and completed before returning, like the reference's cudaMemcpy. ---- */
+int tiramisu_hip_memcpy_to_device(void *to, void *from, uint64_t size);
+int tiramisu_hip_memcpy_to_host(void *to, void *from, uint64_t size);
+int tiramisu_hip_memcpy_to_symbol(void *to, void *from, uint64_t size);
+/* Device-to-device copy; the reference prints such copies as device-to-host
+ * (tiramisu_codegen_cuda.cpp:1416-1419), which its runtime tolerates by accident. */
+int tiramisu_hip_memcpy_device_to_device(void *to, void *from, uint64_t size);
+
+/* ---- synchronisation (replaces tiramisu_cuda_stream_synchronize,
+ *      tiramisu_cuda_wrappers.cpp:164-169); the argument is ignored ---- */
+int32_t tiramisu_hip_stream_synchronize(int32_t dummy);
+
+/* ---- GEMM library call (replaces tiramisu_cublas_sgemm / tiramisu_cublas_dgemm,
+ *      tiramisu_cuda_wrappers.cpp:74-162).  Row-major C = alpha*op(A)*op(B) + beta*C,
+ *      A is MxK, B is KxN after op().  A leading dimension of 0 means tightly packed
+ *      (ldA = transposeA ? M : K, ldB = transposeB ? K : N, ldC = N); offsets are in
+ *      elements.  Runs this library's own MFMA kernels; no BLAS library is involved. ---- */
+int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
+                       float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
+                       uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
+int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha,
+                       double beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
+                       uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
+
+/* ---- code objects and launches.  The reference links nvcc-compiled kernel wrappers
+ *      (_kernel_N_wrapper, tiramisu_codegen_cuda.cpp:1288-1318) into the program; here
+ *      generated host code is plain C++ that embeds a gfx950 code object and launches
+ *      its kernels through these three calls. ---- */
+/* Load a code object image (an .hsaco file's bytes) on the current device. */
+void *tiramisu_hip_module_load(const void *image, uint64_t size);
+/* Look a kernel up by name; exits with status 1 if the module does not define it. */
+void *tiramisu_hip_module_get_function(void *module, const char *kernel_name);
+/* Launch on the current stream.  args[i] points to the i-th kernel argument. */
+int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3],
+                        uint32_t dynamic_lds_bytes, void **args);
+
+/* ---- stream and timing helpers for wrappers and benchmarks (the reference's
+ *      benchmarks bracket device work with get_time() calls,
+ *      benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp:66-69) ---- */
+/* Make `stream` (a hipStream_t) the calling thread's current stream; NULL restores the
+ * per-thread default stream. */
+int tiramisu_hip_set_stream(void *stream);
+void *tiramisu_hip_get_stream(void);
+void *tiramisu_hip_event_create(void);
+int tiramisu_hip_event_record(void *event);              /* on the current stream */
+float tiramisu_hip_event_elapsed_ms(void *start, void *stop); /* waits for `stop` */
+int tiramisu_hip_event_destroy(void *event);
+int tiramisu_hip_device_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

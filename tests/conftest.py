@@ -1,0 +1,22 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X; run through the C ABI on the device")
+
+
+@pytest.fixture(scope="session")
+def programs_dir():
+    return os.path.join(ROOT, "tests", "programs")
+
+
+@pytest.fixture(scope="session")
+def product_programs_dir():
+    return os.path.join(ROOT, "tiramisu_amd", "programs")

@@ -1,0 +1,139 @@
+"""Build steps of the Tiramisu HIP back-end.
+
+Three kinds of artefacts, all in-tree so that they travel to the GPU machine:
+
+* ``tiramisu_amd/libtiramisu.so``              the compiler (front-end over isl, AST lowering,
+                                               HIP + host-glue emitters), plain C++ (g++);
+* ``tiramisu_amd/libtiramisu_hip_wrappers.so`` the runtime C ABI (hipcc, gfx950);
+* ``<dir>/build/lib<program>.so``              one shared library per Tiramisu program: the
+                                               generator is compiled and run here (it calls hipcc
+                                               to produce the gfx950 code object), and the host
+                                               object it writes is linked against the runtime.
+
+Nothing here needs a GPU: hipcc cross-compiles for gfx950.
+"""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "tiramisu_amd")
+CSRC = os.path.join(PKG, "csrc")
+INCLUDE = os.path.join(ROOT, "include")
+HIPCC = os.environ.get("HIPCC_PATH", "/opt/rocm/bin/hipcc")
+ISL = "-l:libisl.so.23"
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+COMPILER_SOURCES = ["expr.cpp", "core.cpp", "astgen.cpp", "c_print.cpp", "hip_backend.cpp",
+                    "recognize.cpp"]
+
+PROGRAM_DIRS = [os.path.join(PKG, "programs"), os.path.join(ROOT, "tests", "programs")]
+
+
+def _run(cmd, cwd=None, quiet=True):
+    r = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        sys.stderr.write("command failed: %s\n%s\n" % (" ".join(cmd), r.stdout))
+        raise RuntimeError("build step failed: " + " ".join(cmd[:3]))
+    if not quiet and r.stdout.strip():
+        print(r.stdout)
+    return r.stdout
+
+
+def _newer(target, sources):
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(s) <= t for s in sources if os.path.exists(s))
+
+
+def compiler_library():
+    return os.path.join(PKG, "libtiramisu.so")
+
+
+def wrappers_library():
+    return os.path.join(PKG, "libtiramisu_hip_wrappers.so")
+
+
+def build_compiler(force=True):
+    srcs = [os.path.join(CSRC, s) for s in COMPILER_SOURCES]
+    deps = srcs + [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".h")] + \
+        [os.path.join(INCLUDE, "tiramisu", h) for h in os.listdir(os.path.join(INCLUDE, "tiramisu"))]
+    kdir = os.path.join(CSRC, "kernels")
+    deps += [os.path.join(kdir, h) for h in os.listdir(kdir)]
+    out = compiler_library()
+    if not force and _newer(out, deps):
+        return out
+    _run(["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-I" + INCLUDE,
+          '-DTIRAMISU_AMD_INCLUDE_DIR="%s"' % INCLUDE,
+          '-DTIRAMISU_AMD_KERNEL_DIR="%s"' % kdir,
+          "-o", out] + srcs + [ISL])
+    return out
+
+
+def build_wrappers(force=True):
+    src = os.path.join(CSRC, "hip_wrappers.hip")
+    kdir = os.path.join(CSRC, "kernels")
+    deps = [src, os.path.join(INCLUDE, "tiramisu_hip_wrappers.h")] + \
+        [os.path.join(kdir, h) for h in os.listdir(kdir)]
+    out = wrappers_library()
+    if not force and _newer(out, deps):
+        return out
+    _run([HIPCC] + HIP_FLAGS + ["-fPIC", "-shared", "-o", out, src])
+    return out
+
+
+def program_library(directory, name):
+    return os.path.join(directory, "build", "lib%s.so" % name)
+
+
+def build_program(source, force=True, extra_objects=(), defines=()):
+    """Compile and run the generator ``source`` (a Tiramisu program), then link every host
+    object it wrote (build/<x>.o) into build/lib<x>.so next to the source."""
+    directory = os.path.dirname(os.path.abspath(source))
+    stem = os.path.splitext(os.path.basename(source))[0]
+    bdir = os.path.join(directory, "build")
+    os.makedirs(bdir, exist_ok=True)
+    gen = os.path.join(bdir, "gen_" + stem)
+    stamp = os.path.join(bdir, stem + ".stamp")
+    if not force and _newer(stamp, [source, compiler_library(), wrappers_library()]):
+        return
+    before = {f: os.path.getmtime(os.path.join(bdir, f)) for f in os.listdir(bdir) if f.endswith(".o")}
+    _run(["g++", "-std=c++17", "-O1", "-I" + INCLUDE, "-I" + directory] + ["-D" + d for d in defines] +
+         ["-o", gen, source] + list(extra_objects) +
+         ["-L" + PKG, "-ltiramisu", "-Wl,-rpath," + PKG])
+    env_out = _run([gen], cwd=directory)
+    produced = [f for f in os.listdir(bdir) if f.endswith(".o") and
+                (f not in before or os.path.getmtime(os.path.join(bdir, f)) > before[f])]
+    for obj in produced:
+        name = obj[:-2]
+        if name.startswith("generated_fct_"):
+            name = name[len("generated_fct_"):]
+        lib = os.path.join(bdir, "lib%s.so" % name)
+        _run(["g++", "-shared", "-o", lib, os.path.join(bdir, obj), "-L" + PKG, "-ltiramisu_hip_wrappers",
+              "-Wl,-rpath,$ORIGIN/" + os.path.relpath(PKG, bdir)])
+    with open(stamp, "w") as f:
+        f.write(env_out)
+    return produced
+
+
+def program_sources():
+    out = []
+    for d in PROGRAM_DIRS:
+        if os.path.isdir(d):
+            out += sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(".cpp"))
+    return out
+
+
+def build_all(force=True, verbose=False):
+    build_compiler(force)
+    build_wrappers(force)
+    for src in program_sources():
+        if verbose:
+            print("[build] program", os.path.relpath(src, ROOT), flush=True)
+        build_program(src, force)
+
+
+if __name__ == "__main__":
+    build_all(force="--force" in sys.argv, verbose=True)

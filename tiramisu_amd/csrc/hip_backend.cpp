@@ -1,0 +1,591 @@
+// HIP back-end driver: walks the lowered loop program, replaces every GPU-tagged loop nest
+// by kernel launches, prints the host glue as plain C++ (no HIP headers: it reaches the
+// device only through the tiramisu_hip_* C ABI), compiles the kernels to a gfx950 code
+// object with hipcc and embeds that object into the host object file.
+//
+// Artefacts for codegen(..., "f.o", true):
+//   f.o.hip       kernel source            (kept when HIP_NO_OVERWRITE is set, like the
+//   f.o.hsaco     gfx950 code object        reference's CUDA_NO_OVERWRITE, tiramisu_codegen_cuda.cpp:1808)
+//   f.o.host.cpp  host glue source
+//   f.o           host object; exports  extern "C" int <function>(halide_buffer_t *...)
+#include "hip_backend.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <sstream>
+
+#include "util.h"
+
+namespace tiramisu {
+namespace hipgen {
+
+using lir::leaf_kind;
+using lir::node;
+using lir::node_kind;
+using lir::node_ptr;
+
+int context::next_kernel_id() {
+    static int counter = 0;  // process-wide, like the reference's kernel_count (tiramisu_codegen_cuda.cpp:1320)
+    return counter++;
+}
+
+namespace {
+
+bool depends_on(const expr &e, const std::set<std::string> &names) {
+    bool d = false;
+    e.visit([&](const expr &x) {
+        if (x.get_expr_type() == e_var && names.count(x.get_name())) d = true;
+    });
+    return d;
+}
+
+std::string pad(int n) { return std::string(n * 4, ' '); }
+
+// ---------------------------------------------------------------- generic kernel
+
+struct generic_kernel_gen {
+    context &ctx;
+    function *f;
+    c_printer dev;
+    std::set<std::string> used_buffers, used_scalars;
+    std::set<std::string> inner;        // iterators and let names defined inside the kernel
+    std::set<std::string> declared;     // buffers declared by an allocate leaf inside the kernel
+    std::vector<expr> grid_ext[3], block_ext[3];
+    int loops_per_dim[2][3] = {{0, 0, 0}, {0, 0, 0}};
+    std::ostringstream body;
+
+    generic_kernel_gen(context &c) : ctx(c), f(c.f) {
+        dev.fct = f;
+        dev.device = true;
+        dev.used_buffers = &used_buffers;
+        dev.used_scalars = &used_scalars;
+    }
+
+    void prepass(const node_ptr &root) {
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind == node_kind::loop) {
+                inner.insert(n->iterator);
+                if (n->gpu_block >= 0) loops_per_dim[0][n->gpu_block]++;
+                if (n->gpu_thread >= 0) loops_per_dim[1][n->gpu_thread]++;
+            }
+            if (n->kind == node_kind::leaf)
+                for (auto &l : n->lets) inner.insert(l.first);
+        });
+    }
+
+    // Extent of a mapped loop as seen from the host: upper - init + 1, where a min() bound that
+    // involves in-kernel iterators contributes only its kernel-invariant arguments.
+    expr host_extent(const node_ptr &n, bool &needs_guard) {
+        if (depends_on(n->init, inner))
+            ERROR("GPU-mapped loop " + n->iterator + " has a lower bound that varies inside the kernel", true);
+        expr up = n->upper;
+        needs_guard = false;
+        if (depends_on(up, inner)) {
+            needs_guard = true;
+            std::vector<expr> parts;
+            std::function<void(const expr &)> split_min = [&](const expr &e) {
+                if (e.get_expr_type() == e_op && e.get_op_type() == o_min) {
+                    split_min(e.get_operand(0));
+                    split_min(e.get_operand(1));
+                } else if (!depends_on(e, inner)) {
+                    parts.push_back(e);
+                }
+            };
+            split_min(up);
+            if (parts.empty())
+                ERROR("GPU-mapped loop " + n->iterator + " has no kernel-invariant upper bound", true);
+            up = parts[0];
+            for (size_t i = 1; i < parts.size(); i++) up = expr(o_min, up, parts[i]);
+        }
+        return lir::simplify(lir::simplify(up - n->init) + 1);
+    }
+
+    void emit(const node_ptr &n, int ind) {
+        if (!n) return;
+        switch (n->kind) {
+        case node_kind::block:
+            for (auto &c : n->children) emit(c, ind);
+            break;
+        case node_kind::cond:
+            body << pad(ind) << "if (" << dev.print(n->condition) << ") {\n";
+            emit(n->then_body, ind + 1);
+            if (n->else_body) {
+                body << pad(ind) << "} else {\n";
+                emit(n->else_body, ind + 1);
+            }
+            body << pad(ind) << "}\n";
+            break;
+        case node_kind::loop: emit_loop(n, ind); break;
+        case node_kind::leaf: emit_leaf(n, ind); break;
+        }
+    }
+
+    void emit_loop(const node_ptr &n, int ind) {
+        const bool is_block = n->gpu_block >= 0, is_thread = n->gpu_thread >= 0;
+        if (is_block || is_thread) {
+            const int dim = is_block ? n->gpu_block : n->gpu_thread;
+            bool guard;
+            expr ext = host_extent(n, guard);
+            (is_block ? grid_ext : block_ext)[dim].push_back(ext);
+            if (loops_per_dim[is_block ? 0 : 1][dim] > 1) guard = true;
+            const char *idx = is_block ? "blockIdx." : "threadIdx.";
+            body << pad(ind) << "{\n";
+            body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)" << idx << "xyz"[dim] << " + "
+                 << dev.print(n->init) << ";\n";
+            if (guard) body << pad(ind + 1) << "if (" << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+            emit(n->body, ind + (guard ? 2 : 1));
+            if (guard) body << pad(ind + 1) << "}\n";
+            body << pad(ind) << "}\n";
+            return;
+        }
+        expr lo = lir::simplify(n->init), up = lir::simplify(n->upper);
+        bool small = lo.is_integer_literal() && up.is_integer_literal() && up.get_int_val() - lo.get_int_val() < 32;
+        if (n->unrolled || small) body << pad(ind) << "#pragma unroll\n";
+        body << pad(ind) << "for (int32_t " << n->iterator << " = " << dev.print(n->init) << "; " << n->iterator
+             << " <= " << dev.print(n->upper) << "; " << n->iterator << " += " << dev.print(n->increment) << ") {\n";
+        emit(n->body, ind + 1);
+        body << pad(ind) << "}\n";
+    }
+
+    std::string declaration(const buffer *b) {
+        std::string t = primitive_c_name(b->get_elements_type());
+        switch (b->get_location()) {
+        case memory_location::reg: return t + " " + b->get_name() + ";";
+        case memory_location::local:
+        case memory_location::shared: {
+            if (!b->has_constant_extents())
+                ERROR("buffer " + b->get_name() + " lives in a GPU kernel and needs constant extents", true);
+            long cnt = 1;
+            for (auto &d : b->get_dim_sizes()) cnt *= lir::simplify(d).get_int_val();
+            return std::string(b->get_location() == memory_location::shared ? "__shared__ " : "") + t + " " +
+                   b->get_name() + "[" + std::to_string(cnt) + "];";
+        }
+        default:
+            ERROR("buffer " + b->get_name() + " is allocated inside a GPU kernel but is neither shared, local nor register", true);
+        }
+        return "";
+    }
+
+    void emit_leaf(const node_ptr &n, int ind) {
+        switch (n->lkind) {
+        case leaf_kind::sync: body << pad(ind) << "__syncthreads();\n"; return;
+        case leaf_kind::allocate:
+            declared.insert(n->target->get_name());
+            body << pad(ind) << declaration(n->target) << "\n";
+            return;
+        case leaf_kind::release: return;
+        case leaf_kind::copy: ERROR("memcpy computation " + n->comp->get_name() + " is scheduled inside a GPU kernel", true);
+        default: break;
+        }
+        int i2 = ind;
+        const bool scoped = !n->lets.empty() || n->predicate.is_defined();
+        if (scoped) { body << pad(ind) << "{\n"; i2++; }
+        for (auto &l : n->lets)
+            body << pad(i2) << "const " << primitive_c_name(l.second.get_data_type()) << " " << l.first << " = "
+                 << dev.print(l.second) << ";\n";
+        if (n->predicate.is_defined()) { body << pad(i2) << "if (" << dev.print(n->predicate) << ") {\n"; i2++; }
+        if (n->lhs) body << pad(i2) << dev.store(n->lhs, n->lhs_index, dev.print(n->rhs), n->rhs.get_data_type()) << "\n";
+        else body << pad(i2) << dev.print(n->rhs) << ";\n";
+        if (n->predicate.is_defined()) { i2--; body << pad(i2) << "}\n"; }
+        if (scoped) body << pad(ind) << "}\n";
+    }
+};
+
+std::string max_text(const std::vector<expr> &v, const c_printer &host) {
+    if (v.empty()) return "1";
+    bool all_lit = true;
+    long m = 0;
+    for (auto &e : v) {
+        if (e.is_integer_literal()) m = std::max<long>(m, e.get_int_val());
+        else all_lit = false;
+    }
+    if (all_lit) return std::to_string(m);
+    std::string s = host.print(v[0]);
+    for (size_t i = 1; i < v.size(); i++) s = "t_max(" + s + ", " + host.print(v[i]) + ")";
+    return "(uint32_t)t_max((int32_t)0, (int32_t)(" + s + "))";
+}
+
+}  // namespace
+
+kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
+    generic_kernel_gen g(ctx);
+    g.prepass(root);
+    g.emit(root, 1);
+
+    kernel k;
+    k.how = "generic";
+    k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
+    function *f = ctx.f;
+
+    // parameters: free scalars sorted by name, then global buffers sorted by name
+    // (reference: tiramisu_codegen_cuda.cpp:1324-1331)
+    c_printer host;
+    host.fct = f;
+    std::set<std::string> extent_scalars, extent_buffers;
+    host.used_scalars = &extent_scalars;
+    host.used_buffers = &extent_buffers;
+    for (int d = 0; d < 3; d++) {
+        k.grid[d] = max_text(g.grid_ext[d], host);
+        k.block[d] = max_text(g.block_ext[d], host);
+    }
+    std::vector<std::string> top_decls;
+    for (auto &nm : g.used_scalars) {
+        if (g.inner.count(nm)) continue;
+        primitive_t t = global::get_loop_iterator_data_type();
+        for (auto c : f->get_invariants())
+            if (c->get_name() == nm) t = c->get_data_type();
+        k.params.push_back({false, nm, t});
+    }
+    for (auto &nm : g.used_buffers) {
+        buffer *b = f->get_buffers().at(nm);
+        switch (b->get_location()) {
+        case memory_location::global: k.params.push_back({true, nm, b->get_elements_type()}); break;
+        case memory_location::host:
+            ERROR("buffer " + nm + " is used inside a GPU kernel but lives in host memory; tag it with tag_gpu_global() "
+                  "and copy it with memcpy()", true);
+        case memory_location::constant:
+            ERROR("buffer " + nm + ": constant memory is not provided by this back-end; use tag_gpu_global()", true);
+        default:
+            if (!g.declared.count(nm)) top_decls.push_back(g.declaration(b));
+        }
+    }
+
+    std::ostringstream os;
+    long threads = 1;
+    bool lit = true;
+    for (int d = 0; d < 3; d++) {
+        char *end = nullptr;
+        long v = strtol(k.block[d].c_str(), &end, 10);
+        if (end && *end == 0) threads *= v; else lit = false;
+    }
+    os << "extern \"C\" __global__ void ";
+    if (lit) os << "__launch_bounds__(" << threads << ") ";
+    os << k.name << "(";
+    for (size_t i = 0; i < k.params.size(); i++) {
+        auto &p = k.params[i];
+        os << (i ? ", " : "");
+        if (p.is_buffer) os << primitive_c_name(p.type) << " *__restrict__ " << p.name;
+        else os << "const " << primitive_c_name(p.type) << " " << p.name;
+    }
+    os << ")\n{\n";
+    for (auto &d : top_decls) os << "    " << d << "\n";
+    os << g.body.str() << "}\n";
+    k.source = os.str();
+    return k;
+}
+
+std::string launch_text(const kernel &k, const std::string &ind) {
+    std::ostringstream os;
+    os << ind << "{\n";
+    os << ind << "    void *_args[] = {";
+    for (size_t i = 0; i < k.params.size(); i++) os << (i ? ", " : "") << "(void *)&" << k.params[i].name;
+    if (k.params.empty()) os << "nullptr";
+    os << "};\n";
+    os << ind << "    const uint32_t _grid[3] = {(uint32_t)(" << k.grid[0] << "), (uint32_t)(" << k.grid[1] << "), (uint32_t)("
+       << k.grid[2] << ")};\n";
+    os << ind << "    const uint32_t _block[3] = {(uint32_t)(" << k.block[0] << "), (uint32_t)(" << k.block[1]
+       << "), (uint32_t)(" << k.block[2] << ")};\n";
+    os << ind << "    static void *_fn = tiramisu_hip_module_get_function(_tiramisu_module(), \"" << k.name << "\");\n";
+    os << ind << "    tiramisu_hip_launch(_fn, _grid, _block, (uint32_t)(" << k.lds_bytes << "), _args);\n";
+    os << ind << "}\n";
+    return os.str();
+}
+
+namespace {
+
+// ---------------------------------------------------------------- host glue
+
+struct host_gen {
+    context &ctx;
+    function *f;
+    c_printer hp;
+    std::ostringstream out;
+    std::set<std::string> extern_calls;
+    std::vector<std::string> extern_decls;
+    std::vector<node *> loop_stack;
+
+    host_gen(context &c) : ctx(c), f(c.f) { hp.fct = f; }
+
+    static bool is_gpu_loop(const node_ptr &n) { return n->kind == node_kind::loop && (n->gpu_block >= 0 || n->gpu_thread >= 0); }
+
+    void require_host(const buffer *b, const std::string &who) {
+        if (b->get_location() != memory_location::host)
+            ERROR("computation " + who + " runs on the host but touches GPU buffer " + b->get_name() +
+                  "; map its loops to the GPU (gpu_tile / tag_gpu_level)", true);
+    }
+
+    void declare_call(const expr &call) {
+        const std::string &nm = call.get_name();
+        if (nm.rfind("tiramisu_hip_", 0) == 0 || extern_calls.count(nm)) return;
+        extern_calls.insert(nm);
+        std::string s = "extern \"C\" " + primitive_c_name(call.get_data_type()) + " " + nm + "(";
+        for (size_t i = 0; i < call.get_arguments().size(); i++) {
+            const expr &a = call.get_arguments()[i];
+            std::string t = (a.get_expr_type() == e_op && a.get_op_type() == o_buffer)
+                                ? "void *" : primitive_c_name(a.get_data_type());
+            s += (i ? ", " : "") + t;
+        }
+        extern_decls.push_back(s + ");");
+    }
+
+    void emit(const node_ptr &n, int ind) {
+        if (!n) return;
+        switch (n->kind) {
+        case node_kind::block:
+            for (auto &c : n->children) emit(c, ind);
+            break;
+        case node_kind::cond:
+            out << pad(ind) << "if (" << hp.print(n->condition) << ") {\n";
+            emit(n->then_body, ind + 1);
+            if (n->else_body) {
+                out << pad(ind) << "} else {\n";
+                emit(n->else_body, ind + 1);
+            }
+            out << pad(ind) << "}\n";
+            break;
+        case node_kind::loop:
+            if (is_gpu_loop(n)) {
+                emit_kernel_nest(n, ind);
+            } else {
+                // a time loop around a stencil nest may be taken over as a whole
+                launch_plan plan;
+                if (emit_stencil(ctx, nullptr, n, plan)) {
+                    for (auto &k : plan.kernels) ctx.kernels.push_back(k);
+                    out << plan.host_code;
+                    break;
+                }
+                out << pad(ind) << "for (int32_t " << n->iterator << " = " << hp.print(n->init) << "; " << n->iterator
+                    << " <= " << hp.print(n->upper) << "; " << n->iterator << " += " << hp.print(n->increment) << ") {\n";
+                emit(n->body, ind + 1);
+                out << pad(ind) << "}\n";
+            }
+            break;
+        case node_kind::leaf: emit_leaf(n, ind); break;
+        }
+    }
+
+    void emit_kernel_nest(const node_ptr &n, int ind) {
+        launch_plan plan;
+        if (emit_contraction(ctx, n, plan) || emit_stencil(ctx, n, nullptr, plan)) {
+            for (auto &k : plan.kernels) ctx.kernels.push_back(k);
+            if (!plan.host_code.empty()) out << plan.host_code;
+            else for (auto &k : plan.kernels) out << launch_text(k, pad(ind));
+            return;
+        }
+        kernel k = emit_generic_kernel(ctx, n);
+        ctx.kernels.push_back(k);
+        out << launch_text(k, pad(ind));
+    }
+
+    void emit_leaf(const node_ptr &n, int ind) {
+        switch (n->lkind) {
+        case leaf_kind::sync: return;
+        case leaf_kind::copy: {
+            buffer *s = n->copy_from, *d = n->copy_to;
+            bool sg = s->get_location() == memory_location::global, dg = d->get_location() == memory_location::global;
+            std::string bytes = "(uint64_t)(" + hp.element_count(s) + ") * sizeof(" + primitive_c_name(s->get_elements_type()) + ")";
+            const char *fn = (!sg && dg) ? "tiramisu_hip_memcpy_to_device" : (sg && !dg) ? "tiramisu_hip_memcpy_to_host"
+                             : (sg && dg) ? "tiramisu_hip_memcpy_device_to_device" : nullptr;
+            if (fn) out << pad(ind) << fn << "((void *)" << d->get_name() << ", (void *)" << s->get_name() << ", " << bytes << ");\n";
+            else out << pad(ind) << "memcpy((void *)" << d->get_name() << ", (void *)" << s->get_name() << ", " << bytes << ");\n";
+            return;
+        }
+        case leaf_kind::allocate: {
+            buffer *b = n->target;
+            std::string t = primitive_c_name(b->get_elements_type());
+            std::string bytes = "(uint64_t)(" + hp.element_count(b) + ") * sizeof(" + t + ")";
+            if (b->get_location() == memory_location::global)
+                out << pad(ind) << b->get_name() << " = (" << t << " *)tiramisu_hip_malloc(" << bytes << ");\n";
+            else if (b->get_location() == memory_location::host)
+                out << pad(ind) << b->get_name() << " = (" << t << " *)malloc(" << bytes << ");\n";
+            else
+                ERROR("allocation of " + b->get_name() + " (a shared/local/register buffer) is scheduled outside a GPU kernel", true);
+            return;
+        }
+        case leaf_kind::release: {
+            buffer *b = n->target;
+            if (b->get_location() == memory_location::global) out << pad(ind) << "tiramisu_hip_free((void *)" << b->get_name() << ");\n";
+            else out << pad(ind) << "free((void *)" << b->get_name() << ");\n";
+            return;
+        }
+        default: break;
+        }
+        // host-side assignment or call
+        n->rhs.visit([&](const expr &e) {
+            if (e.get_expr_type() == e_op && e.get_op_type() == o_access) require_host(f->get_buffers().at(e.get_name()), n->comp->get_name());
+            if (e.get_expr_type() == e_op && e.get_op_type() == o_call) declare_call(e);
+        });
+        if (n->lhs) require_host(n->lhs, n->comp->get_name());
+        int i2 = ind;
+        const bool scoped = !n->lets.empty() || n->predicate.is_defined();
+        if (scoped) { out << pad(ind) << "{\n"; i2++; }
+        for (auto &l : n->lets)
+            out << pad(i2) << "const " << primitive_c_name(l.second.get_data_type()) << " " << l.first << " = " << hp.print(l.second) << ";\n";
+        if (n->predicate.is_defined()) { out << pad(i2) << "if (" << hp.print(n->predicate) << ") {\n"; i2++; }
+        if (n->lhs) out << pad(i2) << hp.store(n->lhs, n->lhs_index, hp.print(n->rhs), n->rhs.get_data_type()) << "\n";
+        else out << pad(i2) << hp.print(n->rhs) << ";\n";
+        if (n->predicate.is_defined()) { i2--; out << pad(i2) << "}\n"; }
+        if (scoped) out << pad(ind) << "}\n";
+    }
+};
+
+void collect_used_buffers(const node_ptr &root, std::set<std::string> &used) {
+    lir::walk(root, [&](const node_ptr &n) {
+        auto scan = [&](const expr &e) {
+            if (!e.is_defined()) return;
+            e.visit([&](const expr &x) {
+                if (x.get_expr_type() == e_op && (x.get_op_type() == o_access || x.get_op_type() == o_buffer || x.get_op_type() == o_address_of))
+                    used.insert(x.get_name());
+            });
+        };
+        if (n->kind != node_kind::leaf) return;
+        if (n->lhs) used.insert(n->lhs->get_name());
+        if (n->copy_from) used.insert(n->copy_from->get_name());
+        if (n->copy_to) used.insert(n->copy_to->get_name());
+        if (n->target) used.insert(n->target->get_name());
+        scan(n->rhs);
+        scan(n->predicate);
+        for (auto &l : n->lets) scan(l.second);
+    });
+}
+
+int run(const std::string &cmd) {
+    if (debug_level() >= 1) std::cout << "[tiramisu-hip] " << cmd << std::endl;
+    return std::system(cmd.c_str());
+}
+
+std::string sanitize(const std::string &s) {
+    std::string r;
+    for (char c : s) r += (isalnum((unsigned char)c) ? c : '_');
+    return r;
+}
+
+class hip_backend : public backend {
+public:
+    void generate(function &f, lir::program &prog, const std::string &obj) override {
+        context ctx;
+        ctx.f = &f;
+        ctx.prog = &prog;
+        host_gen hg(ctx);
+
+        std::set<std::string> used;
+        collect_used_buffers(prog.root, used);
+        for (auto &inv : prog.invariants)
+            inv.value.visit([&](const expr &x) {
+                if (x.get_expr_type() == e_op && x.get_op_type() == o_access) used.insert(x.get_name());
+            });
+
+        std::ostringstream body;
+        // arguments
+        const auto &args = f.get_arguments();
+        std::set<std::string> arg_names;
+        for (size_t i = 0; i < args.size(); i++) {
+            buffer *b = args[i];
+            arg_names.insert(b->get_name());
+            std::string t = primitive_c_name(b->get_elements_type());
+            if (b->get_location() == memory_location::global)
+                body << "    " << t << " *" << b->get_name() << " = (" << t << " *)(_a" << i << "->device ? (void *)_a" << i
+                     << "->device : (void *)_a" << i << "->host);\n";
+            else
+                body << "    " << t << " *" << b->get_name() << " = (" << t << " *)_a" << i << "->host;\n";
+        }
+        // function-wide constants
+        for (auto &inv : prog.invariants)
+            body << "    const " << primitive_c_name(inv.type) << " " << inv.name << " = " << hg.hp.print(inv.value) << ";\n";
+        // temporaries (reference: entry allocation / exit release, tiramisu_codegen_halide.cpp:2488-2530)
+        std::vector<std::string> releases;
+        for (auto &kv : f.get_buffers()) {
+            buffer *b = kv.second;
+            if (arg_names.count(b->get_name()) || !used.count(b->get_name())) continue;
+            std::string t = primitive_c_name(b->get_elements_type());
+            std::string bytes = "(uint64_t)(" + hg.hp.element_count(b) + ") * sizeof(" + t + ")";
+            if (b->get_location() == memory_location::global) {
+                if (b->get_auto_allocate()) {
+                    body << "    " << t << " *" << b->get_name() << " = (" << t << " *)tiramisu_hip_malloc(" << bytes << ");\n";
+                    releases.push_back("    tiramisu_hip_free((void *)" + b->get_name() + ");\n");
+                } else {
+                    body << "    " << t << " *" << b->get_name() << " = nullptr;\n";
+                }
+            } else if (b->get_location() == memory_location::host) {
+                if (b->get_auto_allocate()) {
+                    body << "    " << t << " *" << b->get_name() << " = (" << t << " *)malloc(" << bytes << ");\n";
+                    releases.push_back("    free((void *)" + b->get_name() + ");\n");
+                } else {
+                    body << "    " << t << " *" << b->get_name() << " = nullptr;\n";
+                }
+            }
+        }
+        hg.emit(prog.root, 1);
+        body << hg.out.str();
+        for (auto it = releases.rbegin(); it != releases.rend(); ++it) body << *it;
+        body << "    return 0;\n";
+
+        // ---- kernel file
+        const std::string hip_file = obj + ".hip", hsaco = obj + ".hsaco", host_file = obj + ".host.cpp";
+        if (!ctx.kernels.empty() && !std::getenv("HIP_NO_OVERWRITE")) {
+            std::ofstream k(hip_file);
+            if (!k) ERROR("cannot write " + hip_file, true);
+            k << "// Generated by the Tiramisu HIP back-end for gfx950.  Function: " << f.get_name() << "\n";
+            k << "#include <hip/hip_runtime.h>\n#include <stdint.h>\n";
+            k << ctx.includes;
+            k << c_prelude(true) << "\n";
+            for (auto &kr : ctx.kernels) k << "// " << kr.name << ": " << kr.how << "\n" << kr.source << "\n";
+        }
+        if (!ctx.kernels.empty()) {
+            const char *hipcc = std::getenv("HIPCC_PATH");
+            const char *arch = std::getenv("TIRAMISU_HIP_ARCH");
+            const char *flags = std::getenv("TIRAMISU_HIP_FLAGS");
+            std::string cmd = std::string(hipcc ? hipcc : "/opt/rocm/bin/hipcc") + " --genco --offload-arch=" +
+                              (arch ? arch : "gfx950") + " -std=c++17 " + (flags ? flags : "-O3") +
+                              " -Xclang -target-feature -Xclang -packed-fp32-ops -o " + hsaco + " " + hip_file + " 2>" + obj + ".hipcc.log";
+            if (run(cmd) != 0) {
+                std::ifstream log(obj + ".hipcc.log");
+                std::cerr << log.rdbuf();
+                ERROR("hipcc failed on " + hip_file, true);
+            }
+        }
+        // ---- host glue
+        {
+            std::ofstream h(host_file);
+            if (!h) ERROR("cannot write " + host_file, true);
+            std::string sym = "_tiramisu_hsaco_" + sanitize(f.get_name());
+            h << "// Generated by the Tiramisu HIP back-end: host glue of function " << f.get_name() << "\n";
+            h << "#include <stdint.h>\n#include <stdlib.h>\n#include <string.h>\n#include <math.h>\n";
+            h << "#include <tiramisu_hip_wrappers.h>\n";
+            h << halide_buffer_definition() << c_prelude(false) << "\n";
+            for (auto &d : hg.extern_decls) h << d << "\n";
+            if (!ctx.kernels.empty()) {
+                char *abs_path = realpath(hsaco.c_str(), nullptr);
+                const std::string hsaco_abs = abs_path ? abs_path : hsaco;
+                free(abs_path);
+                h << "__asm__(\".section .rodata\\n.balign 4096\\n.global " << sym << "\\n" << sym << ":\\n.incbin \\\"" << hsaco_abs
+                  << "\\\"\\n.global " << sym << "_end\\n" << sym << "_end:\\n.byte 0\\n.previous\\n\");\n";
+                h << "extern \"C\" const unsigned char " << sym << "[], " << sym << "_end[];\n";
+                h << "static void *_tiramisu_module() {\n    static void *m = tiramisu_hip_module_load((const void *)" << sym
+                  << ", (uint64_t)(" << sym << "_end - " << sym << "));\n    return m;\n}\n";
+            }
+            h << "extern \"C\" int " << f.get_name() << "(";
+            for (size_t i = 0; i < args.size(); i++) h << (i ? ", " : "") << "halide_buffer_t *_a" << i;
+            h << ")\n{\n" << body.str() << "}\n";
+        }
+        {
+            const char *cxx = std::getenv("TIRAMISU_HOST_CXX");
+            std::string inc = TIRAMISU_AMD_INCLUDE_DIR;
+            if (const char *e = std::getenv("TIRAMISU_AMD_INCLUDE")) inc = e;
+            std::string cmd = std::string(cxx ? cxx : "g++") + " -std=c++17 -O2 -fPIC -I" + inc + " -c " + host_file + " -o " + obj;
+            if (run(cmd) != 0) ERROR("host compiler failed on " + host_file, true);
+        }
+        for (auto &k : ctx.kernels) f.log(k.name + ": " + k.how);
+        if (debug_level() >= 1 || std::getenv("TIRAMISU_HIP_REPORT"))
+            for (auto &k : ctx.kernels) std::cout << "[tiramisu-hip] " << f.get_name() << " " << k.name << ": " << k.how << std::endl;
+    }
+};
+
+struct registrar {
+    registrar() { backend::register_backend(hardware_architecture_t::arch_amd_gpu, new hip_backend); }
+} the_registrar;
+
+}  // namespace
+}  // namespace hipgen
+}  // namespace tiramisu

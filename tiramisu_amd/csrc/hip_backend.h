@@ -1,0 +1,67 @@
+// The HIP (gfx950) back-end: shared declarations of the kernel emitters and the host-glue
+// emitter.  Replaces the reference's CUDA printer (src/tiramisu_codegen_cuda.cpp,
+// include/tiramisu/cuda_ast.h) and the GPU half of its Halide host path
+// (src/tiramisu_codegen_halide.cpp:2014-2040, :1773-1862, :2576-2607).
+#ifndef TIRAMISU_AMD_HIP_BACKEND_H
+#define TIRAMISU_AMD_HIP_BACKEND_H
+#include <set>
+#include <string>
+#include <vector>
+
+#include <tiramisu/core.h>
+
+#include "c_print.h"
+#include "lir.h"
+
+namespace tiramisu {
+namespace hipgen {
+
+struct kernel_param {
+    bool is_buffer;
+    std::string name;
+    primitive_t type;  // element type for buffers
+};
+
+/** One device kernel plus everything the host needs to launch it.  grid/block hold host-side
+  * expression texts, x first. */
+struct kernel {
+    std::string name;
+    std::string source;                 // text of the kernel (and its private helpers)
+    std::vector<kernel_param> params;   // launch order: scalars sorted by name, then buffers
+    std::string grid[3] = {"1", "1", "1"};
+    std::string block[3] = {"1", "1", "1"};
+    std::string lds_bytes = "0";
+    std::string how;                    // "generic", "mfma-contraction", "stencil", ...
+};
+
+/** A launch sequence that replaces one GPU-tagged loop nest. */
+struct launch_plan {
+    std::vector<kernel> kernels;
+    /** Host statements run instead of a plain launch of kernels[0] (empty = launch each once). */
+    std::string host_code;
+};
+
+struct context {
+    function *f = nullptr;
+    lir::program *prog = nullptr;
+    std::vector<kernel> kernels;        // all kernels of the function, in emission order
+    std::string includes;               // extra text at the top of the kernel file
+    std::set<std::string> include_once;
+    int next_kernel_id();
+};
+
+/** Schedule-faithful kernel: one thread per (block-iterator, thread-iterator) point, untagged
+  * inner loops serial in the thread (reference: tiramisu_codegen_cuda.cpp:239-326, :549-707). */
+kernel emit_generic_kernel(context &ctx, const lir::node_ptr &root);
+
+/** Pattern-directed emitters.  Each returns false when the nest is not provably of its kind, in
+  * which case the generic emitter is used. */
+bool emit_contraction(context &ctx, const lir::node_ptr &root, launch_plan &plan);
+bool emit_stencil(context &ctx, const lir::node_ptr &root, const lir::node_ptr &time_loop, launch_plan &plan);
+
+/** Text of the launch of \p k with the argument list taken from host variables of the same names. */
+std::string launch_text(const kernel &k, const std::string &indent);
+
+}  // namespace hipgen
+}  // namespace tiramisu
+#endif

@@ -1,0 +1,230 @@
+// Runtime layer between generated Tiramisu host code and HIP: the C ABI declared in
+// include/tiramisu_hip_wrappers.h.  Replaces src/tiramisu_cuda_wrappers.cpp of the reference
+// (same failure model: print and exit(1)), adds code-object loading and kernel launch so that
+// generated host code needs no HIP headers, and implements the GEMM library call with this
+// build's own MFMA kernel instead of a vendor BLAS.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <mutex>
+
+#include "../../include/tiramisu_hip_wrappers.h"
+#include "kernels/gemm_mfma.hip.h"
+
+namespace {
+
+inline void check(hipError_t e, const char *fn) {
+    if (e != hipSuccess) {
+        fprintf(stderr, "Error at %s: %s\n", fn, hipGetErrorString(e));
+        exit(1);
+    }
+}
+
+thread_local hipStream_t current_stream = hipStreamPerThread;
+
+// One thread per element of C; any strides, any sizes.  Used for double precision and for
+// shapes the MFMA path does not take.
+template <typename T>
+__global__ void gemm_generic_kernel(const T *__restrict__ A, const T *__restrict__ B, T *__restrict__ C, int M, int N,
+                                    int K, long a_rs, long a_cs, long b_rs, long b_cs, long ldc, T alpha, T beta) {
+    const int col = blockIdx.x * blockDim.x + threadIdx.x;
+    const int row = blockIdx.y * blockDim.y + threadIdx.y;
+    if (row >= M || col >= N) return;
+    T acc = 0;
+    for (int k = 0; k < K; k++) acc += A[row * a_rs + k * a_cs] * B[k * b_rs + col * b_cs];
+    T *p = C + (long)row * ldc + col;
+    *p = (beta == (T)0) ? alpha * acc : alpha * acc + beta * *p;
+}
+
+template <class CFG>
+void launch_mfma(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
+                 float alpha, float beta, bool vec_ok) {
+    const int tiles = ((M + CFG::BM - 1) / CFG::BM) * ((N + CFG::BN - 1) / CFG::BN);
+    hipLaunchKernelGGL((tgemm::sgemm_kernel<CFG>), dim3(tiles), dim3(CFG::NT), CFG::LDS_BYTES, current_stream, A, B, C,
+                       M, N, K, lda, ldb, ldc, alpha, beta, vec_ok ? 1 : 0);
+    check(hipGetLastError(), "tiramisu_hip_sgemm");
+}
+
+template <bool AK, bool BK_, bool EDGE>
+void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
+                   float alpha, float beta, bool vec_ok) {
+    // Large problems: 128x128 tiles (4 waves of 64x64).  When those would leave most of the 256
+    // compute units idle, 64x64 tiles (4 waves of 32x32).
+    const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (big_tiles >= 512)
+        launch_mfma<tgemm::config<128, 128, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+    else
+        launch_mfma<tgemm::config<64, 64, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+}
+
+template <bool AK, bool BK_>
+void dispatch_edge(bool edge, const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb,
+                   long ldc, float alpha, float beta, bool vec_ok) {
+    if (edge) dispatch_tile<AK, BK_, true>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+    else dispatch_tile<AK, BK_, false>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+}
+
+}  // namespace
+
+extern "C" {
+
+void *tiramisu_hip_malloc(uint64_t size) {
+    void *p = nullptr;
+    check(hipMalloc(&p, size), __FUNCTION__);
+    return p;
+}
+
+int tiramisu_hip_free(void *ptr) {
+    check(hipFree(ptr), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_memcpy_to_device(void *to, void *from, uint64_t size) {
+    check(hipMemcpyAsync(to, from, size, hipMemcpyHostToDevice, current_stream), __FUNCTION__);
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_memcpy_to_host(void *to, void *from, uint64_t size) {
+    check(hipMemcpyAsync(to, from, size, hipMemcpyDeviceToHost, current_stream), __FUNCTION__);
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_memcpy_device_to_device(void *to, void *from, uint64_t size) {
+    check(hipMemcpyAsync(to, from, size, hipMemcpyDeviceToDevice, current_stream), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_memcpy_to_symbol(void *to, void *from, uint64_t size) {
+    // `to` is the device address of the symbol (generated code resolves it when it loads
+    // its code object), so this is an ordinary host-to-device copy.
+    check(hipMemcpyAsync(to, from, size, hipMemcpyHostToDevice, current_stream), __FUNCTION__);
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);
+    return 0;
+}
+
+int32_t tiramisu_hip_stream_synchronize(int32_t) {
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                       uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
+                       bool transposeA, bool transposeB) {
+    if (ldA == 0) ldA = transposeA ? M : K;
+    if (ldB == 0) ldB = transposeB ? K : N;
+    if (ldC == 0) ldC = N;
+    if (M == 0 || N == 0) return 0;
+    const float *a = A + offsetA, *b = B + offsetB;
+    float *c = C + offsetC;
+    if (M > 0x7fffffffull || N > 0x7fffffffull || K > 0x7fffffffull) {
+        fprintf(stderr, "Error at %s: dimension exceeds 2^31-1\n", __FUNCTION__);
+        exit(1);
+    }
+    const int m = (int)M, n = (int)N, k = (int)K;
+    const bool vec_ok = (ldA % 4 == 0) && (ldB % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0);
+    const bool small = (m < 32 || n < 32 || k < 8);
+    if (small) {
+        dim3 blk(16, 16), grd((n + 15) / 16, (m + 15) / 16);
+        hipLaunchKernelGGL(gemm_generic_kernel<float>, grd, blk, 0, current_stream, a, b, c, m, n, k,
+                           transposeA ? 1L : (long)ldA, transposeA ? (long)ldA : 1L, transposeB ? 1L : (long)ldB,
+                           transposeB ? (long)ldB : 1L, (long)ldC, alpha, beta);
+        check(hipGetLastError(), __FUNCTION__);
+        return 0;
+    }
+    const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
+    const int bm = big_tiles >= 512 ? 128 : 64;
+    const bool edge = !(vec_ok && m % bm == 0 && n % bm == 0 && k % 16 == 0);
+    // A is K-contiguous unless transposed; B is K-contiguous only when transposed.
+    if (!transposeA && !transposeB) dispatch_edge<true, false>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
+    else if (!transposeA && transposeB) dispatch_edge<true, true>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
+    else if (transposeA && !transposeB) dispatch_edge<false, false>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
+    else dispatch_edge<false, true>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
+    return 0;
+}
+
+int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha, double beta,
+                       uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
+                       bool transposeA, bool transposeB) {
+    if (ldA == 0) ldA = transposeA ? M : K;
+    if (ldB == 0) ldB = transposeB ? K : N;
+    if (ldC == 0) ldC = N;
+    if (M == 0 || N == 0) return 0;
+    dim3 blk(16, 16), grd((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
+    hipLaunchKernelGGL(gemm_generic_kernel<double>, grd, blk, 0, current_stream, (const double *)(A + offsetA),
+                       (const double *)(B + offsetB), C + offsetC, (int)M, (int)N, (int)K,
+                       transposeA ? 1L : (long)ldA, transposeA ? (long)ldA : 1L, transposeB ? 1L : (long)ldB,
+                       transposeB ? (long)ldB : 1L, (long)ldC, alpha, beta);
+    check(hipGetLastError(), __FUNCTION__);
+    return 0;
+}
+
+void *tiramisu_hip_module_load(const void *image, uint64_t) {
+    hipModule_t m;
+    check(hipModuleLoadData(&m, image), __FUNCTION__);
+    return (void *)m;
+}
+
+void *tiramisu_hip_module_get_function(void *module, const char *kernel_name) {
+    hipFunction_t f;
+    hipError_t e = hipModuleGetFunction(&f, (hipModule_t)module, kernel_name);
+    if (e != hipSuccess) {
+        fprintf(stderr, "Error at %s: kernel %s: %s\n", __FUNCTION__, kernel_name, hipGetErrorString(e));
+        exit(1);
+    }
+    return (void *)f;
+}
+
+int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3], uint32_t dynamic_lds_bytes,
+                        void **args) {
+    if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return 0;  // empty iteration space
+    if ((uint64_t)block[0] * block[1] * block[2] > 1024) {
+        fprintf(stderr, "Error at %s: thread block %ux%ux%u exceeds 1024 threads\n", __FUNCTION__, block[0], block[1], block[2]);
+        exit(1);
+    }
+    check(hipModuleLaunchKernel((hipFunction_t)function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                dynamic_lds_bytes, current_stream, args, nullptr),
+          __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_set_stream(void *stream) {
+    current_stream = stream ? (hipStream_t)stream : hipStreamPerThread;
+    return 0;
+}
+
+void *tiramisu_hip_get_stream(void) { return (void *)current_stream; }
+
+void *tiramisu_hip_event_create(void) {
+    hipEvent_t e;
+    check(hipEventCreate(&e), __FUNCTION__);
+    return (void *)e;
+}
+
+int tiramisu_hip_event_record(void *event) {
+    check(hipEventRecord((hipEvent_t)event, current_stream), __FUNCTION__);
+    return 0;
+}
+
+float tiramisu_hip_event_elapsed_ms(void *start, void *stop) {
+    float ms = 0.f;
+    check(hipEventSynchronize((hipEvent_t)stop), __FUNCTION__);
+    check(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop), __FUNCTION__);
+    return ms;
+}
+
+int tiramisu_hip_event_destroy(void *event) {
+    check(hipEventDestroy((hipEvent_t)event), __FUNCTION__);
+    return 0;
+}
+
+int tiramisu_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+}  // extern "C"

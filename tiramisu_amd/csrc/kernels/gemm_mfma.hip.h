@@ -1,0 +1,225 @@
+// fp32 dense contraction on the gfx950 matrix cores: C[m,n] = epilogue(sum_k A[m,k] * B[k,n]).
+//
+// One workgroup of WGM x WGN wave64 wavefronts computes a BM x BN tile of C; each wavefront
+// owns (BM/WGM) x (BN/WGN) of it as 32x32 accumulator tiles of v_mfma_f32_32x32x2_f32
+// (16 accumulator registers per tile and lane).  K is walked in slices of BK through two
+// LDS stages: while the matrix cores work on one stage, the next slice travels
+// global -> registers -> other stage, with a single workgroup barrier per slice.
+//
+// LDS layouts are chosen so that neither the global loads nor the LDS accesses need a
+// transposition in registers:
+//   * an operand whose K index is contiguous in memory (row-major A, or a transposed B) is
+//     stored K-interleaved, [BK/4][X+1][4]: a 16-byte global load is a 16-byte LDS store, and a
+//     lane fetches 4 consecutive k for its row with one 16-byte LDS read (one read feeds 4 MFMA);
+//   * an operand whose M/N index is contiguous (row-major B, or a transposed A) is stored as
+//     it lies, [BK][X]: 16-byte stores, 4-byte conflict-free reads (lanes read consecutive words).
+// For one 16-byte read q, the lower half of the wave (lanes 0-31) holds k = 8q+0..3 and the
+// upper half k = 8q+4..7; MFMA step s multiplies the pairs {8q+s, 8q+4+s} -- both operands use
+// the same assignment, which is all the instruction requires.
+//
+// The block index is remapped so that the workgroups that run on one XCD (hardware deals
+// consecutive workgroup ids round-robin over the 8 XCDs) cover a compact group of C tiles and
+// share their A rows / B columns in that XCD's L2.
+#ifndef TIRAMISU_AMD_GEMM_MFMA_HIP_H
+#define TIRAMISU_AMD_GEMM_MFMA_HIP_H
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tgemm {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// One operand tile of X x BK elements (X = BM for A, BN for B).
+template <int X, int BK, int NT, bool KMAJOR, bool EDGE>
+struct operand_tile {
+    static constexpr int NV = X * BK / 4 / NT;                 // 16-byte loads per thread and slice
+    static constexpr int ROW = KMAJOR ? (X + 1) * 4 : X;        // LDS floats per k-group / per k
+    static constexpr int LDS_FLOATS = KMAJOR ? (BK / 4) * ROW : BK * ROW;
+    static_assert(X * BK / 4 % NT == 0, "tile must split evenly over the threads");
+    static_assert(BK % 8 == 0, "BK must be a multiple of 8");
+
+    // element (x, k) lives at base[x*ld + k] (KMAJOR) or base[k*ld + x]
+    static __device__ __forceinline__ void load_global(const float *__restrict__ base, long ld, int x0, int k0,
+                                                       int XE, int KE, bool vec_ok, f32x4 (&regs)[NV]) {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            const int idx = t + NT * v;
+            int x, k;
+            if (KMAJOR) { k = 4 * (idx % (BK / 4)); x = idx / (BK / 4); }
+            else        { x = 4 * (idx % (X / 4));  k = idx / (X / 4); }
+            const long off = KMAJOR ? (long)(x0 + x) * ld + (k0 + k) : (long)(k0 + k) * ld + (x0 + x);
+            if (!EDGE) {
+                regs[v] = *reinterpret_cast<const f32x4 *>(base + off);
+            } else {
+                const bool full = KMAJOR ? (x0 + x < XE && k0 + k + 3 < KE) : (k0 + k < KE && x0 + x + 3 < XE);
+                if (full && vec_ok) {
+                    regs[v] = *reinterpret_cast<const f32x4 *>(base + off);
+                } else {
+                    f32x4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int xx = KMAJOR ? x : x + e, kk = KMAJOR ? k + e : k;
+                        if (x0 + xx < XE && k0 + kk < KE)
+                            r[e] = base[KMAJOR ? (long)(x0 + xx) * ld + (k0 + kk) : (long)(k0 + kk) * ld + (x0 + xx)];
+                    }
+                    regs[v] = r;
+                }
+            }
+        }
+    }
+
+    static __device__ __forceinline__ void store_lds(float *lds, const f32x4 (&regs)[NV]) {
+        const int t = threadIdx.x;
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            const int idx = t + NT * v;
+            if (KMAJOR) {
+                const int kq = idx % (BK / 4), x = idx / (BK / 4);
+                *reinterpret_cast<f32x4 *>(lds + kq * ROW + x * 4) = regs[v];
+            } else {
+                const int xq = idx % (X / 4), k = idx / (X / 4);
+                *reinterpret_cast<f32x4 *>(lds + k * ROW + 4 * xq) = regs[v];
+            }
+        }
+    }
+
+    // Values for the 4 MFMA steps of 16-byte read q: out[s] = element (x, 8q + 4h + s).
+    static __device__ __forceinline__ f32x4 read_frag(const float *lds, int x, int q, int h) {
+        if (KMAJOR) {
+            return *reinterpret_cast<const f32x4 *>(lds + (2 * q + h) * ROW + x * 4);
+        } else {
+            const float *p = lds + (8 * q + 4 * h) * ROW + x;
+            f32x4 r = {p[0], p[ROW], p[2 * ROW], p[3 * ROW]};
+            return r;
+        }
+    }
+};
+
+// Position of the workgroup's tile: consecutive ids on one XCD walk groups of GROUP tile-rows.
+__device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tm, int &tn) {
+    const int total = tiles_m * tiles_n;
+    int id = blockIdx.x;
+    constexpr int XCDS = 8;
+    if (total % XCDS == 0) id = (id % XCDS) * (total / XCDS) + id / XCDS;
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * tiles_n;
+    const int g = id / per_group;
+    const int first_m = g * GROUP;
+    const int gsize = (tiles_m - first_m < GROUP) ? (tiles_m - first_m) : GROUP;
+    tm = first_m + (id % per_group) % gsize;
+    tn = (id % per_group) / gsize;
+}
+
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_>
+struct config {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+    static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, EDGE = EDGE_;
+    static constexpr int NT = 64 * WGM * WGN;
+    static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    typedef operand_tile<BM, BK, NT, A_KMAJOR, EDGE> opA;
+    typedef operand_tile<BN, BK, NT, B_KMAJOR, EDGE> opB;
+    static constexpr int STAGE_FLOATS = opA::LDS_FLOATS + opB::LDS_FLOATS;
+    static constexpr int LDS_BYTES = 2 * STAGE_FLOATS * 4;
+    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
+};
+
+// Accumulates the BM x BN tile at (m0, n0) into acc and hands every element to the epilogue:
+// epi(row, col, value).  A(m,k) = A[m*lda + k] if A_KMAJOR else A[k*lda + m]; B(k,n) = B[n*ldb + k]
+// if B_KMAJOR else B[k*ldb + n].  `lds` must hold config::LDS_BYTES bytes.
+template <class CFG, class EPI>
+__device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long lda, const float *__restrict__ B,
+                                              long ldb, int M, int N, int K, int m0, int n0, bool vec_ok,
+                                              float *lds, EPI epi) {
+    typedef typename CFG::opA opA;
+    typedef typename CFG::opB opB;
+    constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    f32x4 ra[opA::NV], rb[opB::NV];
+    float *sA[2] = {lds, lds + CFG::STAGE_FLOATS};
+    float *sB[2] = {lds + opA::LDS_FLOATS, lds + CFG::STAGE_FLOATS + opA::LDS_FLOATS};
+
+    const int KT = (K + BK - 1) / BK;
+    opA::load_global(A, lda, m0, 0, M, K, vec_ok, ra);
+    opB::load_global(B, ldb, n0, 0, N, K, vec_ok, rb);
+    opA::store_lds(sA[0], ra);
+    opB::store_lds(sB[0], rb);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            opA::load_global(A, lda, m0, (kt + 1) * BK, M, K, vec_ok, ra);
+            opB::load_global(B, ldb, n0, (kt + 1) * BK, N, K, vec_ok, rb);
+        }
+#pragma unroll
+        for (int q = 0; q < BK / 8; q++) {
+            f32x4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) fa[i] = opA::read_frag(sA[cur], wm * CFG::WM + i * 32 + l32, q, h);
+#pragma unroll
+            for (int j = 0; j < TN; j++) fb[j] = opB::read_frag(sB[cur], wn * CFG::WN + j * 32 + l32, q, h);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            opA::store_lds(sA[cur ^ 1], ra);
+            opB::store_lds(sB[cur ^ 1], rb);
+        }
+        __syncthreads();
+    }
+
+    // accumulator register r of a lane holds row 8*(r/4) + 4*h + r%4, column lane%32 of its tile
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * CFG::WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+                const int col = n0 + wn * CFG::WN + j * 32 + l32;
+                if (!CFG::EDGE || (row < M && col < N)) epi(row, col, acc[i][j][r]);
+            }
+}
+
+struct axpby_epilogue {
+    float *C;
+    long ldc;
+    float alpha, beta;
+    __device__ __forceinline__ void operator()(int row, int col, float v) const {
+        float *p = C + (long)row * ldc + col;
+        *p = (beta == 0.f) ? alpha * v : alpha * v + beta * *p;
+    }
+};
+
+template <class CFG>
+__global__ void __launch_bounds__(CFG::NT) sgemm_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                         float *__restrict__ C, int M, int N, int K, long lda, long ldb,
+                                                         long ldc, float alpha, float beta, int vec_ok) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    int tm, tn;
+    tile_of_block((M + CFG::BM - 1) / CFG::BM, (N + CFG::BN - 1) / CFG::BN, tm, tn);
+    axpby_epilogue epi{C, ldc, alpha, beta};
+    tile_mainloop<CFG>(A, lda, B, ldb, M, N, K, tm * CFG::BM, tn * CFG::BN, vec_ok != 0, lds, epi);
+}
+
+}  // namespace tgemm
+#endif

@@ -1,0 +1,152 @@
+"""Calling compiled Tiramisu functions from Python through their C ABI.
+
+A compiled Tiramisu function is ``extern "C" int f(halide_buffer_t *arg0, ...)``
+(reference: the generated headers, e.g. tests/wrapper_test_167.h, and the buffer layout at
+benchmarks/linear_algebra/blas/level1/dot/generated_dot.o.h:1157-1219).  This module is the
+Python counterpart of the reference's C++ wrapper programs: it describes numpy arrays (host
+memory) or raw device pointers as ``halide_buffer_t`` and calls the function with ctypes.
+It contains no compute of its own and has no CPU fallback: loading fails loudly when the
+HIP libraries were not built.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import build as _build
+
+
+class halide_dimension_t(ctypes.Structure):
+    _fields_ = [("min", ctypes.c_int32), ("extent", ctypes.c_int32), ("stride", ctypes.c_int32),
+                ("flags", ctypes.c_uint32)]
+
+
+class halide_type_t(ctypes.Structure):
+    _fields_ = [("code", ctypes.c_uint8), ("bits", ctypes.c_uint8), ("lanes", ctypes.c_uint16)]
+
+
+class halide_buffer_t(ctypes.Structure):
+    _fields_ = [("device", ctypes.c_uint64), ("device_interface", ctypes.c_void_p),
+                ("host", ctypes.c_void_p), ("flags", ctypes.c_uint64), ("type", halide_type_t),
+                ("dimensions", ctypes.c_int32), ("dim", ctypes.POINTER(halide_dimension_t)),
+                ("padding", ctypes.c_void_p)]
+
+
+_TYPE_CODES = {"i": 0, "u": 1, "f": 2, "b": 1}
+
+
+class Buffer:
+    """Owns the ``halide_buffer_t`` (and its dimension array) describing one argument.
+
+    Dimensions are stored innermost first, as Halide does: a C-contiguous numpy array of shape
+    (M, N) has dim[0] = N (stride 1) and dim[1] = M (stride N)."""
+
+    def __init__(self, shape, dtype, host_ptr=0, device_ptr=0, keepalive=None):
+        dtype = np.dtype(dtype)
+        self.keepalive = keepalive
+        nd = len(shape)
+        self.dims = (halide_dimension_t * max(nd, 1))()
+        stride = 1
+        for i, extent in enumerate(reversed(shape)):
+            self.dims[i] = halide_dimension_t(0, int(extent), stride, 0)
+            stride *= int(extent)
+        self.raw = halide_buffer_t()
+        self.raw.device = device_ptr
+        self.raw.device_interface = None
+        self.raw.host = host_ptr
+        self.raw.flags = 0
+        self.raw.type = halide_type_t(_TYPE_CODES[dtype.kind], dtype.itemsize * 8, 1)
+        self.raw.dimensions = nd
+        self.raw.dim = ctypes.cast(self.dims, ctypes.POINTER(halide_dimension_t))
+
+    @staticmethod
+    def from_numpy(a):
+        if not a.flags["C_CONTIGUOUS"]:
+            raise ValueError("Tiramisu buffers are dense row-major: pass a C-contiguous array")
+        return Buffer(a.shape, a.dtype, host_ptr=a.ctypes.data, keepalive=a)
+
+    @staticmethod
+    def from_device(ptr, shape, dtype, keepalive=None):
+        """A buffer that already lives in GPU memory (an argument tagged tag_gpu_global())."""
+        return Buffer(shape, dtype, host_ptr=0, device_ptr=int(ptr), keepalive=keepalive)
+
+    def pointer(self):
+        return ctypes.byref(self.raw)
+
+
+_wrappers = None
+
+
+def wrappers():
+    """The runtime C ABI (include/tiramisu_hip_wrappers.h), loaded with global symbol visibility
+    so that program libraries resolve against it."""
+    global _wrappers
+    if _wrappers is None:
+        path = _build.wrappers_library()
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: run __graft_entry__.build() first" % path)
+        lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+        lib.tiramisu_hip_malloc.restype = ctypes.c_void_p
+        lib.tiramisu_hip_malloc.argtypes = [ctypes.c_uint64]
+        lib.tiramisu_hip_free.argtypes = [ctypes.c_void_p]
+        for fn in (lib.tiramisu_hip_memcpy_to_device, lib.tiramisu_hip_memcpy_to_host,
+                   lib.tiramisu_hip_memcpy_device_to_device):
+            fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64]
+        lib.tiramisu_hip_stream_synchronize.argtypes = [ctypes.c_int32]
+        lib.tiramisu_hip_set_stream.argtypes = [ctypes.c_void_p]
+        lib.tiramisu_hip_get_stream.restype = ctypes.c_void_p
+        lib.tiramisu_hip_event_create.restype = ctypes.c_void_p
+        lib.tiramisu_hip_event_record.argtypes = [ctypes.c_void_p]
+        lib.tiramisu_hip_event_elapsed_ms.restype = ctypes.c_float
+        lib.tiramisu_hip_event_elapsed_ms.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        lib.tiramisu_hip_event_destroy.argtypes = [ctypes.c_void_p]
+        u64 = ctypes.c_uint64
+        lib.tiramisu_hip_sgemm.argtypes = [ctypes.c_void_p] * 3 + [u64] * 3 + [ctypes.c_float] * 2 + \
+            [u64] * 6 + [ctypes.c_bool] * 2
+        lib.tiramisu_hip_dgemm.argtypes = [ctypes.c_void_p] * 3 + [u64] * 3 + [ctypes.c_double] * 2 + \
+            [u64] * 6 + [ctypes.c_bool] * 2
+        _wrappers = lib
+    return _wrappers
+
+
+class Program:
+    """One compiled Tiramisu function: ``Program(path, "test_167")(A, B, C)`` with numpy arrays
+    and/or ``Buffer`` objects as arguments."""
+
+    def __init__(self, library_path, function_name, needs_gpu_runtime=True):
+        if not os.path.exists(library_path):
+            raise RuntimeError("%s is missing: run __graft_entry__.build() first" % library_path)
+        if needs_gpu_runtime:
+            wrappers()
+        self.lib = ctypes.CDLL(library_path)
+        self.fn = getattr(self.lib, function_name)
+        self.fn.restype = ctypes.c_int
+
+    def __call__(self, *args):
+        bufs = [a if isinstance(a, Buffer) else Buffer.from_numpy(a) for a in args]
+        rc = self.fn(*[b.pointer() for b in bufs])
+        if rc != 0:
+            raise RuntimeError("Tiramisu function returned %d" % rc)
+        return rc
+
+
+def load(directory, name, function_name=None):
+    return Program(_build.program_library(directory, name), function_name or name)
+
+
+class DeviceTimer:
+    """HIP-event timing on the stream that generated code launches on."""
+
+    def __init__(self):
+        self.w = wrappers()
+        self.start = self.w.tiramisu_hip_event_create()
+        self.stop = self.w.tiramisu_hip_event_create()
+
+    def __enter__(self):
+        self.w.tiramisu_hip_event_record(self.start)
+        return self
+
+    def __exit__(self, *exc):
+        self.w.tiramisu_hip_event_record(self.stop)
+        self.ms = self.w.tiramisu_hip_event_elapsed_ms(self.start, self.stop)
+        return False
