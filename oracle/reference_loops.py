@@ -29,3 +29,40 @@ def sgemm(A, B, C, alpha, beta):
 def transpose(A):
     """Reference: tests/wrapper_test_168.cpp:8-19."""
     return np.ascontiguousarray(A.T)
+
+
+def alloc_in_time_loop_expected(steps, px, qx):
+    """What tests/programs/alloc_in_time_loop.cpp must leave in its two buffers: every time slice
+    overwritten by its fill expression (structure of the reference's tests/wrapper_test_197.cpp:8-41,
+    which expects constant fills; here the fill depends on the indices so that a wrong index or a
+    skipped slice shows)."""
+    t = np.arange(steps)[:, None, None]
+    p0, p1 = np.arange(px)[None, :, None], np.arange(px)[None, None, :]
+    q0, q1 = np.arange(qx)[None, :, None], np.arange(qx)[None, None, :]
+    P = (7 + p0 * 100 + p1 + t).astype(np.int32)
+    Q = (-3 + q0 - q1 * 2 + t).astype(np.int32)
+    return P, Q
+
+
+def sgemm_strided(Abuf, Bbuf, Cbuf, M, N, K, alpha, beta, ldA, ldB, ldC, offA, offB, offC, tA, tB):
+    """Row-major GEMM on flat buffers with leading dimensions, element offsets and optional
+    transposition, as tiramisu_cublas_sgemm defines them (tiramisu_cuda_wrappers.cpp:74-115):
+    ld == 0 means tightly packed."""
+    if ldA == 0:
+        ldA = M if tA else K
+    if ldB == 0:
+        ldB = K if tB else N
+    if ldC == 0:
+        ldC = N
+    out = Cbuf.copy().ravel()
+    a, b = Abuf.ravel(), Bbuf.ravel()
+    for m in range(M):
+        for n in range(N):
+            acc = np.float32(0)
+            for k in range(K):
+                av = a[offA + (k * ldA + m if tA else m * ldA + k)]
+                bv = b[offB + (n * ldB + k if tB else k * ldB + n)]
+                acc = np.float32(acc + np.float32(av * bv))
+            idx = offC + m * ldC + n
+            out[idx] = np.float32(alpha) * acc + (np.float32(beta) * out[idx] if beta != 0 else np.float32(0))
+    return out.reshape(Cbuf.shape)

@@ -1,24 +1,88 @@
-"""GPU parity tests: the reference's own GPU test programs (tests/test_167.cpp ... of the
-reference tree), compiled by the HIP back-end and compared with the nested-loop references
-their wrappers use.  Inputs are small integers, as in the reference, so fp32 results are
-exact and the comparison is bit-for-bit."""
+"""GPU parity tests for the schedule-faithful (generic) emitter: programs with the features of
+the reference's own GPU tests (tests/test_162.cpp, test_164-171.cpp, test_197.cpp of the
+reference tree), compiled by the HIP back-end, called through the C ABI and compared
+
+  * with the nested-loop references the reference's wrappers use (numpy restatements), and
+  * with the CPU-generated code of the very same Tiramisu program (CPU back-end restatement).
+
+Inputs are small integers, as in the reference's wrappers, so fp32 results are exact and every
+comparison is bit-for-bit."""
+import os
+
 import numpy as np
 import pytest
 
+from oracle import build as oracle_build
 from oracle import reference_loops as ref
 from tiramisu_amd import runtime
 
 pytestmark = pytest.mark.gpu
 
 
-def _ints(rng, shape):
+def ints(rng, shape):
     return (rng.randint(0, 10, shape) - 5).astype(np.float32)
 
 
-def test_167_gemm_gpu_tile(programs_dir):
-    prog = runtime.load(programs_dir, "test_167")
+def cpu_variant(programs_dir, name):
+    return runtime.Program(oracle_build.cpu_program_library(programs_dir, name), name, needs_gpu_runtime=False)
+
+
+def test_gemm_gpu_tile(programs_dir):
     rng = np.random.RandomState(167)
-    A, B, C = _ints(rng, (128, 128)), _ints(rng, (128, 128)), _ints(rng, (128, 128))
+    A, B, C = ints(rng, (96, 64)), ints(rng, (64, 160)), ints(rng, (96, 160))
     expected = ref.gemm_accumulate(A, B, C)
-    prog(A, B, C)
+    C_cpu = C.copy()
+    cpu_variant(programs_dir, "gemm_gpu_tile")(A, B, C_cpu)
+    runtime.load(programs_dir, "gemm_gpu_tile")(A, B, C)
     assert np.array_equal(C, expected)
+    assert np.array_equal(C, C_cpu)
+
+
+def test_transpose_gpu_tile(programs_dir):
+    rng = np.random.RandomState(168)
+    A = ints(rng, (144, 80))
+    out = np.zeros((80, 144), np.float32)
+    runtime.load(programs_dir, "transpose_gpu_tile")(A, out)
+    assert np.array_equal(out, ref.transpose(A))
+
+
+def test_gemm_register_tile(programs_dir):
+    rng = np.random.RandomState(170)
+    A, B, C = ints(rng, (128, 96)), ints(rng, (96, 192)), ints(rng, (128, 192))
+    expected = ref.gemm_accumulate(A, B, C)
+    C_cpu = C.copy()
+    cpu_variant(programs_dir, "gemm_register_tile")(A, B, C_cpu)
+    runtime.load(programs_dir, "gemm_register_tile")(A, B, C)
+    assert np.array_equal(C, expected)
+    assert np.array_equal(C, C_cpu)
+
+
+def test_alloc_in_time_loop(programs_dir):
+    P = np.zeros((3, 24, 24), np.int32)
+    Q = np.zeros((3, 40, 40), np.int32)
+    runtime.load(programs_dir, "alloc_in_time_loop")(P, Q)
+    eP, eQ = ref.alloc_in_time_loop_expected(3, 24, 40)
+    assert np.array_equal(P, eP) and np.array_equal(Q, eQ)
+
+
+@pytest.mark.parametrize("M,N,K,alpha,beta,pad,off", [
+    (1, 2, 3, 1.0, 0.0, 0, 0),        # the reference's smallest case (test_162: 1x2x3)
+    (12, 20, 7, 3.0, 2.0, 0, 0),
+    (33, 40, 9, 0.0, 1.0, 3, 5),      # alpha = 0 keeps beta*C
+    (64, 96, 32, 2.0, 0.0, 4, 8),     # beta = 0 must not read C
+    (130, 70, 50, -1.0, 0.5, 1, 3),   # MFMA path with ragged edges and unaligned rows
+    (256, 256, 64, 1.0, 1.0, 0, 0),   # MFMA path, whole tiles
+])
+def test_sgemm_library_call(programs_dir, M, N, K, alpha, beta, pad, off):
+    rng = np.random.RandomState(162 + M)
+    ldA, ldB, ldC = M + pad, N + pad, N + 2 * pad
+    sizes = np.array([M, N, K, ldA, ldB, ldC, off, off + 1, off + 2], np.int32)
+    scal = np.array([alpha, beta], np.float32)
+    A = ints(rng, (K + 1, ldA))     # stored transposed: K rows
+    B = ints(rng, (K + 1, ldB))
+    C = ints(rng, (M + 1, ldC))
+    if beta == 0.0:
+        C[:] = np.nan               # reading C would poison the result
+    expected = ref.sgemm_strided(A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, off, off + 1, off + 2, True, False)
+    runtime.load(programs_dir, "sgemm_library_call")(sizes, scal, A, B, C)
+    assert np.array_equal(C, expected, equal_nan=True)

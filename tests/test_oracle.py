@@ -1,0 +1,130 @@
+"""CPU-side tests (no GPU): the CPU back-end restatement against the numpy restatements of the
+reference's wrapper loops, and the schedule algebra against brute-force enumeration."""
+import itertools
+import os
+
+import numpy as np
+import pytest
+
+from oracle import build as oracle_build
+from oracle import reference_loops as ref
+from tiramisu_amd import runtime
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROGRAMS = os.path.join(ROOT, "tests", "programs")
+
+
+def cpu_program(name, directory=PROGRAMS):
+    return runtime.Program(oracle_build.cpu_program_library(directory, name), name, needs_gpu_runtime=False)
+
+
+def ints(rng, shape):
+    return (rng.randint(0, 10, shape) - 5).astype(np.float32)
+
+
+# ---------------------------------------------------------------- oracle pins
+
+def test_gemm_restatement_closed_forms():
+    # all-ones: C = alpha*K + beta (reference: sgemm/cpu/sgemm_wrapper.cpp:166-169)
+    M, N, K = 5, 7, 9
+    A, B, C = np.ones((M, K), np.float32), np.ones((K, N), np.float32), np.ones((M, N), np.float32)
+    assert np.array_equal(ref.sgemm(A, B, C, 3.0, 2.0), np.full((M, N), 3.0 * K + 2.0, np.float32))
+    # a transposed operand or a dropped accumulation term must fail this: compare with float64 matmul
+    rng = np.random.RandomState(1)
+    A, B, C = ints(rng, (M, K)), ints(rng, (K, N)), ints(rng, (M, N))
+    assert np.array_equal(ref.gemm_accumulate(A, B, C), (C.astype(np.float64) + A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(ref.sgemm(A, B, C, 0.0, 1.0), C)
+    assert np.array_equal(ref.sgemm(A, B, C, 1.0, 0.0), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+
+
+# ---------------------------------------------------------------- CPU back-end vs restatements
+
+def test_cpu_gemm_gpu_tile():
+    rng = np.random.RandomState(167)
+    A, B, C = ints(rng, (96, 64)), ints(rng, (64, 160)), ints(rng, (96, 160))
+    expected = ref.gemm_accumulate(A, B, C)
+    cpu_program("gemm_gpu_tile")(A, B, C)
+    assert np.array_equal(C, expected)
+
+
+def test_cpu_transpose():
+    rng = np.random.RandomState(168)
+    A = ints(rng, (144, 80))
+    out = np.zeros((80, 144), np.float32)
+    cpu_program("transpose_gpu_tile")(A, out)
+    assert np.array_equal(out, ref.transpose(A))
+
+
+def test_cpu_gemm_register_tile():
+    rng = np.random.RandomState(170)
+    A, B, C = ints(rng, (128, 96)), ints(rng, (96, 192)), ints(rng, (128, 192))
+    expected = ref.gemm_accumulate(A, B, C)
+    cpu_program("gemm_register_tile")(A, B, C)
+    assert np.array_equal(C, expected)
+
+
+def test_cpu_alloc_in_time_loop():
+    P = np.zeros((3, 24, 24), np.int32)
+    Q = np.zeros((3, 40, 40), np.int32)
+    cpu_program("alloc_in_time_loop")(P, Q)
+    eP, eQ = ref.alloc_in_time_loop_expected(3, 24, 40)
+    assert np.array_equal(P, eP) and np.array_equal(Q, eQ)
+
+
+# ---------------------------------------------------------------- schedule algebra, brute force
+
+P_, Q_ = 10, 14
+
+
+def stamps(name):
+    clock = np.zeros(1, np.int32)
+    stamp = np.full((P_, Q_), -1, np.int32)
+    cpu_program(name)(clock, stamp)
+    assert clock[0] == P_ * Q_
+    return stamp
+
+
+def order_to_stamps(points):
+    out = np.full((P_, Q_), -1, np.int32)
+    for n, (i, j) in enumerate(points):
+        out[i, j] = n
+    return out
+
+
+def all_points():
+    return list(itertools.product(range(P_), range(Q_)))
+
+
+def test_order_identity():
+    assert np.array_equal(stamps("order_identity"), order_to_stamps(all_points()))
+
+
+def test_order_split():
+    pts = sorted(all_points(), key=lambda p: (p[0], p[1] // 4, p[1] % 4))
+    assert np.array_equal(stamps("order_split"), order_to_stamps(pts))
+
+
+def test_order_tile():
+    pts = sorted(all_points(), key=lambda p: (p[0] // 3, p[1] // 5, p[0] % 3, p[1] % 5))
+    assert np.array_equal(stamps("order_tile"), order_to_stamps(pts))
+
+
+def test_order_interchange():
+    pts = sorted(all_points(), key=lambda p: (p[1], p[0]))
+    assert np.array_equal(stamps("order_interchange"), order_to_stamps(pts))
+
+
+def test_order_skew_shift():
+    pts = sorted(all_points(), key=lambda p: (p[0], 2 * p[0] + p[1] + 3))
+    assert np.array_equal(stamps("order_skew_shift"), order_to_stamps(pts))
+
+
+def test_order_fuse_outer():
+    # per row: Q stamps read the clock before any tick of that row runs
+    expected = np.repeat(np.arange(P_, dtype=np.int32)[:, None] * Q_, Q_, axis=1)
+    assert np.array_equal(stamps("order_fuse_outer"), expected)
+
+
+def test_order_tags_do_not_change_results():
+    pts = sorted(all_points(), key=lambda p: (p[0], p[1] // 4, p[1] % 4))
+    assert np.array_equal(stamps("order_tags"), order_to_stamps(pts))

@@ -130,6 +130,8 @@ def build_all(force=True, verbose=False):
     build_compiler(force)
     build_wrappers(force)
     for src in program_sources():
+        if "CPU_ONLY_PROGRAM" in open(src).read():
+            continue  # needs the CPU back-end, which lives with the oracle
         if verbose:
             print("[build] program", os.path.relpath(src, ROOT), flush=True)
         build_program(src, force)

@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <cassert>
+#include <cstdlib>
 #include <queue>
 #include <sstream>
 
@@ -272,9 +273,21 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
             gen_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu);
 }
 
-void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
+void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename_in,
                        hardware_architecture_t arch) {
     if (arch == hardware_architecture_t::arch_nvidia_gpu) arch = hardware_architecture_t::arch_amd_gpu;
+    std::string obj_filename = obj_filename_in;
+    // TIRAMISU_FORCE_ARCH=cpu compiles a GPU program for the host instead (GPU-mapped loops run
+    // serially) and writes <name>_cpu.o: how the parity tests obtain CPU-generated code for the
+    // very same Tiramisu program.
+    if (const char *force = std::getenv("TIRAMISU_FORCE_ARCH")) {
+        if (std::string(force) == "cpu" && arch != hardware_architecture_t::arch_cpu) {
+            arch = hardware_architecture_t::arch_cpu;
+            size_t dot = obj_filename.rfind(".o");
+            if (dot != std::string::npos && dot + 2 == obj_filename.size()) obj_filename.insert(dot, "_cpu");
+            else obj_filename += "_cpu";
+        }
+    }
     backend *b = backend::find(arch);
     if (!b) {
         if (arch == hardware_architecture_t::arch_cpu)
