@@ -66,3 +66,45 @@ def sgemm_strided(Abuf, Bbuf, Cbuf, M, N, K, alpha, beta, ldA, ldB, ldC, offA, o
             idx = offC + m * ldC + n
             out[idx] = np.float32(alpha) * acc + (np.float32(beta) * out[idx] if beta != 0 else np.float32(0))
     return out.reshape(Cbuf.shape)
+
+
+def heat2d(grid, steps, boundary_other=None):
+    """STEPS sweeps of out = 0.2*(c + n + s + w + e) over the interior of a square grid on two
+    ping-pong planes; returns both planes as the un-tiled program leaves them (plane t % 2 holds
+    step t).  Association and rounding follow the program text in tiramisu_amd/programs/heat2d.cpp
+    -- ((((c+n)+s)+w)+e)*0.2f in fp32 -- which is the 5-point form of the reference's
+    benchmarks/halide/heat2d_tiramisu.cpp:52-86 with BASELINE's coefficients, iterated in time like
+    benchmarks/halide/heat3d_tiramisu.cpp:27-45.  `boundary_other` is the initial content of
+    plane 1 (its boundary cells are read by even steps); zeros if omitted."""
+    g = grid.astype(np.float32)
+    planes = np.zeros((2,) + g.shape, np.float32)
+    planes[0] = g
+    if boundary_other is not None:
+        planes[1] = boundary_other
+    c02 = np.float32(0.2)
+    for t in range(1, steps + 1):
+        src, dst = planes[(t - 1) % 2], planes[t % 2]
+        acc = src[1:-1, 1:-1] + src[:-2, 1:-1]
+        acc = acc + src[2:, 1:-1]
+        acc = acc + src[1:-1, :-2]
+        acc = acc + src[1:-1, 2:]
+        dst[1:-1, 1:-1] = acc * c02
+    return planes
+
+
+def heat2d_loops(grid, steps):
+    """The same sweep as plain Python loops (tiny grids only): the brute-force pin of heat2d()."""
+    n = grid.shape[0]
+    planes = np.zeros((2, n, n), np.float32)
+    planes[0] = grid
+    c02 = np.float32(0.2)
+    for t in range(1, steps + 1):
+        s, d = planes[(t - 1) % 2], planes[t % 2]
+        for y in range(1, n - 1):
+            for x in range(1, n - 1):
+                v = np.float32(s[y, x] + s[y - 1, x])
+                v = np.float32(v + s[y + 1, x])
+                v = np.float32(v + s[y, x - 1])
+                v = np.float32(v + s[y, x + 1])
+                d[y, x] = np.float32(v * c02)
+    return planes

@@ -74,31 +74,42 @@ struct generic_kernel_gen {
         });
     }
 
-    // Extent of a mapped loop as seen from the host: upper - init + 1, where a min() bound that
-    // involves in-kernel iterators contributes only its kernel-invariant arguments.
-    expr host_extent(const node_ptr &n, bool &needs_guard) {
-        if (depends_on(n->init, inner))
-            ERROR("GPU-mapped loop " + n->iterator + " has a lower bound that varies inside the kernel", true);
-        expr up = n->upper;
+    // Kernel-invariant part of a bound that is a min() (upper bounds) or max() (lower bounds) of
+    // several expressions: the arguments that do not involve in-kernel iterators.
+    expr invariant_part(const expr &bound, op_t combiner, const std::string &what) {
+        std::vector<expr> parts;
+        std::function<void(const expr &)> split = [&](const expr &e) {
+            if (e.get_expr_type() == e_op && e.get_op_type() == combiner) {
+                split(e.get_operand(0));
+                split(e.get_operand(1));
+            } else if (!depends_on(e, inner)) {
+                parts.push_back(e);
+            }
+        };
+        split(bound);
+        if (parts.empty()) ERROR("GPU-mapped loop " + what + " has no kernel-invariant bound", true);
+        expr r = parts[0];
+        for (size_t i = 1; i < parts.size(); i++) r = expr(combiner, r, parts[i]);
+        return r;
+    }
+
+    // Extent and first value of a mapped loop as seen from the host.  Bounds that vary inside the
+    // kernel (partial tiles: min()/max() with outer mapped iterators) contribute their invariant
+    // arguments to the launch size and are enforced by a guard in the kernel.  (The reference
+    // ignores lower bounds here, tiramisu_codegen_cuda.cpp:523-554.)
+    expr host_extent(const node_ptr &n, expr &first, bool &needs_guard) {
         needs_guard = false;
+        first = n->init;
+        if (depends_on(first, inner)) {
+            needs_guard = true;
+            first = invariant_part(first, o_max, n->iterator);
+        }
+        expr up = n->upper;
         if (depends_on(up, inner)) {
             needs_guard = true;
-            std::vector<expr> parts;
-            std::function<void(const expr &)> split_min = [&](const expr &e) {
-                if (e.get_expr_type() == e_op && e.get_op_type() == o_min) {
-                    split_min(e.get_operand(0));
-                    split_min(e.get_operand(1));
-                } else if (!depends_on(e, inner)) {
-                    parts.push_back(e);
-                }
-            };
-            split_min(up);
-            if (parts.empty())
-                ERROR("GPU-mapped loop " + n->iterator + " has no kernel-invariant upper bound", true);
-            up = parts[0];
-            for (size_t i = 1; i < parts.size(); i++) up = expr(o_min, up, parts[i]);
+            up = invariant_part(up, o_min, n->iterator);
         }
-        return lir::simplify(lir::simplify(up - n->init) + 1);
+        return lir::simplify(lir::simplify(up - first) + 1);
     }
 
     void emit(const node_ptr &n, int ind) {
@@ -126,14 +137,17 @@ struct generic_kernel_gen {
         if (is_block || is_thread) {
             const int dim = is_block ? n->gpu_block : n->gpu_thread;
             bool guard;
-            expr ext = host_extent(n, guard);
+            expr first;
+            expr ext = host_extent(n, first, guard);
             (is_block ? grid_ext : block_ext)[dim].push_back(ext);
             if (loops_per_dim[is_block ? 0 : 1][dim] > 1) guard = true;
             const char *idx = is_block ? "blockIdx." : "threadIdx.";
             body << pad(ind) << "{\n";
             body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)" << idx << "xyz"[dim] << " + "
-                 << dev.print(n->init) << ";\n";
-            if (guard) body << pad(ind + 1) << "if (" << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+                 << dev.print(first) << ";\n";
+            if (guard)
+                body << pad(ind + 1) << "if (" << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator
+                     << " <= " << dev.print(n->upper) << ") {\n";
             emit(n->body, ind + (guard ? 2 : 1));
             if (guard) body << pad(ind + 1) << "}\n";
             body << pad(ind) << "}\n";
