@@ -438,6 +438,64 @@ void function::gen_isl_ast() {
     if (debug_level() >= 1) std::cout << lir::dump(lowered->root) << std::endl;
 }
 
+namespace lir {
+
+node_ptr canonical_nest(function &f, computation &c) {
+    isl_ctx *ctx = f.get_isl_ctx();
+    int n = isl_set_dim(c.get_iteration_domain(), isl_dim_set);
+    std::vector<std::string> in;
+    for (int i = 0; i < n; i++) in.push_back("t" + std::to_string(i));
+    std::string ms = "{ " + c.get_name() + "[" + join(in, ",") + "] -> [" + join(in, ",") + "] }";
+    isl_map *m = isl_map_read_from_str(ctx, ms.c_str());
+    isl_set *d = isl_set_copy(c.get_iteration_domain());
+    if (f.get_program_context()) d = isl_set_intersect_params(d, isl_set_copy(f.get_program_context()));
+    m = isl_map_intersect_domain(m, d);
+    lowering lw;
+    lw.f = &f;
+    isl_ast_build *build = f.get_program_context() ? isl_ast_build_from_context(isl_set_copy(f.get_program_context()))
+                                                   : isl_ast_build_alloc(ctx);
+    build = isl_ast_build_set_at_each_domain(build, &at_each_domain, &lw);
+    isl_ast_node *ast = isl_ast_build_node_from_schedule_map(build, isl_union_map_from_map(m));
+    isl_ast_build_free(build);
+    if (!ast) return nullptr;
+    node_ptr root = convert(lw, ast);
+    isl_ast_node_free(ast);
+    return root;
+}
+
+bool mentions(const expr &e, const std::string &v) {
+    bool m = false;
+    e.visit([&](const expr &x) { if (x.get_expr_type() == e_var && x.get_name() == v) m = true; });
+    return m;
+}
+
+expr coefficient(const expr &e, const std::string &v, bool &ok) {
+    primitive_t t = global::get_loop_iterator_data_type();
+    const expr zero = value_cast(t, (int64_t)0), one = value_cast(t, (int64_t)1);
+    if (!mentions(e, v)) return zero;
+    switch (e.get_expr_type()) {
+    case e_var: return one;
+    case e_op:
+        switch (e.get_op_type()) {
+        case o_add: return simplify(coefficient(e.get_operand(0), v, ok) + coefficient(e.get_operand(1), v, ok));
+        case o_sub: return simplify(coefficient(e.get_operand(0), v, ok) - coefficient(e.get_operand(1), v, ok));
+        case o_minus: return simplify(zero - coefficient(e.get_operand(0), v, ok));
+        case o_cast: return is_int_type(e.get_data_type()) ? coefficient(e.get_operand(0), v, ok) : (ok = false, zero);
+        case o_mul: {
+            const expr &a = e.get_operand(0), &b = e.get_operand(1);
+            if (!mentions(a, v)) return simplify(cast(t, a) * coefficient(b, v, ok));
+            if (!mentions(b, v)) return simplify(coefficient(a, v, ok) * cast(t, b));
+            ok = false;
+            return zero;
+        }
+        default: ok = false; return zero;
+        }
+    default: ok = false; return zero;
+    }
+}
+
+}  // namespace lir
+
 void function::gen_c_code() const {
     char *s = isl_ast_node_to_C_str(ast);
     std::cout << s << std::endl;

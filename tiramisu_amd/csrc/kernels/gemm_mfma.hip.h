@@ -31,10 +31,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // One operand tile of X x BK elements (X = BM for A, BN for B).
-template <int X, int BK, int NT, bool KMAJOR, bool EDGE>
+template <int X, int BK, int NT, bool KMAJOR, bool EDGE, int PAD>
 struct operand_tile {
     static constexpr int NV = X * BK / 4 / NT;                 // 16-byte loads per thread and slice
-    static constexpr int ROW = KMAJOR ? (X + 1) * 4 : X;        // LDS floats per k-group / per k
+    static constexpr int ROW = KMAJOR ? (X + PAD) * 4 : X;      // LDS floats per k-group / per k
     static constexpr int LDS_FLOATS = KMAJOR ? (BK / 4) * ROW : BK * ROW;
     static_assert(X * BK / 4 % NT == 0, "tile must split evenly over the threads");
     static_assert(BK % 8 == 0, "BK must be a multiple of 8");
@@ -112,40 +112,47 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tm,
     tn = (id % per_group) / gsize;
 }
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_>
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_, int PAD_ = 1>
 struct config {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
     static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, EDGE = EDGE_;
     static constexpr int NT = 64 * WGM * WGN;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
-    typedef operand_tile<BM, BK, NT, A_KMAJOR, EDGE> opA;
-    typedef operand_tile<BN, BK, NT, B_KMAJOR, EDGE> opB;
+    typedef operand_tile<BM, BK, NT, A_KMAJOR, EDGE, PAD_> opA;
+    typedef operand_tile<BN, BK, NT, B_KMAJOR, EDGE, PAD_> opB;
     static constexpr int STAGE_FLOATS = opA::LDS_FLOATS + opB::LDS_FLOATS;
     static constexpr int LDS_BYTES = 2 * STAGE_FLOATS * 4;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
 };
 
-// Accumulates the BM x BN tile at (m0, n0) into acc and hands every element to the epilogue:
-// epi(row, col, value).  A(m,k) = A[m*lda + k] if A_KMAJOR else A[k*lda + m]; B(k,n) = B[n*ldb + k]
-// if B_KMAJOR else B[k*ldb + n].  `lds` must hold config::LDS_BYTES bytes.
-template <class CFG, class EPI>
-__device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long lda, const float *__restrict__ B,
-                                              long ldb, int M, int N, int K, int m0, int n0, bool vec_ok,
-                                              float *lds, EPI epi) {
+// Accumulator tiles of one wavefront.
+template <class CFG>
+struct accumulators {
+    f32x16 t[CFG::TM][CFG::TN];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int i = 0; i < CFG::TM; i++)
+#pragma unroll
+            for (int j = 0; j < CFG::TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) t[i][j][r] = 0.f;
+    }
+};
+
+// acc += A(m0.., :) * B(:, n0..) over K.  A(m,k) = A[m*lda + k] if A_KMAJOR else A[k*lda + m];
+// B(k,n) = B[n*ldb + k] if B_KMAJOR else B[k*ldb + n].  `lds` must hold config::LDS_BYTES bytes;
+// all threads of the workgroup must call this together (it ends with a barrier, so it may be
+// called again, e.g. for a second pair of operands feeding the same accumulators).
+template <class CFG>
+__device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const float *__restrict__ A, long lda,
+                                                const float *__restrict__ B, long ldb, int M, int N, int K, int m0,
+                                                int n0, bool vec_ok, float *lds) {
     typedef typename CFG::opA opA;
     typedef typename CFG::opB opB;
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
-
-    f32x16 acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     f32x4 ra[opA::NV], rb[opB::NV];
     float *sA[2] = {lds, lds + CFG::STAGE_FLOATS};
@@ -178,7 +185,7 @@ __device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long 
                 for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+                        acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc.t[i][j], 0, 0, 0);
         }
         if (more) {
             opA::store_lds(sA[cur ^ 1], ra);
@@ -186,18 +193,35 @@ __device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long 
         }
         __syncthreads();
     }
+}
 
+// Hands every element of the tile to the epilogue: epi(row, col, value).
+template <class CFG, class EPI>
+__device__ __forceinline__ void tile_epilogue(const accumulators<CFG> &acc, int M, int N, int m0, int n0, EPI epi) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
+    const int l32 = lane & 31, h = lane >> 5;
     // accumulator register r of a lane holds row 8*(r/4) + 4*h + r%4, column lane%32 of its tile
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < CFG::TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+        for (int j = 0; j < CFG::TN; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * CFG::WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
                 const int col = n0 + wn * CFG::WN + j * 32 + l32;
-                if (!CFG::EDGE || (row < M && col < N)) epi(row, col, acc[i][j][r]);
+                if (!CFG::EDGE || (row < M && col < N)) epi(row, col, acc.t[i][j][r]);
             }
+}
+
+template <class CFG, class EPI>
+__device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long lda, const float *__restrict__ B,
+                                              long ldb, int M, int N, int K, int m0, int n0, bool vec_ok,
+                                              float *lds, EPI epi) {
+    accumulators<CFG> acc;
+    acc.clear();
+    tile_accumulate<CFG>(acc, A, lda, B, ldb, M, N, K, m0, n0, vec_ok, lds);
+    tile_epilogue<CFG>(acc, M, N, m0, n0, epi);
 }
 
 struct axpby_epilogue {

@@ -92,6 +92,18 @@ template <typename F> void walk(const node_ptr &n, F &&f) {
 
 std::string dump(const node_ptr &n, int indent = 0);
 
+/** Lower computation \p c on its own with the identity schedule.  The result is the loop nest
+  * over the computation's iteration-domain dimensions ("c0", "c1", ... outermost first; a
+  * dimension with a single value has no loop) with one leaf whose index expressions and value
+  * are written in those iterators: the canonical, schedule-independent form that the pattern
+  * recognisers analyse. */
+node_ptr canonical_nest(function &f, computation &c);
+
+/** d e / d v for an expression that is affine in variable \p v (other symbols are constants);
+  * sets \p ok to false when e is not affine in v. */
+expr coefficient(const expr &e, const std::string &v, bool &ok);
+bool mentions(const expr &e, const std::string &v);
+
 }  // namespace lir
 }  // namespace tiramisu
 #endif

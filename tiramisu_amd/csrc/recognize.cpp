@@ -229,7 +229,459 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     return true;
 }
 
-bool emit_contraction(context &, const node_ptr &, launch_plan &) { return false; }
+// ------------------------------------------------------------------------------------------
+// Dense contraction:   acc(i, j) [= init(i, j)];   acc(i, j) += X(i, k) * Y(k, j) [+ ...];
+//                      [D(i, j) = f(acc(i, j), ...)]
+// fused in one GPU-mapped nest.  What is checked, on each computation's canonical form (its own
+// iteration-domain dimensions, independent of the schedule):
+//   * the update's value is its own element plus products of two loads, its store index does not
+//     involve the reduction dimension, the first factor of each product does not involve j and
+//     the second does not involve i -- so the only loop-carried dependence is the accumulation
+//     along k, with distance (0, 0, 1);
+//   * iteration domains are boxes; index functions are affine with unit stride along k or i
+//     (resp. k or j); the operands are not written in the nest;
+//   * an initialisation / epilogue fused into the nest touches the same (i, j) element and has
+//     no reduction dimension.
+// The nest is then replaced by an MFMA kernel (kernels/gemm_mfma.hip.h) whose epilogue is the
+// program's own initialisation + epilogue expression, evaluated once per element of the tile.
+// Floating-point sums are reassociated (pairs of k per MFMA step), which is what the 1e-4
+// relative tolerance of the parity statement is for; integer-valued data stays exact.
+namespace {
+
+struct canon_dim {
+    std::string name;   // dimension name in the computation's iteration domain
+    std::string cvar;   // "c<p>" in the canonical nest
+    expr lo, hi;        // inclusive bounds (undefined when the dimension has a single value)
+    bool in_kernel = false;
+    std::string kvar;   // name in the emitted kernel
+};
+
+struct canon {
+    computation *comp = nullptr;
+    node_ptr leaf;       // canonical leaf
+    node_ptr real;       // leaf in the scheduled program
+    std::vector<canon_dim> dims;
+    std::map<std::string, expr> subs;  // cvar -> kernel variable / parameter
+};
+
+bool canonicalize(function *f, const node_ptr &real, const std::set<std::string> &inner, canon &out) {
+    out.comp = real->comp;
+    out.real = real;
+    node_ptr n = lir::canonical_nest(*f, *real->comp);
+    const auto &names = real->comp->get_iteration_domain_dimension_names();
+    out.dims.resize(names.size());
+    for (size_t p = 0; p < names.size(); p++) {
+        out.dims[p].name = names[p];
+        out.dims[p].cvar = "c" + std::to_string(p);
+    }
+    while (n && n->kind != node_kind::leaf) {
+        if (n->kind == node_kind::loop) {
+            int p = std::atoi(n->iterator.c_str() + 1);
+            if (p < 0 || p >= (int)out.dims.size()) return false;
+            out.dims[p].lo = n->init;
+            out.dims[p].hi = n->upper;
+            if (!lir::simplify(n->increment).is_integer_literal() || lir::simplify(n->increment).get_int_val() != 1) return false;
+            n = n->body;
+        } else if (n->kind == node_kind::cond) {
+            if (n->else_body) return false;
+            n = n->then_body;
+        } else if (n->kind == node_kind::block && n->children.size() == 1) {
+            n = n->children[0];
+        } else {
+            return false;
+        }
+    }
+    if (!n) return false;
+    out.leaf = n;
+    // box: no bound mentions another dimension
+    for (auto &d : out.dims)
+        for (auto &o : out.dims)
+            if (d.lo.is_defined() && (lir::mentions(d.lo, o.cvar) || lir::mentions(d.hi, o.cvar))) return false;
+    for (auto &d : out.dims) {
+        auto it = real->iterators.find(d.name);
+        if (it == real->iterators.end()) return false;
+        for (auto &in : inner)
+            if (lir::mentions(it->second, in)) d.in_kernel = true;
+    }
+    return true;
+}
+
+void flatten_sum(const expr &e, std::vector<expr> &terms) {
+    if (e.get_expr_type() == e_op && e.get_op_type() == o_add) {
+        flatten_sum(e.get_operand(0), terms);
+        flatten_sum(e.get_operand(1), terms);
+    } else {
+        terms.push_back(e);
+    }
+}
+
+bool is_load(const expr &e) { return e.get_expr_type() == e_op && e.get_op_type() == o_access; }
+
+bool same_element(const expr &load, const buffer *b, const std::vector<expr> &idx) {
+    if (!is_load(load) || load.get_name() != b->get_name() || load.get_access().size() != idx.size()) return false;
+    for (size_t i = 0; i < idx.size(); i++)
+        if (!lir::simplify(load.get_access()[i]).is_equal(lir::simplify(idx[i]))) return false;
+    return true;
+}
+
+bool reads_buffer(const expr &e, const std::string &bn) {
+    bool r = false;
+    e.visit([&](const expr &x) { if (is_load(x) && x.get_name() == bn) r = true; });
+    return r;
+}
+
+struct gemm_operand {
+    buffer *buf = nullptr;
+    expr base, ld;
+    bool kmajor = false;
+};
+
+std::string sanitize_id(const std::string &s) {
+    std::string r;
+    for (char c : s) r += (isalnum((unsigned char)c) ? c : '_');
+    return r;
+}
+
+bool literal_value(const expr &e, long &v) {
+    expr s = lir::simplify(e);
+    if (!s.is_integer_literal()) return false;
+    v = s.get_int_val();
+    return true;
+}
+
+bool reject(int where) {
+    if (std::getenv("TIRAMISU_HIP_REPORT")) std::cout << "[tiramisu-hip] contraction check " << where << " failed" << std::endl;
+    return false;
+}
+
+}  // namespace
+
+bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
+    if (std::getenv("TIRAMISU_NO_MFMA")) return false;
+    function *f = ctx.f;
+    std::set<std::string> inner;
+    std::vector<node_ptr> leaves;
+    bool bad = false;
+    lir::walk(root, [&](const node_ptr &x) {
+        if (x->kind == node_kind::loop) inner.insert(x->iterator);
+        if (x->kind != node_kind::leaf) return;
+        if (x->lkind == leaf_kind::allocate || x->lkind == leaf_kind::release) {
+            if (x->target->get_location() == memory_location::global || x->target->get_location() == memory_location::host) bad = true;
+            return;
+        }
+        if (x->lkind != leaf_kind::assign || x->predicate.is_defined() || !x->lets.empty()) bad = true;
+        leaves.push_back(x);
+    });
+    if (bad || leaves.empty() || leaves.size() > 3) return reject(2);
+
+    // ---- find the update: own element + products of loads
+    int ui = -1;
+    std::vector<canon> cs(leaves.size());
+    for (size_t l = 0; l < leaves.size(); l++)
+        if (!canonicalize(f, leaves[l], inner, cs[l])) return reject(3);
+    std::vector<std::pair<expr, expr>> products;
+    for (size_t l = 0; l < leaves.size() && ui < 0; l++) {
+        const node_ptr &cl = cs[l].leaf;
+        if (!cl->lhs || cl->rhs.get_data_type() != p_float32) continue;
+        std::vector<expr> terms;
+        flatten_sum(cl->rhs, terms);
+        int self = 0;
+        std::vector<std::pair<expr, expr>> prods;
+        bool shape = true;
+        for (auto &t : terms) {
+            if (same_element(t, cl->lhs, cl->lhs_index)) { self++; continue; }
+            if (t.get_expr_type() == e_op && t.get_op_type() == o_mul && is_load(t.get_operand(0)) && is_load(t.get_operand(1)))
+                prods.push_back({t.get_operand(0), t.get_operand(1)});
+            else
+                shape = false;
+        }
+        if (shape && self == 1 && !prods.empty()) { ui = (int)l; products = prods; }
+    }
+    if (ui < 0) return reject(4);
+    canon &U = cs[ui];
+    const node_ptr ureal = leaves[ui];
+    const int ii = ui - 1, ei = ui + 1;   // optional initialisation before, epilogue after
+    if (ii > 0 || ei < (int)leaves.size() - 1) return reject(5);
+    const bool has_init = ii == 0, has_epi = ei == (int)leaves.size() - 1 && ei > ui;
+
+    // ---- dimensions of the update.  A spatial dimension is one that the accumulator's store
+    // index involves or, for a per-thread accumulator (whose index is constant or a tile
+    // remainder), one that the fused initialisation / epilogue also iterates: same expression
+    // of the loop iterators in the scheduled program.  The remaining in-kernel dimensions are
+    // reduction dimensions.
+    const bool private_acc = ureal->lhs->get_location() == memory_location::reg || ureal->lhs->get_location() == memory_location::local;
+    std::vector<int> spatial, reduction;
+    for (size_t p = 0; p < U.dims.size(); p++) {
+        if (!U.dims[p].in_kernel || !U.dims[p].lo.is_defined()) continue;
+        bool is_spatial = false;
+        if (!private_acc) {
+            for (auto &ix : U.leaf->lhs_index)
+                if (lir::mentions(ix, U.dims[p].cvar)) is_spatial = true;
+        } else {
+            const expr mine = lir::simplify(ureal->iterators.at(U.dims[p].name));
+            for (int other : {ii, ei}) {
+                if (other < 0 || other >= (int)leaves.size() || other == ui) continue;
+                for (auto &d : cs[other].dims)
+                    if (d.in_kernel && d.lo.is_defined() && lir::simplify(leaves[other]->iterators.at(d.name)).is_equal(mine)) is_spatial = true;
+            }
+        }
+        (is_spatial ? spatial : reduction).push_back((int)p);
+    }
+    if (spatial.size() != 2 || reduction.size() != 1) return reject(6);
+
+    // kernel names: outer dimensions become scalar parameters whose value the host computes
+    struct outer_param { std::string name; expr host_value; };
+    std::vector<outer_param> outers;
+    auto name_outer_dims = [&](canon &c) {
+        for (size_t p = 0; p < c.dims.size(); p++) {
+            canon_dim &d = c.dims[p];
+            if (d.in_kernel || !d.lo.is_defined()) continue;
+            d.kvar = "_o_" + sanitize_id(c.comp->get_name()) + "_" + std::to_string(p);
+            outers.push_back({d.kvar, c.real->iterators.at(d.name)});
+            c.subs[d.cvar] = var(d.kvar);
+        }
+    };
+    name_outer_dims(U);
+    // which spatial dimension runs along rows of the output is decided below; name them first
+    const buffer *out_buf = has_epi ? cs[ei].leaf->lhs : U.leaf->lhs;
+    if (!out_buf) return reject(7);
+    // the column dimension is the one with unit stride in the update's operands' "j" role; decide
+    // it from the second factors: the dimension no first factor mentions
+    int di = -1, dj = -1;
+    for (int cand = 0; cand < 2; cand++) {
+        const std::string &a = U.dims[spatial[cand]].cvar, &b = U.dims[spatial[1 - cand]].cvar;
+        bool okc = true;
+        for (auto &pr : products) {
+            bool x_has_b = false, y_has_a = false;
+            for (auto &ix : pr.first.get_access()) if (lir::mentions(ix, b)) x_has_b = true;
+            for (auto &ix : pr.second.get_access()) if (lir::mentions(ix, a)) y_has_a = true;
+            if (x_has_b || y_has_a) okc = false;
+        }
+        if (okc) { di = spatial[cand]; dj = spatial[1 - cand]; break; }
+    }
+    if (di < 0) {
+        // maybe the factors are written the other way round (Y * X): swap every product
+        for (auto &pr : products) std::swap(pr.first, pr.second);
+        for (int cand = 0; cand < 2; cand++) {
+            const std::string &a = U.dims[spatial[cand]].cvar, &b = U.dims[spatial[1 - cand]].cvar;
+            bool okc = true;
+            for (auto &pr : products) {
+                bool x_has_b = false, y_has_a = false;
+                for (auto &ix : pr.first.get_access()) if (lir::mentions(ix, b)) x_has_b = true;
+                for (auto &ix : pr.second.get_access()) if (lir::mentions(ix, a)) y_has_a = true;
+                if (x_has_b || y_has_a) okc = false;
+            }
+            if (okc) { di = spatial[cand]; dj = spatial[1 - cand]; break; }
+        }
+    }
+    if (di < 0) return reject(8);
+    const int dk = reduction[0];
+    U.dims[di].kvar = "_row"; U.dims[dj].kvar = "_col"; U.dims[dk].kvar = "_k";
+    U.subs[U.dims[di].cvar] = var("_row");
+    U.subs[U.dims[dj].cvar] = var("_col");
+    U.subs[U.dims[dk].cvar] = var("_k");
+
+    // initialisation / epilogue: their in-kernel dimensions must be the update's (i, j)
+    auto bind_to_update = [&](canon &c) -> bool {
+        for (size_t p = 0; p < c.dims.size(); p++) {
+            canon_dim &d = c.dims[p];
+            if (!d.lo.is_defined() || !d.in_kernel) continue;
+            const expr &mine = c.real->iterators.at(d.name);
+            int match = -1;
+            for (int sp : {di, dj})
+                if (lir::simplify(mine).is_equal(lir::simplify(ureal->iterators.at(U.dims[sp].name)))) match = sp;
+            if (match < 0) return reject(9);
+            // same extent as the update's dimension
+            if (!lir::simplify(d.lo).is_equal(lir::simplify(U.dims[match].lo)) || !lir::simplify(d.hi).is_equal(lir::simplify(U.dims[match].hi)))
+                return reject(10);
+            c.subs[d.cvar] = var(match == di ? "_row" : "_col");
+        }
+        name_outer_dims(c);
+        return true;
+    };
+    if (has_init && !bind_to_update(cs[ii])) return reject(11);
+    if (has_epi && !bind_to_update(cs[ei])) return reject(12);
+
+    // the accumulator element is the same in all fused statements (compared in the scheduled program)
+    const buffer *acc_buf = ureal->lhs;
+    if (has_init && (leaves[ii]->lhs != acc_buf || !same_element(expr(o_access, acc_buf->get_name(), leaves[ii]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
+        return reject(13);
+    if (has_init && reads_buffer(cs[ii].leaf->rhs, acc_buf->get_name())) return reject(14);
+    const bool acc_private = acc_buf->get_location() == memory_location::reg || acc_buf->get_location() == memory_location::local;
+    if (!acc_private && acc_buf->get_location() != memory_location::global) return reject(15);
+    if (!has_init && acc_private) return reject(16);   // a private accumulator must be initialised in the nest
+
+    // ---- operands
+    const expr lo_i = U.dims[di].lo, lo_j = U.dims[dj].lo, lo_k = U.dims[dk].lo;
+    std::map<std::string, expr> at_origin = U.subs;
+    at_origin[U.dims[di].cvar] = lo_i;
+    at_origin[U.dims[dj].cvar] = lo_j;
+    at_origin[U.dims[dk].cvar] = lo_k;
+    std::vector<std::pair<gemm_operand, gemm_operand>> operands;
+    std::set<std::string> written = {acc_buf->get_name(), out_buf->get_name()};
+    for (auto &pr : products) {
+        gemm_operand ops[2];
+        for (int w = 0; w < 2; w++) {
+            const expr &ld = w == 0 ? pr.first : pr.second;
+            buffer *b = f->get_buffers().at(ld.get_name());
+            if (b->get_location() != memory_location::global || b->get_elements_type() != p_float32 || written.count(b->get_name())) return reject(17);
+            expr lin = lir::linearize(b, ld.get_access());
+            bool okc = true;
+            expr cx = lir::coefficient(lin, U.dims[w == 0 ? di : dj].cvar, okc);
+            expr ck = lir::coefficient(lin, U.dims[dk].cvar, okc);
+            expr cother = lir::coefficient(lin, U.dims[w == 0 ? dj : di].cvar, okc);
+            long v;
+            if (!okc || !literal_value(cother, v) || v != 0) return reject(18);
+            cx = lir::simplify(cx.substitute(U.subs));
+            ck = lir::simplify(ck.substitute(U.subs));
+            if (literal_value(ck, v) && v == 1) { ops[w].kmajor = true; ops[w].ld = cx; }
+            else if (literal_value(cx, v) && v == 1) { ops[w].kmajor = false; ops[w].ld = ck; }
+            else return reject(19);
+            ops[w].buf = b;
+            ops[w].base = lir::simplify(lin.substitute(at_origin));
+        }
+        operands.push_back({ops[0], ops[1]});
+    }
+    for (auto &o : operands)
+        if (o.first.kmajor != operands[0].first.kmajor || o.second.kmajor != operands[0].second.kmajor) return reject(20);
+
+    // ---- sizes and tile configuration
+    const expr Me = lir::simplify(lir::simplify(U.dims[di].hi - lo_i) + 1).substitute(U.subs);
+    const expr Ne = lir::simplify(lir::simplify(U.dims[dj].hi - lo_j) + 1).substitute(U.subs);
+    const expr Ke = lir::simplify(lir::simplify(U.dims[dk].hi - lo_k) + 1).substitute(U.subs);
+    long Ml = -1, Nl = -1, Kl = -1;
+    const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
+    int BM = 64, BN = 64, BK = 16, PADX = 1;
+    if (lit) {
+        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0) { BM = BN = 256; PADX = 0; }
+        else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256) { BM = BN = 128; }
+    } else {
+        BM = BN = 64;
+    }
+    if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; }
+    bool edge = !(lit && Ml % BM == 0 && Nl % BN == 0 && Kl % BK == 0);
+    for (auto &o : operands)
+        for (const gemm_operand *g : {&o.first, &o.second}) {
+            long v;
+            if (!literal_value(g->ld, v) || v % 4 != 0) edge = true;
+            if (!literal_value(g->base, v) || v % 4 != 0) edge = true;
+        }
+
+    // ---- kernel text
+    c_printer dev;
+    dev.fct = f;
+    dev.device = true;
+    std::set<std::string> used_buffers, used_scalars;
+    dev.used_buffers = &used_buffers;
+    dev.used_scalars = &used_scalars;
+    auto replace_acc = [&](const expr &e) {
+        return e.transform([&](const expr &x) -> expr {
+            if (is_load(x) && x.get_name() == acc_buf->get_name()) return var(p_float32, "_accv");
+            return x;
+        });
+    };
+    std::ostringstream body;
+    const std::string cfg = "tgemm::config<" + std::to_string(BM) + ", " + std::to_string(BN) + ", " + std::to_string(BK) + ", 2, 2, " +
+                            (operands[0].first.kmajor ? "true" : "false") + ", " + (operands[0].second.kmajor ? "true" : "false") + ", " +
+                            (edge ? "true" : "false") + ", " + std::to_string(PADX) + ">";
+    body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
+    body << "    typedef " << cfg << " CFG;\n";
+    body << "    const int _M = " << dev.print(Me) << ", _N = " << dev.print(Ne) << ", _K = " << dev.print(Ke) << ";\n";
+    body << "    int _tm, _tn;\n    tgemm::tile_of_block((_M + CFG::BM - 1) / CFG::BM, (_N + CFG::BN - 1) / CFG::BN, _tm, _tn);\n";
+    body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
+    for (auto &o : operands) {
+        body << "    {\n        const float *_A = " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << ");\n";
+        body << "        const float *_B = " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << ");\n";
+        body << "        const long _lda = " << dev.print(o.first.ld) << ", _ldb = " << dev.print(o.second.ld) << ";\n";
+        body << "        const bool _vec = (_lda % 4 == 0) && (_ldb % 4 == 0) && ((uintptr_t)_A % 16 == 0) && ((uintptr_t)_B % 16 == 0);\n";
+        body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _lda, _B, _ldb, _M, _N, _K, _tm * CFG::BM, _tn * CFG::BN, _vec, _lds);\n    }\n";
+        used_buffers.insert(o.first.buf->get_name());
+        used_buffers.insert(o.second.buf->get_name());
+    }
+    body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, [&](int _r, int _c, float _sum) {\n";
+    body << "        const int32_t _row = _r + (" << dev.print(lo_i.substitute(U.subs)) << "), _col = _c + (" << dev.print(lo_j.substitute(U.subs)) << ");\n";
+    if (has_init) {
+        expr init = cs[ii].leaf->rhs.substitute(cs[ii].subs);
+        expr z = lir::simplify(init);
+        if (z.is_constant() && z.get_double_val() == 0.0) body << "        float _accv = _sum;\n";
+        else body << "        float _accv = " << dev.print(init) << " + _sum;\n";
+    } else {
+        body << "        float _accv = " << dev.element(acc_buf, [&] { std::vector<expr> ix; for (auto &e : U.leaf->lhs_index) ix.push_back(e.substitute(U.subs)); return ix; }())
+             << " + _sum;\n";
+    }
+    if (!acc_private) {
+        std::vector<expr> ix;
+        for (auto &e : U.leaf->lhs_index) ix.push_back(e.substitute(U.subs));
+        body << "        " << dev.store(acc_buf, ix, "_accv", p_float32) << "\n";
+    }
+    if (has_epi) {
+        canon &E = cs[ei];
+        std::vector<expr> ix;
+        for (auto &e : E.leaf->lhs_index) ix.push_back(e.substitute(E.subs));
+        expr val = replace_acc(E.leaf->rhs.substitute(E.subs));
+        body << "        " << dev.store(E.leaf->lhs, ix, dev.print(val), val.get_data_type()) << "\n";
+    }
+    body << "    });\n";
+
+    kernel k;
+    k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
+    k.how = "mfma-contraction: v_mfma_f32_32x32x2_f32, tile " + std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) +
+            (edge ? ", guarded edges" : ", whole tiles") + ", " + std::to_string(operands.size()) + " product term(s)" +
+            (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
+    static const std::set<std::string> locals = {"_row", "_col", "_k", "_accv", "_sum", "_r", "_c"};
+    std::ostringstream host;
+    host << "    {\n";
+    for (auto &nm : used_scalars) {
+        if (locals.count(nm)) continue;
+        primitive_t t = p_int32;
+        bool known = false;
+        for (auto &o : outers)
+            if (o.name == nm) known = true;
+        for (auto c : f->get_invariants())
+            if (c->get_name() == nm) { t = c->get_data_type(); known = true; }
+        if (!known) return reject(21);
+        k.params.push_back({false, nm, t});
+    }
+    {
+        c_printer hp;
+        hp.fct = f;
+        std::set<std::string> declared;
+        for (auto &o : outers)
+            if (used_scalars.count(o.name) && declared.insert(o.name).second)
+                host << "        const int32_t " << o.name << " = " << hp.print(o.host_value) << ";\n";
+        // grid: number of tiles (outer parameters are in scope here)
+        k.grid[0] = "((" + hp.print(Me) + " + " + std::to_string(BM - 1) + ") / " + std::to_string(BM) + ") * ((" + hp.print(Ne) + " + " +
+                    std::to_string(BN - 1) + ") / " + std::to_string(BN) + ")";
+    }
+    for (auto &nm : used_buffers) {
+        buffer *b = f->get_buffers().at(nm);
+        if (b->get_location() != memory_location::global) return reject(22);
+        k.params.push_back({true, nm, b->get_elements_type()});
+    }
+    k.block[0] = "256";
+    // two LDS stages of an A and a B slice
+    {
+        const int rowA = operands[0].first.kmajor ? (BK / 4) * (BM + PADX) * 4 : BK * BM;
+        const int rowB = operands[0].second.kmajor ? (BK / 4) * (BN + PADX) * 4 : BK * BN;
+        k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
+    }
+    std::ostringstream src;
+    src << "extern \"C\" __global__ void __launch_bounds__(256) " << k.name << "(";
+    for (size_t i = 0; i < k.params.size(); i++) {
+        auto &p = k.params[i];
+        src << (i ? ", " : "");
+        if (p.is_buffer) src << primitive_c_name(p.type) << " *__restrict__ " << p.name;
+        else src << "const " << primitive_c_name(p.type) << " " << p.name;
+    }
+    src << ")\n{\n" << body.str() << "}\n";
+    k.source = src.str();
+    add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma.hip.h\"");
+    host << launch_text(k, "        ") << "    }\n";
+    plan.kernels.push_back(k);
+    plan.host_code = host.str();
+    return true;
+}
+
 
 }  // namespace hipgen
 }  // namespace tiramisu
