@@ -77,6 +77,16 @@ float tiramisu_hip_event_elapsed_ms(void *start, void *stop); /* waits for `stop
 int tiramisu_hip_event_destroy(void *event);
 int tiramisu_hip_device_count(void);
 
+/* ---- per-launch timing.  Between profile_start and profile_stop every tiramisu_hip_launch
+ *      (and GEMM library call) of the calling thread is bracketed by two events on the current
+ *      stream; profile_stop waits for them and keeps one (kernel name, milliseconds) record
+ *      per launch, readable until the next profile_start.  The reference has no counterpart:
+ *      its benchmarks use nvprof (utils/run_gpu_bench.py). ---- */
+int tiramisu_hip_profile_start(void);
+int tiramisu_hip_profile_stop(void);                 /* returns the number of records */
+const char *tiramisu_hip_profile_name(int record);
+float tiramisu_hip_profile_ms(int record);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,7 +8,10 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <map>
 #include <mutex>
+#include <string>
+#include <vector>
 
 #include "../../include/tiramisu_hip_wrappers.h"
 #include "kernels/gemm_mfma.hip.h"
@@ -23,6 +26,36 @@ inline void check(hipError_t e, const char *fn) {
 }
 
 thread_local hipStream_t current_stream = hipStreamPerThread;
+
+// ---- per-launch timing records
+struct launch_record {
+    std::string name;
+    hipEvent_t start, stop;
+    float ms;
+};
+thread_local bool profiling = false;
+thread_local std::vector<launch_record> records;
+std::mutex names_mutex;
+std::map<void *, std::string> function_names;
+
+struct scoped_record {
+    bool on;
+    size_t idx = 0;
+    scoped_record(const std::string &name) : on(profiling) {
+        if (!on) return;
+        launch_record r;
+        r.name = name;
+        r.ms = 0.f;
+        check(hipEventCreate(&r.start), "tiramisu_hip_profile");
+        check(hipEventCreate(&r.stop), "tiramisu_hip_profile");
+        check(hipEventRecord(r.start, current_stream), "tiramisu_hip_profile");
+        records.push_back(r);
+        idx = records.size() - 1;
+    }
+    ~scoped_record() {
+        if (on) check(hipEventRecord(records[idx].stop, current_stream), "tiramisu_hip_profile");
+    }
+};
 
 // One thread per element of C; any strides, any sizes.  Used for double precision and for
 // shapes the MFMA path does not take.
@@ -47,13 +80,22 @@ void launch_mfma(const float *A, const float *B, float *C, int M, int N, int K, 
     check(hipGetLastError(), "tiramisu_hip_sgemm");
 }
 
+// 256x256 tiles (4 waves of 128x128) once they give every compute unit work; 128x128 tiles
+// (4 waves of 64x64) for mid sizes; 64x64 tiles when larger ones would leave most of the 256
+// compute units idle.
+int tile_for(int M, int N) {
+    if ((long)(M / 256) * (N / 256) >= 192 && M % 256 == 0 && N % 256 == 0) return 256;
+    if ((long)((M + 127) / 128) * ((N + 127) / 128) >= 256) return 128;
+    return 64;
+}
+
 template <bool AK, bool BK_, bool EDGE>
 void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
                    float alpha, float beta, bool vec_ok) {
-    // Large problems: 128x128 tiles (4 waves of 64x64).  When those would leave most of the 256
-    // compute units idle, 64x64 tiles (4 waves of 32x32).
-    const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (big_tiles >= 512)
+    const int bm = tile_for(M, N);
+    if (bm == 256)
+        launch_mfma<tgemm::config<256, 256, 16, 2, 2, AK, BK_, EDGE, 0>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+    else if (bm == 128)
         launch_mfma<tgemm::config<128, 128, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
     else
         launch_mfma<tgemm::config<64, 64, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
@@ -118,6 +160,7 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
     if (ldB == 0) ldB = transposeB ? K : N;
     if (ldC == 0) ldC = N;
     if (M == 0 || N == 0) return 0;
+    scoped_record rec("tiramisu_hip_sgemm");
     const float *a = A + offsetA, *b = B + offsetB;
     float *c = C + offsetC;
     if (M > 0x7fffffffull || N > 0x7fffffffull || K > 0x7fffffffull) {
@@ -135,8 +178,7 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
         check(hipGetLastError(), __FUNCTION__);
         return 0;
     }
-    const long big_tiles = (long)((m + 127) / 128) * ((n + 127) / 128);
-    const int bm = big_tiles >= 512 ? 128 : 64;
+    const int bm = tile_for(m, n);
     const bool edge = !(vec_ok && m % bm == 0 && n % bm == 0 && k % 16 == 0);
     // A is K-contiguous unless transposed; B is K-contiguous only when transposed.
     if (!transposeA && !transposeB) dispatch_edge<true, false>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
@@ -153,6 +195,7 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
     if (ldB == 0) ldB = transposeB ? K : N;
     if (ldC == 0) ldC = N;
     if (M == 0 || N == 0) return 0;
+    scoped_record rec("tiramisu_hip_dgemm");
     dim3 blk(16, 16), grd((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
     hipLaunchKernelGGL(gemm_generic_kernel<double>, grd, blk, 0, current_stream, (const double *)(A + offsetA),
                        (const double *)(B + offsetB), C + offsetC, (int)M, (int)N, (int)K,
@@ -175,6 +218,10 @@ void *tiramisu_hip_module_get_function(void *module, const char *kernel_name) {
         fprintf(stderr, "Error at %s: kernel %s: %s\n", __FUNCTION__, kernel_name, hipGetErrorString(e));
         exit(1);
     }
+    {
+        std::lock_guard<std::mutex> g(names_mutex);
+        function_names[(void *)f] = kernel_name;
+    }
     return (void *)f;
 }
 
@@ -185,6 +232,12 @@ int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t b
         fprintf(stderr, "Error at %s: thread block %ux%ux%u exceeds 1024 threads\n", __FUNCTION__, block[0], block[1], block[2]);
         exit(1);
     }
+    std::string nm;
+    if (profiling) {
+        std::lock_guard<std::mutex> g(names_mutex);
+        nm = function_names[function];
+    }
+    scoped_record rec(nm);
     check(hipModuleLaunchKernel((hipFunction_t)function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                 dynamic_lds_bytes, current_stream, args, nullptr),
           __FUNCTION__);
@@ -219,6 +272,33 @@ float tiramisu_hip_event_elapsed_ms(void *start, void *stop) {
 int tiramisu_hip_event_destroy(void *event) {
     check(hipEventDestroy((hipEvent_t)event), __FUNCTION__);
     return 0;
+}
+
+int tiramisu_hip_profile_start(void) {
+    for (auto &r : records) {
+        hipEventDestroy(r.start);
+        hipEventDestroy(r.stop);
+    }
+    records.clear();
+    profiling = true;
+    return 0;
+}
+
+int tiramisu_hip_profile_stop(void) {
+    profiling = false;
+    for (auto &r : records) {
+        check(hipEventSynchronize(r.stop), __FUNCTION__);
+        check(hipEventElapsedTime(&r.ms, r.start, r.stop), __FUNCTION__);
+    }
+    return (int)records.size();
+}
+
+const char *tiramisu_hip_profile_name(int record) {
+    return (record >= 0 && record < (int)records.size()) ? records[record].name.c_str() : "";
+}
+
+float tiramisu_hip_profile_ms(int record) {
+    return (record >= 0 && record < (int)records.size()) ? records[record].ms : 0.f;
 }
 
 int tiramisu_hip_device_count(void) {

@@ -100,6 +100,10 @@ def wrappers():
         lib.tiramisu_hip_event_elapsed_ms.restype = ctypes.c_float
         lib.tiramisu_hip_event_elapsed_ms.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         lib.tiramisu_hip_event_destroy.argtypes = [ctypes.c_void_p]
+        lib.tiramisu_hip_profile_name.restype = ctypes.c_char_p
+        lib.tiramisu_hip_profile_name.argtypes = [ctypes.c_int]
+        lib.tiramisu_hip_profile_ms.restype = ctypes.c_float
+        lib.tiramisu_hip_profile_ms.argtypes = [ctypes.c_int]
         u64 = ctypes.c_uint64
         lib.tiramisu_hip_sgemm.argtypes = [ctypes.c_void_p] * 3 + [u64] * 3 + [ctypes.c_float] * 2 + \
             [u64] * 6 + [ctypes.c_bool] * 2
@@ -132,6 +136,15 @@ class Program:
 
 def load(directory, name, function_name=None):
     return Program(_build.program_library(directory, name), function_name or name)
+
+
+def profile(fn):
+    """Run ``fn()`` with per-launch timing on; returns [(kernel name, milliseconds), ...]."""
+    w = wrappers()
+    w.tiramisu_hip_profile_start()
+    fn()
+    n = w.tiramisu_hip_profile_stop()
+    return [(w.tiramisu_hip_profile_name(i).decode(), float(w.tiramisu_hip_profile_ms(i))) for i in range(n)]
 
 
 class DeviceTimer:
