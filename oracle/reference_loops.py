@@ -108,3 +108,41 @@ def heat2d_loops(grid, steps):
                 v = np.float32(v + s[y, x + 1])
                 d[y, x] = np.float32(v * c02)
     return planes
+
+
+def conv2d_bias_relu(in_pad, w, bias):
+    """out[n,co,y,x] = max(0, bias[co] + sum_{ci,ky,kx} in_pad[n,ci,y+ky,x+kx] * w[co,ci,ky,kx]) on an
+    input the caller has already padded (reference: benchmarks/DNN/layers/convolution/direct/cpu/
+    conv_layer_generator_tiramisu.cpp:19-21 pads the same way; loop nest of
+    benchmarks/auto-scheduler_benchmarks/convolution/convolution_generator.cpp:17-25; ReLU of
+    benchmarks/DNN/layers/relu/cpu/relu_layer_generator_tiramisu.cpp:20).  Accumulates in float64 and
+    rounds once, so it is the exact value for integer-valued data and the reference point for
+    tolerance checks otherwise."""
+    N, CI, HP, WP = in_pad.shape
+    CO, _, KH, KW = w.shape
+    H, W = HP - KH + 1, WP - KW + 1
+    acc = np.zeros((N, CO, H, W), np.float64) + bias.astype(np.float64)[None, :, None, None]
+    for ky in range(KH):
+        for kx in range(KW):
+            win = in_pad[:, :, ky:ky + H, kx:kx + W].astype(np.float64)
+            acc += np.einsum("nchw,oc->nohw", win, w[:, :, ky, kx].astype(np.float64))
+    return np.maximum(acc, 0.0).astype(np.float32)
+
+
+def conv2d_bias_relu_loops(in_pad, w, bias):
+    """Seven nested loops in the program's order, fp32 accumulation (tiny shapes only)."""
+    N, CI, HP, WP = in_pad.shape
+    CO, _, KH, KW = w.shape
+    H, W = HP - KH + 1, WP - KW + 1
+    out = np.zeros((N, CO, H, W), np.float32)
+    for n in range(N):
+        for co in range(CO):
+            for y in range(H):
+                for x in range(W):
+                    a = np.float32(bias[co])
+                    for ci in range(CI):
+                        for ky in range(KH):
+                            for kx in range(KW):
+                                a = np.float32(a + np.float32(in_pad[n, ci, y + ky, x + kx] * w[co, ci, ky, kx]))
+                    out[n, co, y, x] = a if a > 0 else np.float32(0)
+    return out

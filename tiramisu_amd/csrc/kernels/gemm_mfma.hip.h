@@ -30,6 +30,32 @@ namespace tgemm {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
+typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));   // 4-byte aligned 16-byte load
+
+// An operand stored with one unit stride: element (x, k) lives at base[x*ld + k] (KMAJOR) or
+// base[k*ld + x].  With EDGE, elements outside XE x KE read as zero and rows need not be
+// 16-byte aligned (vec_ok false).
+template <bool KMAJOR, bool EDGE>
+struct linear_source {
+    const float *__restrict__ base;
+    long ld;
+    int XE, KE;
+    bool vec_ok;
+    __device__ __forceinline__ f32x4 load4(int x, int k) const {
+        const long off = KMAJOR ? (long)x * ld + k : (long)k * ld + x;
+        if (!EDGE) return *reinterpret_cast<const f32x4 *>(base + off);
+        const bool full = KMAJOR ? (x < XE && k + 3 < KE) : (k < KE && x + 3 < XE);
+        if (full && vec_ok) return *reinterpret_cast<const f32x4 *>(base + off);
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int xx = KMAJOR ? x : x + e, kk = KMAJOR ? k + e : k;
+            if (xx < XE && kk < KE) r[e] = base[KMAJOR ? (long)xx * ld + kk : (long)kk * ld + xx];
+        }
+        return r;
+    }
+};
+
 // One operand tile of X x BK elements (X = BM for A, BN for B).
 template <int X, int BK, int NT, bool KMAJOR, bool EDGE, int PAD>
 struct operand_tile {
@@ -39,9 +65,10 @@ struct operand_tile {
     static_assert(X * BK / 4 % NT == 0, "tile must split evenly over the threads");
     static_assert(BK % 8 == 0, "BK must be a multiple of 8");
 
-    // element (x, k) lives at base[x*ld + k] (KMAJOR) or base[k*ld + x]
-    static __device__ __forceinline__ void load_global(const float *__restrict__ base, long ld, int x0, int k0,
-                                                       int XE, int KE, bool vec_ok, f32x4 (&regs)[NV]) {
+    // SRC::load4(x, k) returns 4 consecutive elements along the operand's contiguous direction:
+    // (x, k..k+3) for a K-major operand, (x..x+3, k) otherwise.
+    template <class SRC>
+    static __device__ __forceinline__ void load_global(const SRC &src, int x0, int k0, f32x4 (&regs)[NV]) {
         const int t = threadIdx.x;
 #pragma unroll
         for (int v = 0; v < NV; v++) {
@@ -49,24 +76,7 @@ struct operand_tile {
             int x, k;
             if (KMAJOR) { k = 4 * (idx % (BK / 4)); x = idx / (BK / 4); }
             else        { x = 4 * (idx % (X / 4));  k = idx / (X / 4); }
-            const long off = KMAJOR ? (long)(x0 + x) * ld + (k0 + k) : (long)(k0 + k) * ld + (x0 + x);
-            if (!EDGE) {
-                regs[v] = *reinterpret_cast<const f32x4 *>(base + off);
-            } else {
-                const bool full = KMAJOR ? (x0 + x < XE && k0 + k + 3 < KE) : (k0 + k < KE && x0 + x + 3 < XE);
-                if (full && vec_ok) {
-                    regs[v] = *reinterpret_cast<const f32x4 *>(base + off);
-                } else {
-                    f32x4 r = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int xx = KMAJOR ? x : x + e, kk = KMAJOR ? k + e : k;
-                        if (x0 + xx < XE && k0 + kk < KE)
-                            r[e] = base[KMAJOR ? (long)(x0 + xx) * ld + (k0 + kk) : (long)(k0 + kk) * ld + (x0 + xx)];
-                    }
-                    regs[v] = r;
-                }
-            }
+            regs[v] = src.load4(x0 + x, k0 + k);
         }
     }
 
@@ -139,14 +149,14 @@ struct accumulators {
     }
 };
 
-// acc += A(m0.., :) * B(:, n0..) over K.  A(m,k) = A[m*lda + k] if A_KMAJOR else A[k*lda + m];
-// B(k,n) = B[n*ldb + k] if B_KMAJOR else B[k*ldb + n].  `lds` must hold config::LDS_BYTES bytes;
-// all threads of the workgroup must call this together (it ends with a barrier, so it may be
-// called again, e.g. for a second pair of operands feeding the same accumulators).
-template <class CFG>
-__device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const float *__restrict__ A, long lda,
-                                                const float *__restrict__ B, long ldb, int M, int N, int K, int m0,
-                                                int n0, bool vec_ok, float *lds) {
+// acc += A(m0.., :) * B(:, n0..) over K, the operands read through sources (linear_source, or
+// an emitter-generated gather such as the im2col view of a convolution input).  `lds` must hold
+// config::LDS_BYTES bytes; all threads of the workgroup must call this together (it ends with a
+// barrier, so it may be called again, e.g. for a second pair of operands feeding the same
+// accumulators).
+template <class CFG, class SRCA, class SRCB>
+__device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SRCA &A, const SRCB &B, int K, int m0,
+                                                int n0, float *lds) {
     typedef typename CFG::opA opA;
     typedef typename CFG::opB opB;
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK;
@@ -159,8 +169,8 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const fl
     float *sB[2] = {lds + opA::LDS_FLOATS, lds + CFG::STAGE_FLOATS + opA::LDS_FLOATS};
 
     const int KT = (K + BK - 1) / BK;
-    opA::load_global(A, lda, m0, 0, M, K, vec_ok, ra);
-    opB::load_global(B, ldb, n0, 0, N, K, vec_ok, rb);
+    opA::load_global(A, m0, 0, ra);
+    opB::load_global(B, n0, 0, rb);
     opA::store_lds(sA[0], ra);
     opB::store_lds(sB[0], rb);
     __syncthreads();
@@ -169,8 +179,8 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const fl
         const int cur = kt & 1;
         const bool more = kt + 1 < KT;
         if (more) {
-            opA::load_global(A, lda, m0, (kt + 1) * BK, M, K, vec_ok, ra);
-            opB::load_global(B, ldb, n0, (kt + 1) * BK, N, K, vec_ok, rb);
+            opA::load_global(A, m0, (kt + 1) * BK, ra);
+            opB::load_global(B, n0, (kt + 1) * BK, rb);
         }
 #pragma unroll
         for (int q = 0; q < BK / 8; q++) {
@@ -220,7 +230,9 @@ __device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long 
                                               float *lds, EPI epi) {
     accumulators<CFG> acc;
     acc.clear();
-    tile_accumulate<CFG>(acc, A, lda, B, ldb, M, N, K, m0, n0, vec_ok, lds);
+    linear_source<CFG::A_KMAJOR, CFG::EDGE> sa{A, lda, M, K, vec_ok};
+    linear_source<CFG::B_KMAJOR, CFG::EDGE> sb{B, ldb, N, K, vec_ok};
+    tile_accumulate<CFG>(acc, sa, sb, K, m0, n0, lds);
     tile_epilogue<CFG>(acc, M, N, m0, n0, epi);
 }
 

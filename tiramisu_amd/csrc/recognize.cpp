@@ -409,12 +409,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     // remainder), one that the fused initialisation / epilogue also iterates: same expression
     // of the loop iterators in the scheduled program.  The remaining in-kernel dimensions are
     // reduction dimensions.
-    const bool private_acc = ureal->lhs->get_location() == memory_location::reg || ureal->lhs->get_location() == memory_location::local;
+    const buffer *acc_buf = ureal->lhs;
+    const bool acc_private = acc_buf->get_location() == memory_location::reg || acc_buf->get_location() == memory_location::local;
+    if (!acc_private && acc_buf->get_location() != memory_location::global) return reject(15);
+    if (!has_init && acc_private) return reject(16);   // a private accumulator must be initialised in the nest
     std::vector<int> spatial, reduction;
     for (size_t p = 0; p < U.dims.size(); p++) {
         if (!U.dims[p].in_kernel || !U.dims[p].lo.is_defined()) continue;
         bool is_spatial = false;
-        if (!private_acc) {
+        if (!acc_private) {
             for (auto &ix : U.leaf->lhs_index)
                 if (lir::mentions(ix, U.dims[p].cvar)) is_spatial = true;
         } else {
@@ -427,9 +430,38 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         }
         (is_spatial ? spatial : reduction).push_back((int)p);
     }
-    if (spatial.size() != 2 || reduction.size() != 1) return reject(6);
+    if (spatial.size() < 2 || reduction.empty()) return reject(6);
 
-    // kernel names: outer dimensions become scalar parameters whose value the host computes
+    // ---- the GEMM view: N dimensions are the spatial dimensions of the factor that involves the
+    // innermost spatial dimension, M dimensions are the others; every product must have one
+    // factor over (M, K) and one over (K, N)
+    auto dims_of = [&](const expr &load, const std::vector<int> &among) {
+        std::set<int> r;
+        for (int p : among)
+            for (auto &ix : load.get_access())
+                if (lir::mentions(ix, U.dims[p].cvar)) r.insert(p);
+        return r;
+    };
+    const int innermost = spatial.back();
+    std::set<int> Nset;
+    for (auto &pr : products)
+        for (const expr *ld : {&pr.first, &pr.second}) {
+            std::set<int> d = dims_of(*ld, spatial);
+            if (d.count(innermost)) { if (Nset.empty()) Nset = d; else if (Nset != d) return reject(7); }
+        }
+    if (Nset.empty()) return reject(7);
+    std::vector<int> Mg, Ng, Kg = reduction;
+    for (int p : spatial) (Nset.count(p) ? Ng : Mg).push_back(p);
+    if (Mg.empty()) return reject(8);
+    for (auto &pr : products) {
+        std::set<int> dx = dims_of(pr.first, spatial), dy = dims_of(pr.second, spatial);
+        std::set<int> Mset(Mg.begin(), Mg.end());
+        if (dx == Nset && dy == Mset) std::swap(pr.first, pr.second);   // written as Y * X
+        else if (!(dx == Mset && dy == Nset)) return reject(8);
+    }
+
+    // ---- kernel names.  Outer dimensions become scalar parameters whose value the host computes;
+    // in-kernel dimensions become _d<p>, recovered from the flattened row / column / k index.
     struct outer_param { std::string name; expr host_value; };
     std::vector<outer_param> outers;
     auto name_outer_dims = [&](canon &c) {
@@ -442,129 +474,135 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         }
     };
     name_outer_dims(U);
-    // which spatial dimension runs along rows of the output is decided below; name them first
-    const buffer *out_buf = has_epi ? cs[ei].leaf->lhs : U.leaf->lhs;
-    if (!out_buf) return reject(7);
-    // the column dimension is the one with unit stride in the update's operands' "j" role; decide
-    // it from the second factors: the dimension no first factor mentions
-    int di = -1, dj = -1;
-    for (int cand = 0; cand < 2; cand++) {
-        const std::string &a = U.dims[spatial[cand]].cvar, &b = U.dims[spatial[1 - cand]].cvar;
-        bool okc = true;
-        for (auto &pr : products) {
-            bool x_has_b = false, y_has_a = false;
-            for (auto &ix : pr.first.get_access()) if (lir::mentions(ix, b)) x_has_b = true;
-            for (auto &ix : pr.second.get_access()) if (lir::mentions(ix, a)) y_has_a = true;
-            if (x_has_b || y_has_a) okc = false;
-        }
-        if (okc) { di = spatial[cand]; dj = spatial[1 - cand]; break; }
-    }
-    if (di < 0) {
-        // maybe the factors are written the other way round (Y * X): swap every product
-        for (auto &pr : products) std::swap(pr.first, pr.second);
-        for (int cand = 0; cand < 2; cand++) {
-            const std::string &a = U.dims[spatial[cand]].cvar, &b = U.dims[spatial[1 - cand]].cvar;
-            bool okc = true;
-            for (auto &pr : products) {
-                bool x_has_b = false, y_has_a = false;
-                for (auto &ix : pr.first.get_access()) if (lir::mentions(ix, b)) x_has_b = true;
-                for (auto &ix : pr.second.get_access()) if (lir::mentions(ix, a)) y_has_a = true;
-                if (x_has_b || y_has_a) okc = false;
-            }
-            if (okc) { di = spatial[cand]; dj = spatial[1 - cand]; break; }
-        }
-    }
-    if (di < 0) return reject(8);
-    const int dk = reduction[0];
-    U.dims[di].kvar = "_row"; U.dims[dj].kvar = "_col"; U.dims[dk].kvar = "_k";
-    U.subs[U.dims[di].cvar] = var("_row");
-    U.subs[U.dims[dj].cvar] = var("_col");
-    U.subs[U.dims[dk].cvar] = var("_k");
+    for (int p : spatial) { U.dims[p].kvar = "_d" + std::to_string(p); U.subs[U.dims[p].cvar] = var(U.dims[p].kvar); }
+    for (int p : reduction) { U.dims[p].kvar = "_d" + std::to_string(p); U.subs[U.dims[p].cvar] = var(U.dims[p].kvar); }
 
-    // initialisation / epilogue: their in-kernel dimensions must be the update's (i, j)
+    // initialisation / epilogue: their in-kernel dimensions must be spatial dimensions of the update
     auto bind_to_update = [&](canon &c) -> bool {
         for (size_t p = 0; p < c.dims.size(); p++) {
             canon_dim &d = c.dims[p];
             if (!d.lo.is_defined() || !d.in_kernel) continue;
-            const expr &mine = c.real->iterators.at(d.name);
+            const expr mine = lir::simplify(c.real->iterators.at(d.name));
             int match = -1;
-            for (int sp : {di, dj})
-                if (lir::simplify(mine).is_equal(lir::simplify(ureal->iterators.at(U.dims[sp].name)))) match = sp;
-            if (match < 0) return reject(9);
-            // same extent as the update's dimension
+            for (int sp : spatial)
+                if (mine.is_equal(lir::simplify(ureal->iterators.at(U.dims[sp].name)))) match = sp;
+            if (match < 0) return false;
             if (!lir::simplify(d.lo).is_equal(lir::simplify(U.dims[match].lo)) || !lir::simplify(d.hi).is_equal(lir::simplify(U.dims[match].hi)))
-                return reject(10);
-            c.subs[d.cvar] = var(match == di ? "_row" : "_col");
+                return false;
+            c.subs[d.cvar] = var(U.dims[match].kvar);
         }
         name_outer_dims(c);
         return true;
     };
     if (has_init && !bind_to_update(cs[ii])) return reject(11);
     if (has_epi && !bind_to_update(cs[ei])) return reject(12);
+    const buffer *out_buf = has_epi ? cs[ei].leaf->lhs : U.leaf->lhs;
+    if (!out_buf) return reject(7);
 
     // the accumulator element is the same in all fused statements (compared in the scheduled program)
-    const buffer *acc_buf = ureal->lhs;
     if (has_init && (leaves[ii]->lhs != acc_buf || !same_element(expr(o_access, acc_buf->get_name(), leaves[ii]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
         return reject(13);
     if (has_init && reads_buffer(cs[ii].leaf->rhs, acc_buf->get_name())) return reject(14);
-    const bool acc_private = acc_buf->get_location() == memory_location::reg || acc_buf->get_location() == memory_location::local;
-    if (!acc_private && acc_buf->get_location() != memory_location::global) return reject(15);
-    if (!has_init && acc_private) return reject(16);   // a private accumulator must be initialised in the nest
 
-    // ---- operands
-    const expr lo_i = U.dims[di].lo, lo_j = U.dims[dj].lo, lo_k = U.dims[dk].lo;
-    std::map<std::string, expr> at_origin = U.subs;
-    at_origin[U.dims[di].cvar] = lo_i;
-    at_origin[U.dims[dj].cvar] = lo_j;
-    at_origin[U.dims[dk].cvar] = lo_k;
-    std::vector<std::pair<gemm_operand, gemm_operand>> operands;
-    std::set<std::string> written = {acc_buf->get_name(), out_buf->get_name()};
-    for (auto &pr : products) {
-        gemm_operand ops[2];
-        for (int w = 0; w < 2; w++) {
-            const expr &ld = w == 0 ? pr.first : pr.second;
-            buffer *b = f->get_buffers().at(ld.get_name());
-            if (b->get_location() != memory_location::global || b->get_elements_type() != p_float32 || written.count(b->get_name())) return reject(17);
-            expr lin = lir::linearize(b, ld.get_access());
-            bool okc = true;
-            expr cx = lir::coefficient(lin, U.dims[w == 0 ? di : dj].cvar, okc);
-            expr ck = lir::coefficient(lin, U.dims[dk].cvar, okc);
-            expr cother = lir::coefficient(lin, U.dims[w == 0 ? dj : di].cvar, okc);
+    // ---- extents of the three groups
+    struct group_info { std::vector<int> dims; std::vector<expr> extent; bool literal = true; std::vector<long> ext; expr total; };
+    auto make_group = [&](const std::vector<int> &dims) {
+        group_info g;
+        g.dims = dims;
+        for (int p : dims) {
+            expr e = lir::simplify(lir::simplify(U.dims[p].hi - U.dims[p].lo) + 1).substitute(U.subs);
+            g.extent.push_back(e);
             long v;
-            if (!okc || !literal_value(cother, v) || v != 0) return reject(18);
-            cx = lir::simplify(cx.substitute(U.subs));
-            ck = lir::simplify(ck.substitute(U.subs));
-            if (literal_value(ck, v) && v == 1) { ops[w].kmajor = true; ops[w].ld = cx; }
-            else if (literal_value(cx, v) && v == 1) { ops[w].kmajor = false; ops[w].ld = ck; }
-            else return reject(19);
-            ops[w].buf = b;
-            ops[w].base = lir::simplify(lin.substitute(at_origin));
+            if (literal_value(e, v)) g.ext.push_back(v); else { g.ext.push_back(-1); g.literal = false; }
+            g.total = g.total.is_defined() ? lir::simplify(g.total * e) : e;
         }
-        operands.push_back({ops[0], ops[1]});
+        return g;
+    };
+    group_info GM = make_group(Mg), GN = make_group(Ng), GK = make_group(Kg);
+    for (const group_info *g : {&GM, &GN, &GK})
+        if (g->dims.size() > 1 && !g->literal) return reject(9);   // several dimensions flatten only with constant extents
+
+    // ---- operands: offset of element (row digits, k digits) = base + sum coef_p * (d_p - lo_p)
+    struct operand_info {
+        buffer *buf = nullptr;
+        expr base;
+        std::map<int, expr> coef;        // per in-kernel dimension
+        bool linear = false, kmajor = false;
+        expr ld;
+        bool gather_vec = false;         // gather: 4 consecutive elements are contiguous
+        bool gather_kdir = false;        // gather: vector direction is k
+    };
+    std::map<std::string, expr> at_origin = U.subs;
+    for (int p : spatial) at_origin[U.dims[p].cvar] = U.dims[p].lo;
+    for (int p : reduction) at_origin[U.dims[p].cvar] = U.dims[p].lo;
+    std::set<std::string> written = {acc_buf->get_name(), out_buf->get_name()};
+    // linear: offsets along the group are stride * flattened index
+    auto group_stride = [&](const operand_info &o, const group_info &g, expr &stride) -> bool {
+        stride = o.coef.at(g.dims.back());
+        if (g.dims.size() == 1) return true;
+        long sv;
+        if (!literal_value(stride, sv)) return false;
+        long mult = sv;
+        for (int q = (int)g.dims.size() - 1; q >= 0; q--) {
+            long cv;
+            if (!literal_value(o.coef.at(g.dims[q]), cv) || cv != mult) return false;
+            mult *= g.ext[q];
+        }
+        return true;
+    };
+    auto analyse = [&](const expr &ld, const group_info &rowg, operand_info &o) -> bool {
+        buffer *b = f->get_buffers().at(ld.get_name());
+        if (b->get_location() != memory_location::global || b->get_elements_type() != p_float32 || written.count(b->get_name())) return false;
+        o.buf = b;
+        expr lin = lir::linearize(b, ld.get_access());
+        bool okc = true;
+        for (const group_info *g : std::vector<const group_info *>{&rowg, &GK})
+            for (int p : g->dims) o.coef[p] = lir::simplify(lir::coefficient(lin, U.dims[p].cvar, okc).substitute(U.subs));
+        if (!okc) return false;
+        o.base = lir::simplify(lin.substitute(at_origin));
+        expr rs, ks;
+        long v;
+        const bool rl = group_stride(o, rowg, rs), kl = group_stride(o, GK, ks);
+        if (rl && kl && literal_value(ks, v) && v == 1) { o.linear = true; o.kmajor = true; o.ld = rs; return true; }
+        if (rl && kl && literal_value(rs, v) && v == 1) { o.linear = true; o.kmajor = false; o.ld = ks; return true; }
+        // gather: every coefficient must be a constant
+        for (auto &kv : o.coef)
+            if (!literal_value(kv.second, v)) return false;
+        if (!rowg.literal || !GK.literal) return false;
+        long cr, ck;
+        literal_value(o.coef.at(rowg.dims.back()), cr);
+        literal_value(o.coef.at(GK.dims.back()), ck);
+        if (ck == 1 && GK.ext.back() % 4 == 0) { o.gather_vec = true; o.gather_kdir = true; o.kmajor = true; }
+        else if (cr == 1 && rowg.ext.back() % 4 == 0) { o.gather_vec = true; o.gather_kdir = false; o.kmajor = false; }
+        else { o.gather_vec = false; o.kmajor = false; }
+        return true;
+    };
+    std::vector<std::pair<operand_info, operand_info>> operands;
+    for (auto &pr : products) {
+        operand_info a, b;
+        if (!analyse(pr.first, GM, a) || !analyse(pr.second, GN, b)) return reject(17);
+        operands.push_back({a, b});
     }
     for (auto &o : operands)
         if (o.first.kmajor != operands[0].first.kmajor || o.second.kmajor != operands[0].second.kmajor) return reject(20);
 
     // ---- sizes and tile configuration
-    const expr Me = lir::simplify(lir::simplify(U.dims[di].hi - lo_i) + 1).substitute(U.subs);
-    const expr Ne = lir::simplify(lir::simplify(U.dims[dj].hi - lo_j) + 1).substitute(U.subs);
-    const expr Ke = lir::simplify(lir::simplify(U.dims[dk].hi - lo_k) + 1).substitute(U.subs);
+    const expr Me = GM.total, Ne = GN.total, Ke = GK.total;
     long Ml = -1, Nl = -1, Kl = -1;
     const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
-    int BM = 64, BN = 64, BK = 16, PADX = 1;
+    int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2;
     if (lit) {
         if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0) { BM = BN = 256; PADX = 0; }
-        else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256) { BM = BN = 128; }
-    } else {
-        BM = BN = 64;
+        else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256 && Ml >= 128) { BM = BN = 128; }
+        else if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
     }
-    if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; }
+    if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
     bool edge = !(lit && Ml % BM == 0 && Nl % BN == 0 && Kl % BK == 0);
     for (auto &o : operands)
-        for (const gemm_operand *g : {&o.first, &o.second}) {
+        for (const operand_info *g : {&o.first, &o.second}) {
             long v;
-            if (!literal_value(g->ld, v) || v % 4 != 0) edge = true;
-            if (!literal_value(g->base, v) || v % 4 != 0) edge = true;
+            if (g->linear && (!literal_value(g->ld, v) || v % 4 != 0)) edge = true;
+            if (g->linear && (!literal_value(g->base, v) || v % 4 != 0)) edge = true;
         }
 
     // ---- kernel text
@@ -574,46 +612,100 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     std::set<std::string> used_buffers, used_scalars;
     dev.used_buffers = &used_buffers;
     dev.used_scalars = &used_scalars;
+    std::set<std::string> locals = {"_accv", "_sum", "_r", "_c", "_x", "_k"};
+    for (int p : spatial) locals.insert(U.dims[p].kvar);
+    for (int p : reduction) locals.insert(U.dims[p].kvar);
     auto replace_acc = [&](const expr &e) {
         return e.transform([&](const expr &x) -> expr {
             if (is_load(x) && x.get_name() == acc_buf->get_name()) return var(p_float32, "_accv");
             return x;
         });
     };
-    std::ostringstream body;
-    const std::string cfg = "tgemm::config<" + std::to_string(BM) + ", " + std::to_string(BN) + ", " + std::to_string(BK) + ", 2, 2, " +
-                            (operands[0].first.kmajor ? "true" : "false") + ", " + (operands[0].second.kmajor ? "true" : "false") + ", " +
-                            (edge ? "true" : "false") + ", " + std::to_string(PADX) + ">";
+    // digits of a flattened index: "const int32_t _d<p> = lo + (flat / later extents) % extent;"
+    auto digits = [&](const group_info &g, const std::string &flat, const std::string &ind, bool add_lo) {
+        std::ostringstream os;
+        if (g.dims.size() == 1) {
+            os << ind << "const int32_t " << U.dims[g.dims[0]].kvar << " = " << flat;
+            if (add_lo) os << " + (" << dev.print(U.dims[g.dims[0]].lo.substitute(U.subs)) << ")";
+            os << ";\n";
+            return os.str();
+        }
+        long later = 1;
+        for (int q = (int)g.dims.size() - 1; q >= 0; q--) {
+            os << ind << "const int32_t " << U.dims[g.dims[q]].kvar << " = ";
+            if (q == 0) os << "(" << flat << " / " << later << ")";
+            else os << "((" << flat << " / " << later << ") % " << g.ext[q] << ")";
+            if (add_lo) os << " + (" << dev.print(U.dims[g.dims[q]].lo.substitute(U.subs)) << ")";
+            os << ";\n";
+            later *= g.ext[q];
+        }
+        return os.str();
+    };
+    std::ostringstream pre, body;
+    const std::string cfg = "tgemm::config<" + std::to_string(BM) + ", " + std::to_string(BN) + ", " + std::to_string(BK) + ", " +
+                            std::to_string(WGM) + ", " + std::to_string(WGN) + ", " + (operands[0].first.kmajor ? "true" : "false") + ", " +
+                            (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ">";
+    const int NT = 64 * WGM * WGN;
     body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
     body << "    typedef " << cfg << " CFG;\n";
     body << "    const int _M = " << dev.print(Me) << ", _N = " << dev.print(Ne) << ", _K = " << dev.print(Ke) << ";\n";
     body << "    int _tm, _tn;\n    tgemm::tile_of_block((_M + CFG::BM - 1) / CFG::BM, (_N + CFG::BN - 1) / CFG::BN, _tm, _tn);\n";
     body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
+    int term = 0;
+    const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
     for (auto &o : operands) {
-        body << "    {\n        const float *_A = " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << ");\n";
-        body << "        const float *_B = " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << ");\n";
-        body << "        const long _lda = " << dev.print(o.first.ld) << ", _ldb = " << dev.print(o.second.ld) << ";\n";
-        body << "        const bool _vec = (_lda % 4 == 0) && (_ldb % 4 == 0) && ((uintptr_t)_A % 16 == 0) && ((uintptr_t)_B % 16 == 0);\n";
-        body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _lda, _B, _ldb, _M, _N, _K, _tm * CFG::BM, _tn * CFG::BN, _vec, _lds);\n    }\n";
-        used_buffers.insert(o.first.buf->get_name());
-        used_buffers.insert(o.second.buf->get_name());
+        body << "    {\n";
+        int which = 0;
+        for (const operand_info *g : {&o.first, &o.second}) {
+            const char *nm = which == 0 ? "_A" : "_B";
+            const group_info &rowg = which == 0 ? GM : GN;
+            used_buffers.insert(g->buf->get_name());
+            if (g->linear) {
+                body << "        const float *" << nm << "p = " << g->buf->get_name() << " + (" << dev.print(g->base) << ");\n";
+                body << "        const long " << nm << "ld = " << dev.print(g->ld) << ";\n";
+                body << "        const tgemm::linear_source<" << (g->kmajor ? "true" : "false") << ", " << (edge ? "true" : "false") << "> " << nm
+                     << "{" << nm << "p, " << nm << "ld, " << (which == 0 ? "_M" : "_N") << ", _K, (" << nm << "ld % 4 == 0) && ((uintptr_t)" << nm
+                     << "p % 16 == 0)};\n";
+            } else {
+                // gather source: offsets are separable sums over the digits of the row and k indices
+                const std::string sname = kname + "_src" + std::to_string(term) + (which == 0 ? "a" : "b");
+                pre << "struct " << sname << " {\n    const float *__restrict__ base;\n    int XE, KE;\n";
+                pre << "    __device__ __forceinline__ long offset(int _x, int _k) const {\n";
+                pre << digits(rowg, "_x", "        ", false) << digits(GK, "_k", "        ", false);
+                pre << "        return 0";
+                for (const group_info *gg : std::vector<const group_info *>{&rowg, &GK})
+                    for (int p : gg->dims) pre << " + (long)" << U.dims[p].kvar << " * " << dev.print(g->coef.at(p));
+                pre << ";\n    }\n";
+                pre << "    __device__ __forceinline__ tgemm::f32x4 load4(int x, int k) const {\n";
+                const char *full = g->gather_kdir ? "(x < XE && k + 3 < KE)" : "(k < KE && x + 3 < XE)";
+                if (g->gather_vec)
+                    pre << "        if (" << (edge ? full : "true") << ") { tgemm::f32x4_u v = *reinterpret_cast<const tgemm::f32x4_u *>(base + offset(x, k)); "
+                           "return tgemm::f32x4{v[0], v[1], v[2], v[3]}; }\n";
+                pre << "        tgemm::f32x4 r = {0.f, 0.f, 0.f, 0.f};\n";
+                pre << "        for (int e = 0; e < 4; e++) {\n            const int xx = " << (g->kmajor ? "x" : "x + e") << ", kk = " << (g->kmajor ? "k + e" : "k")
+                    << ";\n            if (xx < XE && kk < KE) r[e] = base[offset(xx, kk)];\n        }\n        return r;\n    }\n};\n";
+                body << "        const " << sname << " " << nm << "{" << g->buf->get_name() << " + (" << dev.print(g->base) << "), " << (which == 0 ? "_M" : "_N")
+                     << ", _K};\n";
+            }
+            which++;
+        }
+        body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _B, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+        term++;
     }
     body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, [&](int _r, int _c, float _sum) {\n";
-    body << "        const int32_t _row = _r + (" << dev.print(lo_i.substitute(U.subs)) << "), _col = _c + (" << dev.print(lo_j.substitute(U.subs)) << ");\n";
+    body << digits(GM, "_r", "        ", true) << digits(GN, "_c", "        ", true);
+    std::vector<expr> acc_index;
+    for (auto &e : U.leaf->lhs_index) acc_index.push_back(e.substitute(U.subs));
     if (has_init) {
         expr init = cs[ii].leaf->rhs.substitute(cs[ii].subs);
         expr z = lir::simplify(init);
         if (z.is_constant() && z.get_double_val() == 0.0) body << "        float _accv = _sum;\n";
         else body << "        float _accv = " << dev.print(init) << " + _sum;\n";
     } else {
-        body << "        float _accv = " << dev.element(acc_buf, [&] { std::vector<expr> ix; for (auto &e : U.leaf->lhs_index) ix.push_back(e.substitute(U.subs)); return ix; }())
-             << " + _sum;\n";
+        body << "        float _accv = " << dev.element(acc_buf, acc_index) << " + _sum;\n";
     }
-    if (!acc_private) {
-        std::vector<expr> ix;
-        for (auto &e : U.leaf->lhs_index) ix.push_back(e.substitute(U.subs));
-        body << "        " << dev.store(acc_buf, ix, "_accv", p_float32) << "\n";
-    }
+    if (!acc_private && !(has_epi && cs[ei].leaf->lhs == acc_buf && same_element(expr(o_access, acc_buf->get_name(), leaves[ei]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
+        body << "        " << dev.store(acc_buf, acc_index, "_accv", p_float32) << "\n";
     if (has_epi) {
         canon &E = cs[ei];
         std::vector<expr> ix;
@@ -624,11 +716,13 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     body << "    });\n";
 
     kernel k;
-    k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
-    k.how = "mfma-contraction: v_mfma_f32_32x32x2_f32, tile " + std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) +
-            (edge ? ", guarded edges" : ", whole tiles") + ", " + std::to_string(operands.size()) + " product term(s)" +
-            (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
-    static const std::set<std::string> locals = {"_row", "_col", "_k", "_accv", "_sum", "_r", "_c"};
+    k.name = kname;
+    bool any_gather = false;
+    for (auto &o : operands) any_gather = any_gather || !o.first.linear || !o.second.linear;
+    k.how = std::string("mfma-contraction: v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
+            std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
+            std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
+            std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
     std::ostringstream host;
     host << "    {\n";
     for (auto &nm : used_scalars) {
@@ -658,7 +752,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         if (b->get_location() != memory_location::global) return reject(22);
         k.params.push_back({true, nm, b->get_elements_type()});
     }
-    k.block[0] = "256";
+    k.block[0] = std::to_string(NT);
     // two LDS stages of an A and a B slice
     {
         const int rowA = operands[0].first.kmajor ? (BK / 4) * (BM + PADX) * 4 : BK * BM;
@@ -666,7 +760,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
     }
     std::ostringstream src;
-    src << "extern \"C\" __global__ void __launch_bounds__(256) " << k.name << "(";
+    src << pre.str();
+    src << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") " << k.name << "(";
     for (size_t i = 0; i < k.params.size(); i++) {
         auto &p = k.params[i];
         src << (i ? ", " : "");
@@ -681,7 +776,6 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     plan.host_code = host.str();
     return true;
 }
-
 
 }  // namespace hipgen
 }  // namespace tiramisu
