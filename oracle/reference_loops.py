@@ -146,3 +146,33 @@ def conv2d_bias_relu_loops(in_pad, w, bias):
                                 a = np.float32(a + np.float32(in_pad[n, ci, y + ky, x + kx] * w[co, ci, ky, kx]))
                     out[n, co, y, x] = a if a > 0 else np.float32(0)
     return out
+
+
+def lstm(weights, biases, x):
+    """Stacked LSTM forward pass in fp32 with numpy matrix products.
+    weights[L, 2, 4H, H] (slot 0 = input weights W, slot 1 = recurrent weights R), biases[L, 4H],
+    x[S, B, H]; gate order i, f, z, o in the 4H rows; zero initial h and c; returns y[S, B, H], the
+    hidden state of the last layer.  Restates benchmarks/DNN/blocks/LSTM/cpu/generator.cpp:31-60 with
+    the library variant's packing (gpu_lib/generator.cpp:69-70, :78-79, :84-87)."""
+    L, _, H4, H = weights.shape
+    S, B, _ = x.shape
+    f32 = np.float32
+    h_prev = np.zeros((L, B, H), f32)
+    c_prev = np.zeros((L, B, H), f32)
+    y = np.zeros((S, B, H), f32)
+    one = f32(1)
+    for m in range(S):
+        below = x[m].astype(f32)
+        for l in range(L):
+            g = biases[l][None, :] + below @ weights[l, 0].T + h_prev[l] @ weights[l, 1].T
+            g = g.astype(f32)
+            i = one / (one + np.exp(-g[:, 0:H]))
+            f = one / (one + np.exp(-g[:, H:2 * H]))
+            z = np.tanh(g[:, 2 * H:3 * H])
+            o = one / (one + np.exp(-g[:, 3 * H:4 * H]))
+            c = (i * z + f * c_prev[l]).astype(f32)
+            h = (np.tanh(c) * o).astype(f32)
+            c_prev[l], h_prev[l] = c, h
+            below = h
+        y[m] = below
+    return y

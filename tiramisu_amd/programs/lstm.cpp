@@ -1,0 +1,138 @@
+// Stacked LSTM forward pass, fp32: L layers, batch B, hidden = input = H, sequence length S.
+//   gates(m, l) = bias(l) + W(l) * h(m, l-1) + R(l) * h(m-1, l)        (4H values per sample)
+//   i, f = sigmoid(gates[0:H]), sigmoid(gates[H:2H]);  z = tanh(gates[2H:3H]);  o = sigmoid(gates[3H:4H])
+//   c(m, l) = i * z + f * c(m-1, l);   h(m, l) = tanh(c(m, l)) * o;   y(m) = h(m, L-1)
+// with h(-1, l) = c(-1, l) = 0 and h(m, -1) = x(m).  Packing follows the reference's library
+// variant: gate order i, f, z, o (benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp:84-87), weight
+// slot 0 = input weights W, slot 1 = recurrent weights R (:69-70, :78-79); the computation
+// structure (merged 4H gate rows, h/c buffers indexed [m+1][l+1]) is that of
+// benchmarks/DNN/blocks/LSTM/cpu/generator.cpp:31-60, and sigmoid is 1 / (1 + exp(-x)) (:43).
+//
+// GPU schedule: time steps and layers are host loops; per cell, the bias initialisation and the
+// two-product reduction are fused in one nest (proved a contraction -> one MFMA kernel with
+// K = 2H split over the two weight matrices), and the nine element-wise computations are fused
+// in a second nest (one kernel).  All tensors are GPU-resident.
+// CPU schedule (-DTIRAMISU_TARGET_CPU): the reference's unscheduled program
+// (cpu/generator.cpp:59-75) with the batch loop parallelized.
+// One generated function per shape: lstm_<L>x<B>x<H>x<S>.
+#include <tiramisu/tiramisu.h>
+
+using namespace tiramisu;
+
+static expr sigmoid(expr v) { return expr((float)1) / (1 + expr(o_expo, -v)); }
+
+static void generate(int L, int B, int H, int S)
+{
+    const std::string name = "lstm_" + std::to_string(L) + "x" + std::to_string(B) + "x" + std::to_string(H) + "x" + std::to_string(S);
+    tiramisu::init(name);
+
+    var l("l", 0, L), m("m", 0, S), k("k", 0, B), i("i", 0, H), j("j", 0, H), g("g", 0, 4 * H);
+
+    buffer buf_weights("buf_weights", {L, 2, 4 * H, H}, p_float32, a_input);
+    buffer buf_biases("buf_biases", {L, 4 * H}, p_float32, a_input);
+    buffer buf_x("buf_x", {S, B, H}, p_float32, a_input);
+    buffer buf_y("buf_y", {S, B, H}, p_float32, a_output);
+    buffer buf_gates("buf_gates", {B, 4 * H}, p_float32, a_temporary);
+    buffer buf_i("buf_i", {B, H}, p_float32, a_temporary);
+    buffer buf_f("buf_f", {B, H}, p_float32, a_temporary);
+    buffer buf_z("buf_z", {B, H}, p_float32, a_temporary);
+    buffer buf_o("buf_o", {B, H}, p_float32, a_temporary);
+    buffer buf_h("buf_h", {S + 1, L + 1, B, H}, p_float32, a_temporary);
+    buffer buf_c("buf_c", {S + 1, L, B, H}, p_float32, a_temporary);
+
+    input W("W", {l, g, j}, p_float32);
+    input R("R", {l, g, j}, p_float32);
+    input bias("bias", {l, g}, p_float32);
+    input x("x", {m, k, i}, p_float32);
+
+    computation h("h", {m, l, k, i}, p_float32);
+    computation c("c", {m, l, k, i}, p_float32);
+    computation h_init("h_init", {l, k, i}, expr((float)0));
+    computation c_init("c_init", {l, k, i}, expr((float)0));
+    computation h_copy_x("h_copy_x", {m, k, i}, x(m, k, i));
+    computation gates_init("gates_init", {m, l, k, g}, bias(l, g));
+    computation gates("gates", {m, l, k, g, j}, p_float32);
+    gates.set_expression(gates(m, l, k, g, 0) + W(l, g, j) * h(m, l - 1, k, j) + R(l, g, j) * h(m - 1, l, k, j));
+    computation sig_i("sig_i", {m, l, k, i}, sigmoid(gates(m, l, k, i, 0)));
+    computation sig_f("sig_f", {m, l, k, i}, sigmoid(gates(m, l, k, i + H, 0)));
+    computation tnh_z("tnh_z", {m, l, k, i}, expr(o_tanh, gates(m, l, k, i + 2 * H, 0)));
+    computation sig_o("sig_o", {m, l, k, i}, sigmoid(gates(m, l, k, i + 3 * H, 0)));
+    computation mul_iz("mul_iz", {m, l, k, i}, sig_i(m, l, k, i) * tnh_z(m, l, k, i));
+    computation mul_fc("mul_fc", {m, l, k, i}, sig_f(m, l, k, i) * c(m - 1, l, k, i));
+    c.set_expression(mul_iz(m, l, k, i) + mul_fc(m, l, k, i));
+    computation tnh_c("tnh_c", {m, l, k, i}, expr(o_tanh, c(m, l, k, i)));
+    h.set_expression(tnh_c(m, l, k, i) * sig_o(m, l, k, i));
+    computation y("y", {m, k, i}, h(m, L - 1, k, i));
+
+    W.store_in(&buf_weights, {l, 0, g, j});
+    R.store_in(&buf_weights, {l, 1, g, j});
+    bias.store_in(&buf_biases, {l, g});
+    x.store_in(&buf_x);
+    y.store_in(&buf_y);
+    gates_init.store_in(&buf_gates, {k, g});
+    gates.store_in(&buf_gates, {k, g});
+    sig_i.store_in(&buf_i, {k, i});
+    sig_f.store_in(&buf_f, {k, i});
+    tnh_z.store_in(&buf_z, {k, i});
+    sig_o.store_in(&buf_o, {k, i});
+    mul_iz.store_in(&buf_i, {k, i});
+    mul_fc.store_in(&buf_f, {k, i});
+    tnh_c.store_in(&buf_i, {k, i});
+    h.store_in(&buf_h, {m + 1, l + 1, k, i});
+    c.store_in(&buf_c, {m + 1, l, k, i});
+    h_init.store_in(&buf_h, {0, l + 1, k, i});
+    c_init.store_in(&buf_c, {0, l, k, i});
+    h_copy_x.store_in(&buf_h, {m + 1, 0, k, i});
+
+#ifdef TIRAMISU_TARGET_CPU
+    for (computation *q : {&gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
+        q->parallelize(k);
+    h_init.then(c_init, computation::root)
+          .then(h_copy_x, computation::root)
+          .then(gates_init, computation::root)
+          .then(gates, l)
+          .then(sig_i, l)
+          .then(sig_f, l)
+          .then(tnh_z, l)
+          .then(sig_o, l)
+          .then(mul_iz, l)
+          .then(mul_fc, l)
+          .then(c, l)
+          .then(tnh_c, l)
+          .then(h, l)
+          .then(y, computation::root);
+    tiramisu::codegen({&buf_weights, &buf_biases, &buf_x, &buf_y}, "build/" + name + "_cpu.o", false);
+#else
+    for (buffer *q : {&buf_weights, &buf_biases, &buf_x, &buf_y, &buf_gates, &buf_i, &buf_f, &buf_z, &buf_o, &buf_h, &buf_c})
+        q->tag_gpu_global();
+    var kb("kb"), kt("kt"), ib("ib"), it("it"), gb("gb"), gt("gt");
+    for (computation *q : {&h_init, &c_init, &h_copy_x, &y, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
+        q->gpu_tile(k, i, 16, 16, kb, ib, kt, it);
+    gates_init.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
+    gates.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
+    h_init.then(c_init, computation::root)
+          .then(h_copy_x, computation::root)
+          .then(gates_init, computation::root)
+          .then(gates, gt)
+          .then(sig_i, l)
+          .then(sig_f, it)
+          .then(tnh_z, it)
+          .then(sig_o, it)
+          .then(mul_iz, it)
+          .then(mul_fc, it)
+          .then(c, it)
+          .then(tnh_c, it)
+          .then(h, it)
+          .then(y, computation::root);
+    tiramisu::codegen({&buf_weights, &buf_biases, &buf_x, &buf_y}, "build/" + name + ".o", true);
+#endif
+}
+
+int main()
+{
+    generate(4, 64, 512, 100);   // benchmark configuration 5
+    generate(2, 8, 32, 5);
+    generate(1, 4, 16, 3);
+    generate(3, 20, 64, 4);
+    return 0;
+}
