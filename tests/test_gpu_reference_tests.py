@@ -86,3 +86,26 @@ def test_sgemm_library_call(programs_dir, M, N, K, alpha, beta, pad, off):
     expected = ref.sgemm_strided(A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, off, off + 1, off + 2, True, False)
     runtime.load(programs_dir, "sgemm_library_call")(sizes, scal, A, B, C)
     assert np.array_equal(C, expected, equal_nan=True)
+
+
+def test_sgemm_cache_shared_register_tile(programs_dir):
+    # generator3-style staged sgemm: LDS tiles via cache_shared, 4x2 register tile, alpha/beta
+    rng = np.random.RandomState(3)
+    M, N, K = 256, 192, 64
+    A, B, C = ints(rng, (M, K)), ints(rng, (K, N)), ints(rng, (M, N))
+    scal = np.array([3.0, 2.0], np.float32)
+    expected = ref.sgemm(A, B, C, 3.0, 2.0)
+    runtime.load(programs_dir, "sgemm_shared_regs")(scal, A, B, C)
+    assert np.array_equal(C, expected)
+
+
+def test_gemm_uint8_cache_shared(programs_dir):
+    # uint8 arithmetic wraps modulo 256 (reference: tutorials/developers/tutorial_04gpu2 wrapper)
+    rng = np.random.RandomState(4)
+    S = 128
+    A = rng.randint(0, 256, (S, S)).astype(np.uint8)
+    B = rng.randint(0, 256, (S, S)).astype(np.uint8)
+    C = rng.randint(0, 256, (S, S)).astype(np.uint8)
+    expected = ((C.astype(np.int64) + A.astype(np.int64) @ B.astype(np.int64)) % 256).astype(np.uint8)
+    runtime.load(programs_dir, "gemm_u8_shared")(A, B, C)
+    assert np.array_equal(C, expected)

@@ -977,6 +977,142 @@ void computation::gpu_tile(var L0, var L1, var L2, int sizeX, int sizeY, int siz
     gpu_tile(L0, L1, L2, sizeX, sizeY, sizeZ, g(L0, "_b"), g(L1, "_b"), g(L2, "_b"), g(L0, "_t"), g(L1, "_t"), g(L2, "_t"));
 }
 
+// ------------------------------------------------------------------ cache_shared
+
+// The loop-level space of this computation restricted to its first `keep` levels, as an isl set
+// string with the level names as dimension names and `tuple` as its name.
+static std::string level_space(computation &c, int keep, const std::string &tuple) {
+    isl_set *ts = isl_set_apply(isl_set_copy(c.get_iteration_domain()), isl_map_copy(c.get_schedule()));
+    int n = (int)c.get_loop_level_names().size();
+    // range is [dup, s0, d0, s1, ..., d(n-1), sn]: drop everything but d0..d(keep-1)
+    for (int pos = 2 * n + 1; pos >= 0; pos--) {
+        bool dynamic = pos >= 2 && pos % 2 == 0;
+        int level = (pos - 2) / 2;
+        if (!dynamic || level >= keep) ts = isl_set_project_out(ts, isl_dim_set, pos, 1);
+    }
+    for (int l = 0; l < keep; l++) ts = isl_set_set_dim_name(ts, isl_dim_set, l, c.get_loop_level_names()[l].c_str());
+    ts = isl_set_set_tuple_name(ts, tuple.c_str());
+    ts = isl_set_coalesce(ts);
+    char *str = isl_set_to_str(ts);
+    std::string r(str);
+    free(str);
+    isl_set_free(ts);
+    return r;
+}
+
+computation *computation::cache_shared(computation &inp, const var &level, const std::vector<int> buffer_shape,
+                                       const std::vector<expr> copy_offsets, bool pad_buffer) {
+    const size_t nd = inp.iterator_names_.size();
+    if (buffer_shape.size() != nd || copy_offsets.size() != nd)
+        ERROR("cache_shared: buffer shape and copy offsets must have one entry per dimension of " + inp.get_name(), true);
+    const int copy_level = get_loop_level_number_from_dimension_name(level.get_name());
+    std::tuple<int, int, int> block_dims(-1, -1, -1), thread_dims(-1, -1, -1);
+    for (auto &d : fct->gpu_block_dimensions) if (d.first == name) block_dims = d.second;
+    for (auto &d : fct->gpu_thread_dimensions) if (d.first == name) thread_dims = d.second;
+    if (std::get<0>(block_dims) == -1) ERROR("cache_shared: " + name + " is not mapped to the GPU", true);
+    if (thread_block_shape.empty()) ERROR("cache_shared: " + name + " has no thread block shape (use gpu_tile)", true);
+
+    // LDS buffer; padding the innermost dimension by one element avoids bank conflicts of
+    // column accesses (reference: tiramisu_core.cpp:9331-9336)
+    const std::string prefix = "_" + name + "_" + inp.get_name();
+    std::vector<expr> shape;
+    for (int v : buffer_shape) shape.push_back(expr((int32_t)v));
+    if (pad_buffer) shape.back() = expr((int32_t)(buffer_shape.back() + 1));
+    buffer *shared = new buffer(prefix + "_shared", shape, inp.get_data_type(), a_temporary, fct);
+    shared->tag_gpu_shared();
+
+    // reads of inp in this computation now go to the LDS tile: index modulo the tile shape
+    std::vector<var> access_vars;
+    std::vector<expr> access_exprs;
+    for (size_t d = 0; d < nd; d++) {
+        var v(inp.iterator_names_[d]);
+        access_vars.push_back(var(inp.iterator_names_[d], expr((int32_t)0), expr((int32_t)0x3fffffff)));
+        access_exprs.push_back(v % buffer_shape[d]);
+    }
+    bool saved = global::is_auto_data_mapping_set();
+    global::set_auto_data_mapping(false);
+    input *new_access = new input(prefix + "_access", access_vars, inp.get_data_type());
+    global::set_auto_data_mapping(saved);
+    new_access->store_in(shared, access_exprs);
+    set_expression(expression.substitute_access(inp.get_name(), new_access->get_name()));
+
+    int gpu_level = std::get<0>(thread_dims);
+    if (std::get<2>(thread_dims) != -1) gpu_level = std::get<2>(thread_dims);
+    else if (std::get<1>(thread_dims) != -1) gpu_level = std::get<1>(thread_dims);
+
+    auto map_like_this = [&](computation *c) {
+        fct->gpu_block_dimensions.push_back({c->get_name(), block_dims});
+        fct->gpu_thread_dimensions.push_back({c->get_name(), thread_dims});
+    };
+
+    // declaration of the tile at the beginning of the kernel
+    computation *decl = new computation(level_space(*this, gpu_level + 1, prefix + "_dec"), allocate(*shared), true, p_none, fct);
+    map_like_this(decl);
+
+    // cooperative copy: ceil(size / threads) iterations per thread
+    long size = 1, pool = 1;
+    for (int v : buffer_shape) size *= v;
+    for (int v : thread_block_shape) pool *= v;
+    const std::string iter = prefix + "_copy_iter";
+    std::string copy_dom = level_space(*this, copy_level + 1, prefix + "_copy");
+    {
+        // append the copy iterator with its bounds
+        size_t rb = copy_dom.find(']', copy_dom.find(prefix + "_copy["));
+        copy_dom.insert(rb, ", " + iter);
+        size_t end = copy_dom.rfind('}');
+        std::string cond = "0 <= " + iter + " <= " + std::to_string((size - 1) / pool);
+        bool has_constraints = copy_dom.find(':') != std::string::npos;
+        copy_dom.insert(end, std::string(has_constraints ? " and " : " : ") + cond + " ");
+    }
+    // linear thread id, slowest thread dimension first (reference: :9376-9422)
+    expr tid = var(level_names[std::get<0>(thread_dims)]);
+    if (std::get<1>(thread_dims) != -1) tid = tid * thread_block_shape[1] + var(level_names[std::get<1>(thread_dims)]);
+    if (std::get<2>(thread_dims) != -1) tid = tid * thread_block_shape[2] + var(level_names[std::get<2>(thread_dims)]);
+    expr copy_index = var(iter) * (int32_t)pool + tid;
+    std::vector<expr> tile_idx(nd), src_idx(nd);
+    long denom = 1;
+    for (int d = (int)nd - 1; d >= 0; d--) {
+        tile_idx[d] = (denom == 1 ? copy_index : copy_index / (int32_t)denom) % buffer_shape[d];
+        src_idx[d] = tile_idx[d] + copy_offsets[d];
+        denom *= buffer_shape[d];
+    }
+    computation *copy = new computation(copy_dom, expr(o_access, inp.get_name(), src_idx, inp.get_data_type()), true,
+                                        inp.get_data_type(), fct);
+    copy->store_in(shared, tile_idx);
+    if (size % pool != 0) copy->add_predicate(copy_index < (int32_t)size);
+    map_like_this(copy);
+
+    // barriers around the copy
+    computation *sync1 = new computation(level_space(*this, copy_level + 1, prefix + "_sync1"), tiramisu::sync(), true, p_none, fct);
+    computation *sync2 = new computation(level_space(*this, copy_level + 1, prefix + "_sync2"), tiramisu::sync(), true, p_none, fct);
+    map_like_this(sync1);
+    map_like_this(sync2);
+
+    // order: [...] -> sync1 -> copy -> sync2 -> first computation at the copy level
+    // (reference: :9479-9515)
+    {
+        computation *curr = this, *pred = curr->get_predecessor();
+        while (pred != nullptr && fct->sched_graph[pred][curr] >= copy_level) {
+            curr = pred;
+            pred = curr->get_predecessor();
+        }
+        if (pred != nullptr) sync1->between(*pred, fct->sched_graph[pred][curr], *curr, copy_level);
+        else sync1->before(*curr, copy_level);
+        sync2->between(*sync1, copy_level, *curr, copy_level);
+        copy->between(*sync1, copy_level, *sync2, copy_level);
+    }
+    {
+        computation *curr = this, *pred = curr->get_predecessor();
+        while (pred != nullptr && fct->sched_graph[pred][curr] >= gpu_level) {
+            curr = pred;
+            pred = curr->get_predecessor();
+        }
+        if (pred != nullptr) decl->between(*pred, fct->sched_graph[pred][curr], *curr, gpu_level);
+        else decl->before(*curr, gpu_level);
+    }
+    return new_access;
+}
+
 void computation::gen_time_space_domain() {
     if (time_space_domain) isl_set_free(time_space_domain);
     isl_set *d = isl_set_copy(iteration_domain);

@@ -94,6 +94,7 @@ isl_size isl_set_dim(isl_set *set, enum isl_dim_type type);
 const char *isl_set_get_dim_name(isl_set *set, enum isl_dim_type type, unsigned pos);
 const char *isl_set_get_tuple_name(isl_set *set);
 isl_set *isl_set_set_tuple_name(isl_set *set, const char *s);
+isl_set *isl_set_set_dim_name(isl_set *set, enum isl_dim_type type, unsigned pos, const char *s);
 isl_set *isl_set_intersect(isl_set *a, isl_set *b);
 isl_set *isl_set_intersect_params(isl_set *set, isl_set *params);
 isl_set *isl_set_subtract(isl_set *a, isl_set *b);
