@@ -317,6 +317,13 @@ void flatten_sum(const expr &e, std::vector<expr> &terms) {
 
 bool is_load(const expr &e) { return e.get_expr_type() == e_op && e.get_op_type() == o_access; }
 
+// A factor of a product: a load, possibly widened to fp32 (bf16 storage).
+bool is_factor(const expr &e) {
+    if (is_load(e)) return true;
+    return e.get_expr_type() == e_op && e.get_op_type() == o_cast && e.get_data_type() == p_float32 && is_load(e.get_operand(0));
+}
+expr strip_cast(const expr &e) { return is_load(e) ? e : e.get_operand(0); }
+
 bool same_element(const expr &load, const buffer *b, const std::vector<expr> &idx) {
     if (!is_load(load) || load.get_name() != b->get_name() || load.get_access().size() != idx.size()) return false;
     for (size_t i = 0; i < idx.size(); i++)
@@ -390,8 +397,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         bool shape = true;
         for (auto &t : terms) {
             if (same_element(t, cl->lhs, cl->lhs_index)) { self++; continue; }
-            if (t.get_expr_type() == e_op && t.get_op_type() == o_mul && is_load(t.get_operand(0)) && is_load(t.get_operand(1)))
-                prods.push_back({t.get_operand(0), t.get_operand(1)});
+            if (t.get_expr_type() == e_op && t.get_op_type() == o_mul && is_factor(t.get_operand(0)) && is_factor(t.get_operand(1)))
+                prods.push_back({strip_cast(t.get_operand(0)), strip_cast(t.get_operand(1))});
             else
                 shape = false;
         }
@@ -552,7 +559,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     };
     auto analyse = [&](const expr &ld, const group_info &rowg, operand_info &o) -> bool {
         buffer *b = f->get_buffers().at(ld.get_name());
-        if (b->get_location() != memory_location::global || b->get_elements_type() != p_float32 || written.count(b->get_name())) return false;
+        if (b->get_location() != memory_location::global || written.count(b->get_name())) return false;
+        if (b->get_elements_type() != p_float32 && b->get_elements_type() != p_bfloat16) return false;
         o.buf = b;
         expr lin = lir::linearize(b, ld.get_access());
         bool okc = true;
@@ -585,6 +593,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     }
     for (auto &o : operands)
         if (o.first.kmajor != operands[0].first.kmajor || o.second.kmajor != operands[0].second.kmajor) return reject(20);
+    // storage type: all fp32, or all bf16 (plain row-major operands only)
+    bool bf16 = false;
+    {
+        int nb = 0, nf = 0;
+        for (auto &o : operands)
+            for (const operand_info *g : {&o.first, &o.second}) (g->buf->get_elements_type() == p_bfloat16 ? nb : nf)++;
+        if (nb && nf) return reject(23);
+        bf16 = nb > 0;
+    }
 
     // ---- sizes and tile configuration
     const expr Me = GM.total, Ne = GN.total, Ke = GK.total;
@@ -597,6 +614,20 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         else if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
     }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
+    if (bf16) {
+        // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
+        if (!lit) return reject(24);
+        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 32 == 0) { BM = BN = 256; BK = 32; }
+        else if (Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0) { BM = BN = 64; BK = 64; }
+        else return reject(24);
+        WGM = WGN = 2;
+        for (auto &o : operands) {
+            long v;
+            if (!o.first.linear || !o.second.linear || !o.first.kmajor || o.second.kmajor) return reject(25);
+            for (const operand_info *g : {&o.first, &o.second})
+                if (!literal_value(g->ld, v) || v % 8 != 0 || !literal_value(g->base, v) || v % 8 != 0) return reject(25);
+        }
+    }
     bool edge = !(lit && Ml % BM == 0 && Nl % BN == 0 && Kl % BK == 0);
     for (auto &o : operands)
         for (const operand_info *g : {&o.first, &o.second}) {
@@ -646,8 +677,13 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
                             std::to_string(WGM) + ", " + std::to_string(WGN) + ", " + (operands[0].first.kmajor ? "true" : "false") + ", " +
                             (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ">";
     const int NT = 64 * WGM * WGN;
-    body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
-    body << "    typedef " << cfg << " CFG;\n";
+    if (bf16) {
+        body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
+        body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
+    } else {
+        body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
+        body << "    typedef " << cfg << " CFG;\n";
+    }
     body << "    const int _M = " << dev.print(Me) << ", _N = " << dev.print(Ne) << ", _K = " << dev.print(Ke) << ";\n";
     body << "    int _tm, _tn;\n    tgemm::tile_of_block((_M + CFG::BM - 1) / CFG::BM, (_N + CFG::BN - 1) / CFG::BN, _tm, _tn);\n";
     body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
@@ -655,6 +691,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
     for (auto &o : operands) {
         body << "    {\n";
+        if (bf16) {
+            used_buffers.insert(o.first.buf->get_name());
+            used_buffers.insert(o.second.buf->get_name());
+            body << "        tgemm::tile_accumulate_bf16<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
+                 << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << "), " << dev.print(o.second.ld)
+                 << ", _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+            term++;
+            continue;
+        }
         int which = 0;
         for (const operand_info *g : {&o.first, &o.second}) {
             const char *nm = which == 0 ? "_A" : "_B";
@@ -719,7 +764,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     k.name = kname;
     bool any_gather = false;
     for (auto &o : operands) any_gather = any_gather || !o.first.linear || !o.second.linear;
-    k.how = std::string("mfma-contraction: v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
+    k.how = std::string("mfma-contraction: ") + (bf16 ? "v_mfma_f32_32x32x16_bf16, " : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
             std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
             std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
             std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
@@ -758,6 +803,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         const int rowA = operands[0].first.kmajor ? (BK / 4) * (BM + PADX) * 4 : BK * BM;
         const int rowB = operands[0].second.kmajor ? (BK / 4) * (BN + PADX) * 4 : BK * BN;
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
+        if (bf16) k.lds_bytes = std::to_string(2 * ((BK / 8) * BM * 4 + (BK / 2) * BN) * 4);
     }
     std::ostringstream src;
     src << pre.str();
@@ -771,6 +817,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     src << ")\n{\n" << body.str() << "}\n";
     k.source = src.str();
     add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma.hip.h\"");
+    if (bf16) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_bf16.hip.h\"");
     host << launch_text(k, "        ") << "    }\n";
     plan.kernels.push_back(k);
     plan.host_code = host.str();
