@@ -172,15 +172,85 @@ def bench_copy(steps, warmup, with_cpu):
     return out
 
 
+def _generic_bench(name, host_arrays, flop, peak_tflops, steps, warmup, with_cpu, cpu_sample):
+    """A compiled function whose arguments are all GPU-resident (except leading host scalars)."""
+    from tiramisu_amd import runtime
+    from oracle import build as oracle_build
+    devs, args = [], []
+    for a in host_arrays:
+        if isinstance(a, tuple):         # ("host", array): passed as a host buffer
+            args.append(a[1])
+        else:
+            d = device_array(a)
+            devs.append(d)
+            args.append(d.buffer())
+    prog = runtime.load(PROGRAMS, name)
+    ms = time_steps(lambda: prog(*args), steps, warmup)
+    prof = kernel_profile(lambda: prog(*args), max(1, min(steps, 5)))
+    dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
+    dom_flop = flop / dom[1][1]          # the dominant kernel carries the contraction flops
+    achieved = dom_flop / (dom[1][0] * 1e-3) / 1e12
+    out = {"value": flop / (ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": ms,
+           "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
+                        "frac": achieved / peak_tflops, "traffic": None, "kernel": dom[0], "kernel_ms": dom[1][0],
+                        "launches_per_step": dom[1][1]},
+           "kernels": {k: {"ms": v[0], "launches_per_step": v[1]} for k, v in prof.items()}}
+    if with_cpu:
+        cpu = runtime.Program(oracle_build.cpu_program_library(PROGRAMS, name), name, needs_gpu_runtime=False)
+        host = [a[1] if isinstance(a, tuple) else a.copy() for a in host_arrays]
+        sec, runs = cpu_time(lambda: cpu(*host), min_seconds=2.0, max_runs=3)
+        out["cpu_baseline"] = {"value": flop / sec / 1e9, "unit": "GFLOP/s", "cores": cpu_threads(), "kind": "port",
+                               "sample": "whole workload, median of %d run(s) of the CPU-generated code (%s)" % (runs, cpu_sample)}
+    for d in devs:
+        d.free()
+    return out
+
+
+def bench_sgemm_bf16(steps, warmup, with_cpu):
+    M = N = K = 4096
+    rng = np.random.RandomState(16)
+
+    def bf16(a):
+        u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    A, B = bf16(rng.uniform(-1, 1, (M, K))), bf16(rng.uniform(-1, 1, (K, N)))
+    C = np.zeros((M, N), np.float32)
+    return _generic_bench("sgemm_bf16_4096x4096x4096", [("host", np.array([1.0, 0.0], np.float32)), A, B, C],
+                          2.0 * M * N * K, BF16_MFMA_PEAK_TFLOPS, steps, warmup, False, "")
+
+
+def bench_conv2d(steps, warmup, with_cpu):
+    N, CI, CO, H = 32, 64, 64, 112
+    rng = np.random.RandomState(4)
+    xp = np.zeros((N, CI, H + 2, H + 2), np.float32)
+    xp[:, :, 1:-1, 1:-1] = rng.uniform(0, 1, (N, CI, H, H)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (CO, CI, 3, 3)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, (CO,)).astype(np.float32)
+    out = np.zeros((N, CO, H, H), np.float32)
+    return _generic_bench("conv2d_32x64x64x112", [xp, w, b, out], 2.0 * N * CO * H * H * CI * 9, FP32_MFMA_PEAK_TFLOPS,
+                          steps, warmup, with_cpu, "parallelize n, vectorize x by 8")
+
+
+def bench_lstm(steps, warmup, with_cpu):
+    L, B, H, S = 4, 64, 512, 100
+    rng = np.random.RandomState(5)
+    w = rng.uniform(-0.08, 0.08, (L, 2, 4 * H, H)).astype(np.float32)
+    b = rng.uniform(-0.08, 0.08, (L, 4 * H)).astype(np.float32)
+    x = rng.uniform(-1, 1, (S, B, H)).astype(np.float32)
+    y = np.zeros((S, B, H), np.float32)
+    flop = L * S * 2 * (2.0 * B * 4 * H * H)
+    return _generic_bench("lstm_4x64x512x100", [w, b, x, y], flop, FP32_MFMA_PEAK_TFLOPS, max(2, steps // 4), max(1, warmup // 2),
+                          with_cpu, "unscheduled program, batch loop parallelized")
+
+
 WORKLOADS = {
     "heat2d": lambda s, w, c: bench_heat2d(s, w, c),
     "sgemm1024": lambda s, w, c: bench_sgemm(1024, s, w, c),
     "sgemm4096": lambda s, w, c: bench_sgemm(4096, s, w, c),
+    "sgemm4096_bf16": bench_sgemm_bf16,
+    "conv2d": bench_conv2d,
+    "lstm": bench_lstm,
 }
-try:
-    import bench_more  # noqa: F401  (further workloads register themselves when present)
-except ImportError:
-    pass
 
 
 def main():
@@ -212,7 +282,10 @@ def main():
         "dtype": "f32", "data": "synthetic (seeded uniform inputs, already resident in HBM)",
         "config": {"workload": {"heat2d": "heat2d 5-point stencil, fp32 grid 8192x8192, 32 time steps (BASELINE configs[1])",
                                 "sgemm1024": "sgemm fp32 1024^3 (BASELINE configs[0])",
-                                "sgemm4096": "sgemm fp32 4096^3 (BASELINE configs[2])"}.get(head_name, head_name)},
+                                "sgemm4096": "sgemm fp32 4096^3 (BASELINE configs[2])",
+                                "sgemm4096_bf16": "sgemm bf16-in/fp32-acc 4096^3 (BASELINE configs[2], bf16 variant)",
+                                "conv2d": "conv2d+bias+ReLU N32 C64->64 112x112 3x3 (BASELINE configs[3])",
+                                "lstm": "4-layer LSTM B64 H512 S100 (BASELINE configs[4])"}.get(head_name, head_name)},
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
         "workloads": {k: v for k, v in results.items() if k != head_name},
