@@ -33,7 +33,11 @@ PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
 # HBM bytes per launch of the dominant heat2d kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); see profiles/.
-HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {5: (165113.3 * 2.000 + 262080.0 * 1.000) * 1024}  # by time steps per launch
+HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # by time steps per launch; KiB counters x calibration factor
+    7: (180694.2 * 2.000 + 262333.1 * 1.000) * 1024,
+    3: (150888.7 * 2.000 + 264412.5 * 1.000) * 1024,
+    1: (137641.8 * 2.000 + 265178.7 * 1.000) * 1024,
+}
 
 
 def device_array(host):
@@ -81,6 +85,14 @@ def cpu_threads():
 
 # ---------------------------------------------------------------- workloads
 
+def stencil_steps_per_launch(kernel_source):
+    """{kernel name: time steps fused in one launch}, read from the emitted kernel source."""
+    import re
+    text = open(kernel_source).read()
+    return {m.group(1): int(m.group(2))
+            for m in re.finditer(r"#define ST_NAME (\w+)\n(?:#define (?!ST_R )\w+ .*\n)*#define ST_R (\d+)", text)}
+
+
 def bench_heat2d(steps, warmup, with_cpu):
     from tiramisu_amd import runtime
     from oracle import build as oracle_build
@@ -97,7 +109,7 @@ def bench_heat2d(steps, warmup, with_cpu):
     prof = kernel_profile(lambda: prog(buf), steps)
     # dominant kernel: the one with the largest total time per call
     dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
-    fused_steps = int(round((tsteps - 2) / dom[1][1])) if dom[1][1] else 1
+    fused_steps = stencil_steps_per_launch(os.path.join(PROGRAMS, "build", name + ".o.hip"))[dom[0]]
     per_launch_bytes = fused_steps * 2.0 * n * n * 4
     achieved = per_launch_bytes / (dom[1][0] * 1e-3) / 1e9
     out = {

@@ -1,0 +1,225 @@
+// Time-tiled 2-D stencil sweep for gfx950 with the tile held in registers: ST_R consecutive
+// time steps of
+//     new(y, x) = ST_EXPR( old(y+dy, x+dx) ... )   for (y, x) in the iteration domain,
+// on a ping-pong pair of planes, with one global read and one global write per cell for all
+// ST_R steps.  The stencil stays on the vector ALUs.
+//
+// A workgroup of ST_W wavefronts stages a region of ST_W*ST_RPT rows by 256 columns: wavefront w
+// owns rows [w*ST_RPT, (w+1)*ST_RPT), lane l owns columns [4l, 4l+4) of each of them, so a thread
+// keeps a strip of ST_RPT quads in registers through load, all steps and store.
+//   * horizontal neighbours live in the adjacent lanes of the same wavefront and arrive through
+//     DPP wavefront shifts (no memory traffic); the region is exactly one wavefront wide, so no
+//     value ever crosses a wavefront horizontally;
+//   * vertical neighbours across the strip boundary live in the wavefront above / below: every
+//     step each wavefront publishes its ST_RAD top and bottom rows in LDS (double-buffered by the
+//     step's parity, one barrier per step) and reads its neighbours' rows.
+// Every step the part of the region that still holds correct values shrinks by ST_RAD on each
+// side; after ST_R steps the centre (ST_TH x ST_TW) is written to the other plane.  Values outside
+// the shrinking valid part are computed from stale data and never used.
+//
+// Cells outside the iteration domain (the fixed boundary) are never written.  When a step needs
+// their value it takes the one their plane holds at that step's parity, read from global memory
+// (no launch ever writes those cells), so the two planes may hold different boundary values,
+// exactly as in the un-tiled program.  Only workgroups whose region touches the boundary run
+// that path; the choice is uniform over the workgroup.  Reading plane `src` and writing plane
+// `1-src` requires ST_R to be odd; the host code composes the time loop from odd chunks.
+//
+// Macros supplied by the emitter before this file is included:
+//   ST_NAME            kernel name
+//   ST_NY, ST_NX       plane extents (rows, columns)
+//   ST_Y0, ST_Y1, ST_X0, ST_X1   inclusive bounds of the iteration domain
+//   ST_R               time steps fused in one launch (odd)
+//   ST_RAD             stencil radius (<= 4, <= ST_RPT)
+//   ST_W               wavefronts per workgroup
+//   ST_RPT             rows per thread
+//   ST_EXPR            expression of the new value in terms of ST_AT(dy, dx)
+// The tile extents follow: ST_TH = ST_W*ST_RPT - 2*ST_R*ST_RAD, ST_TW = 256 - 2*roundup4(ST_R*ST_RAD).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define ST_HY (ST_R * ST_RAD)                       /* halo rows */
+#define ST_HX ((ST_R * ST_RAD + 3) / 4 * 4)         /* halo columns, multiple of 4 */
+#define ST_LH (ST_W * ST_RPT)
+#define ST_LW 256
+#define ST_TH (ST_LH - 2 * ST_HY)
+#define ST_TW (ST_LW - 2 * ST_HX)
+#define ST_CAT2(a, b) a##b
+#define ST_CAT(a, b) ST_CAT2(a, b)
+
+#ifndef TIRAMISU_AMD_STENCIL2D_REGS_COMMON
+#define TIRAMISU_AMD_STENCIL2D_REGS_COMMON
+typedef float st_f4 __attribute__((ext_vector_type(4)));
+
+// lane i receives lane i-1's value (lane 0 keeps its own)
+__device__ __forceinline__ float st_from_left(float v) {
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+}
+// lane i receives lane i+1's value (lane 63 keeps its own)
+__device__ __forceinline__ float st_from_right(float v) {
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+
+// Four cells of row gy starting at column gx (a multiple of 4) of a plane of NY x NX cells;
+// cells outside the plane read as 0.  With CHECK false the quad is known to be inside.
+// Element loads always use a clamped (valid) address and select afterwards.
+template <bool CHECK, int NY, int NX>
+__device__ __forceinline__ st_f4 st_load_quad(const float *__restrict__ plane, int gy, int gx) {
+    st_f4 v = {0.f, 0.f, 0.f, 0.f};
+    if (NX % 4 == 0) {
+        if (!CHECK) return *reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx);
+        const bool in = gy >= 0 && gy < NY && gx >= 0 && gx < NX;
+        const st_f4 a = *reinterpret_cast<const st_f4 *>(plane + (in ? (size_t)gy * NX + gx : (size_t)0));
+        return in ? a : v;
+    }
+    const bool row_in = !CHECK || (gy >= 0 && gy < NY);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int xx = gx + e;
+        const bool in = row_in && (!CHECK || (xx >= 0 && xx < NX));
+        const float a = plane[in ? (size_t)gy * NX + xx : (size_t)0];
+        v[e] = in ? a : 0.f;
+    }
+    return v;
+}
+#endif
+
+template <bool EDGE>
+__device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int bx, int by) {
+    // values stay in registers from one step to the next: without this the multiply that ends a
+    // step would be fused with an add of the next one, and results would differ from the
+    // un-tiled program's
+#pragma clang fp contract(off)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gy0 = by * ST_TH - ST_HY + wave * ST_RPT;   // plane row of my first row
+    const int gx = bx * ST_TW - ST_HX + 4 * lane;         // plane column of my quads
+    const int wave_up = wave > 0 ? wave - 1 : 0, wave_dn = wave < ST_W - 1 ? wave + 1 : ST_W - 1;
+
+    st_f4 cur[ST_RPT];
+#pragma unroll
+    for (int r = 0; r < ST_RPT; r++) cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
+
+    // xch[parity][wave][top|bottom][row][lane]
+    auto slot = [&](int parity, int w, int side, int i) -> st_f4 * {
+        return xch + ((((parity * ST_W + w) * 2 + side) * ST_RAD + i) * 64 + lane);
+    };
+
+#pragma unroll
+    for (int s = 1; s <= ST_R; s++) {
+        const int parity = s & 1;
+#pragma unroll
+        for (int i = 0; i < ST_RAD; i++) {
+            *slot(parity, wave, 0, i) = cur[i];
+            *slot(parity, wave, 1, i) = cur[ST_RPT - ST_RAD + i];
+        }
+        __syncthreads();
+        // my rows with ST_RAD rows of the neighbouring wavefronts above and below
+        st_f4 ext[ST_RPT + 2 * ST_RAD];
+#pragma unroll
+        for (int i = 0; i < ST_RAD; i++) {
+            ext[i] = *slot(parity, wave_up, 1, i);
+            ext[ST_RAD + ST_RPT + i] = *slot(parity, wave_dn, 0, i);
+        }
+#pragma unroll
+        for (int r = 0; r < ST_RPT; r++) ext[ST_RAD + r] = cur[r];
+        // the ST_RAD cells left and right of every quad, from the adjacent lanes
+        float lf[ST_RPT + 2 * ST_RAD][ST_RAD], rt[ST_RPT + 2 * ST_RAD][ST_RAD];
+#pragma unroll
+        for (int j = 0; j < ST_RPT + 2 * ST_RAD; j++)
+#pragma unroll
+            for (int i = 0; i < ST_RAD; i++) {
+                lf[j][i] = st_from_left(ext[j][4 - ST_RAD + i]);
+                rt[j][i] = st_from_right(ext[j][i]);
+            }
+#pragma unroll
+        for (int r = 0; r < ST_RPT; r++) {
+            // window of old values around the quad: rows -RAD..RAD, columns -RAD..3+RAD
+            float w[2 * ST_RAD + 1][4 + 2 * ST_RAD];
+#pragma unroll
+            for (int dy = -ST_RAD; dy <= ST_RAD; dy++) {
+                const int j = r + ST_RAD + dy;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[dy + ST_RAD][ST_RAD + e] = ext[j][e];
+#pragma unroll
+                for (int i = 0; i < ST_RAD; i++) {
+                    w[dy + ST_RAD][i] = lf[j][i];
+                    w[dy + ST_RAD][ST_RAD + 4 + i] = rt[j][i];
+                }
+            }
+            st_f4 fixed = {0.f, 0.f, 0.f, 0.f};
+            bool row_in = true;
+            if (EDGE) {
+                // a fixed cell shows the value of the plane that step s lives in
+                fixed = st_load_quad<true, ST_NY, ST_NX>(parity ? dst : src, gy0 + r, gx);
+                row_in = gy0 + r >= ST_Y0 && gy0 + r <= ST_Y1;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+#define ST_AT(dy, dx) w[(dy) + ST_RAD][e + (dx) + ST_RAD]
+                const float computed = (ST_EXPR);
+#undef ST_AT
+                if (EDGE) {
+                    const bool in_dom = row_in && gx + e >= ST_X0 && gx + e <= ST_X1;
+                    cur[r][e] = in_dom ? computed : fixed[e];
+                } else {
+                    cur[r][e] = computed;
+                }
+            }
+        }
+    }
+
+    // ---- write the tile centre (cells of the domain only)
+    if (4 * lane >= ST_HX && 4 * lane < ST_HX + ST_TW) {
+#pragma unroll
+        for (int r = 0; r < ST_RPT; r++) {
+            const int row = wave * ST_RPT + r, gy = gy0 + r;
+            if (row < ST_HY || row >= ST_HY + ST_TH) continue;
+            if (EDGE && (gy < ST_Y0 || gy > ST_Y1)) continue;
+            if ((ST_NX % 4 == 0) && (!EDGE || (gx >= ST_X0 && gx + 3 <= ST_X1))) {
+                *reinterpret_cast<st_f4 *>(dst + (size_t)gy * ST_NX + gx) = cur[r];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (!EDGE || (gx + e >= ST_X0 && gx + e <= ST_X1)) dst[(size_t)gy * ST_NX + gx + e] = cur[r][e];
+            }
+        }
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(64 * ST_W)
+#if ST_OCC > 0
+__attribute__((amdgpu_waves_per_eu(ST_OCC)))
+#endif
+ST_NAME(float *__restrict__ planes, const int src_plane)
+{
+    static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
+    static_assert(ST_RPT >= ST_RAD, "a strip must be at least as tall as the stencil radius");
+    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
+    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a band
+    // of consecutive tiles (row-major), so that tiles running together share their halos in L2.
+    const int nb = gridDim.x * gridDim.y, b = blockIdx.y * gridDim.x + blockIdx.x;
+#if ST_XCD
+    const int xcd = b % 8, per = nb / 8, extra = nb % 8;
+    const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / 8;
+#else
+    const int tile = b;
+#endif
+    const int bx = tile % gridDim.x, by = tile / gridDim.x;
+    const int ty0 = by * ST_TH - ST_HY, tx0 = bx * ST_TW - ST_HX;
+    // does the staged region lie inside the iteration domain?
+    const bool interior = ty0 >= ST_Y0 && ty0 + ST_LH - 1 <= ST_Y1 && tx0 >= ST_X0 && tx0 + ST_LW - 1 <= ST_X1;
+    if (interior) ST_CAT(ST_NAME, _sweep)<false>(src, dst, xch, bx, by);
+    else ST_CAT(ST_NAME, _sweep)<true>(src, dst, xch, bx, by);
+}
+
+#undef ST_HY
+#undef ST_HX
+#undef ST_LH
+#undef ST_LW
+#undef ST_TH
+#undef ST_TW
+#undef ST_CAT
+#undef ST_CAT2

@@ -98,7 +98,7 @@ void add_include_once(context &ctx, const std::string &line) {
 //     S(t, y, x) = f( S(t-1, y+dy, x+dx) ... ),   S stored at B[t mod 2, y, x].
 // Every read at step t is of step t-1 within a constant radius, so all flow dependences have
 // distance (1, dy, dx) and overlapped time tiles are legal; the time loop is replaced by
-// launches that each advance an odd number of steps (see kernels/stencil2d.hip.h).
+// launches that each advance an odd number of steps (see kernels/stencil2d_regs.hip.h).
 bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop, launch_plan &plan) {
     // either a host time loop around a mapped nest, or a mapped nest whose time step is fixed
     // (a one-step time loop has no loop node in the AST)
@@ -178,11 +178,16 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     // return both planes hold exactly what the un-tiled loop leaves there
     const long T0 = lo[0], T1 = hi[0];
     const long steps = T1 - T0 + 1;
-    int rmax = env_int("TIRAMISU_STENCIL_STEPS", 5);
+    // region staged by one workgroup: WAVES*ROWS rows by 256 columns (kernels/stencil2d_regs.hip.h)
+    const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", 8);
+    if (WAVES < 1 || WAVES > 16 || ROWS < radius || ROWS > 32) return false;
+    const int LH = WAVES * ROWS, LW = 256;
+    int rmax = env_int("TIRAMISU_STENCIL_STEPS", 7);
+    // keep at least half of the staged rows and columns as the tile
+    while (rmax > 1 && (4 * rmax * radius > LH || 4 * ((rmax * radius + 3) / 4 * 4) > LW)) rmax -= 1;
     if (rmax % 2 == 0) rmax -= 1;
     if (rmax < 1) rmax = 1;
-    const int TW = env_int("TIRAMISU_STENCIL_TW", 256), TH = env_int("TIRAMISU_STENCIL_TH", 32);
-    const int NT = env_int("TIRAMISU_STENCIL_THREADS", 512);
+    if (2 * radius >= LH) return false;
     std::vector<std::pair<long, int>> chunks;  // (first step, number of steps)
     long t = T0, rem = steps - 1;
     while (rem > 0) {
@@ -204,20 +209,23 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
         if (!by_steps.count(ch.second)) {
             kernel k;
             k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
+            const int HY = ch.second * radius, HX = (ch.second * radius + 3) / 4 * 4;
+            const int TH = LH - 2 * HY, TW = LW - 2 * HX;
             k.how = "stencil: " + std::to_string(ch.second) + " time step(s) per launch, radius " + std::to_string(radius) +
-                    ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + ", LDS halo";
+                    ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + " in registers, " + std::to_string(WAVES) +
+                    " wavefronts x " + std::to_string(ROWS) + " rows";
             std::ostringstream s;
             s << "#define ST_NAME " << k.name << "\n#define ST_NY " << NY << "\n#define ST_NX " << NX << "\n#define ST_Y0 " << lo[1]
-              << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2] << "\n#define ST_TH " << TH
-              << "\n#define ST_TW " << TW << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius << "\n#define ST_NT " << NT
-              << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d.hip.h\"\n"
-              << "#undef ST_NAME\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n#undef ST_TH\n"
-              << "#undef ST_TW\n#undef ST_R\n#undef ST_RAD\n#undef ST_NT\n#undef ST_EXPR\n";
+              << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2] << "\n#define ST_W " << WAVES
+              << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0) << "\n#define ST_RPT " << ROWS << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius
+              << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
+              << "#undef ST_NAME\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n#undef ST_W\n#undef ST_OCC\n#undef ST_XCD\n"
+              << "#undef ST_RPT\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
             k.source = s.str();
             k.params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}};
             k.grid[0] = std::to_string((NX + TW - 1) / TW);
             k.grid[1] = std::to_string((NY + TH - 1) / TH);
-            k.block[0] = std::to_string(NT);
+            k.block[0] = std::to_string(64 * WAVES);
             by_steps[ch.second] = k;
         }
         const long src = (((ch.first - 1) % 2) + 2) % 2;
