@@ -92,6 +92,64 @@ def heat2d(grid, steps, boundary_other=None):
     return planes
 
 
+def _shifted(plane, r, dy, dx):
+    """View of the interior (margin r) of `plane` displaced by (dy, dx)."""
+    ny, nx = plane.shape
+    return plane[r + dy:ny - r + dy, r + dx:nx - r + dx]
+
+
+def stencil_box9(planes, steps):
+    """`steps` sweeps of the weighted 3x3 box of tests/programs/stencil_shapes.cpp (box9) on a
+    ping-pong pair of planes (the iterated form of a 3x3 blur such as the reference's
+    benchmarks/halide/blurxy_tiramisu.cpp); fp32 operations in the order of the program text:
+    c*0.25 + (((n+s)+w)+e)*0.125 + (((nw+ne)+sw)+se)*0.0625.  Both planes are given and returned:
+    boundary cells (margin 1) keep the caller's values."""
+    p = planes.astype(np.float32).copy()
+    f = np.float32
+    for t in range(1, steps + 1):
+        s, d = p[(t - 1) % 2], p[t % 2]
+        g = lambda dy, dx: _shifted(s, 1, dy, dx)
+        axis = ((g(-1, 0) + g(1, 0)) + g(0, -1)) + g(0, 1)
+        diag = ((g(-1, -1) + g(-1, 1)) + g(1, -1)) + g(1, 1)
+        d[1:-1, 1:-1] = (g(0, 0) * f(0.25) + axis * f(0.125)) + diag * f(0.0625)
+    return p
+
+
+def stencil_far2(planes, steps):
+    """`steps` sweeps of the radius-2 stencil of tests/programs/stencil_shapes.cpp (far2):
+    c*0.5 + (((n2+s2)+w2)+e2)*0.0625 + (ne+sw)*0.125 with a fixed margin of 2 cells."""
+    p = planes.astype(np.float32).copy()
+    f = np.float32
+    for t in range(1, steps + 1):
+        s, d = p[(t - 1) % 2], p[t % 2]
+        g = lambda dy, dx: _shifted(s, 2, dy, dx)
+        far = ((g(-2, 0) + g(2, 0)) + g(0, -2)) + g(0, 2)
+        diag = g(-1, 1) + g(1, -1)
+        d[2:-2, 2:-2] = (g(0, 0) * f(0.5) + far * f(0.0625)) + diag * f(0.125)
+    return p
+
+
+def stencil_loops(planes, steps, radius, taps):
+    """Brute-force pin of the two functions above (tiny planes): `taps` is a list of
+    (weight, [(dy, dx), ...]) groups, each group summed left to right, scaled, and the scaled
+    groups added left to right."""
+    p = planes.astype(np.float32).copy()
+    ny, nx = p.shape[1:]
+    for t in range(1, steps + 1):
+        s, d = p[(t - 1) % 2], p[t % 2]
+        for y in range(radius, ny - radius):
+            for x in range(radius, nx - radius):
+                total = None
+                for weight, cells in taps:
+                    acc = np.float32(s[y + cells[0][0], x + cells[0][1]])
+                    for dy, dx in cells[1:]:
+                        acc = np.float32(acc + s[y + dy, x + dx])
+                    acc = np.float32(acc * np.float32(weight))
+                    total = acc if total is None else np.float32(total + acc)
+                d[y, x] = total
+    return p
+
+
 def heat2d_loops(grid, steps):
     """The same sweep as plain Python loops (tiny grids only): the brute-force pin of heat2d()."""
     n = grid.shape[0]
