@@ -9,8 +9,10 @@
 // LDS layouts are chosen so that neither the global loads nor the LDS accesses need a
 // transposition in registers:
 //   * an operand whose K index is contiguous in memory (row-major A, or a transposed B) is
-//     stored K-interleaved, [BK/4][X+1][4]: a 16-byte global load is a 16-byte LDS store, and a
-//     lane fetches 4 consecutive k for its row with one 16-byte LDS read (one read feeds 4 MFMA);
+//     stored K-interleaved, [BK/4][X+PAD][4]: a 16-byte global load is a 16-byte LDS store, and a
+//     lane fetches 4 consecutive k for its row with one 16-byte LDS read (one read feeds 4 MFMA).
+//     Row x of k-group kq sits at position x ^ 2*(kq % 4): the 8 lanes that store one 128-byte
+//     piece of two rows then hit 8 different 16-byte bank groups instead of 2;
 //   * an operand whose M/N index is contiguous (row-major B, or a transposed A) is stored as
 //     it lies, [BK][X]: 16-byte stores, 4-byte conflict-free reads (lanes read consecutive words).
 // For one 16-byte read q, the lower half of the wave (lanes 0-31) holds k = 8q+0..3 and the
@@ -24,6 +26,7 @@
 #define TIRAMISU_AMD_GEMM_MFMA_HIP_H
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace tgemm {
 
@@ -65,6 +68,8 @@ struct operand_tile {
     static_assert(X * BK / 4 % NT == 0, "tile must split evenly over the threads");
     static_assert(BK % 8 == 0, "BK must be a multiple of 8");
 
+    static __device__ __forceinline__ int swizzle(int x, int kq) { return x ^ (2 * (kq & 3)); }
+
     // SRC::load4(x, k) returns 4 consecutive elements along the operand's contiguous direction:
     // (x, k..k+3) for a K-major operand, (x..x+3, k) otherwise.
     template <class SRC>
@@ -87,7 +92,7 @@ struct operand_tile {
             const int idx = t + NT * v;
             if (KMAJOR) {
                 const int kq = idx % (BK / 4), x = idx / (BK / 4);
-                *reinterpret_cast<f32x4 *>(lds + kq * ROW + x * 4) = regs[v];
+                *reinterpret_cast<f32x4 *>(lds + kq * ROW + swizzle(x, kq) * 4) = regs[v];
             } else {
                 const int xq = idx % (X / 4), k = idx / (X / 4);
                 *reinterpret_cast<f32x4 *>(lds + k * ROW + 4 * xq) = regs[v];
@@ -98,7 +103,7 @@ struct operand_tile {
     // Values for the 4 MFMA steps of 16-byte read q: out[s] = element (x, 8q + 4h + s).
     static __device__ __forceinline__ f32x4 read_frag(const float *lds, int x, int q, int h) {
         if (KMAJOR) {
-            return *reinterpret_cast<const f32x4 *>(lds + (2 * q + h) * ROW + x * 4);
+            return *reinterpret_cast<const f32x4 *>(lds + (2 * q + h) * ROW + swizzle(x, 2 * q + h) * 4);
         } else {
             const float *p = lds + (8 * q + 4 * h) * ROW + x;
             f32x4 r = {p[0], p[ROW], p[2 * ROW], p[3 * ROW]};
@@ -165,44 +170,119 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     const int l32 = lane & 31, h = lane >> 5;
 
     f32x4 ra[opA::NV], rb[opB::NV];
-    float *sA[2] = {lds, lds + CFG::STAGE_FLOATS};
-    float *sB[2] = {lds + opA::LDS_FLOATS, lds + CFG::STAGE_FLOATS + opA::LDS_FLOATS};
+    // stage addresses are computed from `lds` (never selected between pointers) so that every
+    // access stays an LDS instruction
+    auto stage_a = [&](int stage) -> float * { return lds + stage * CFG::STAGE_FLOATS; };
+    auto stage_b = [&](int stage) -> float * { return lds + stage * CFG::STAGE_FLOATS + opA::LDS_FLOATS; };
+    constexpr int Q = BK / 8;                       // 16-byte fragment reads per slice
+    static_assert(Q >= 2 && Q % 2 == 0, "the pipeline needs an even number of fragment reads per slice");
+    f32x4 fa[2][TM], fb[2][TN];                     // fragments: one set in use, one in flight
 
+    auto read_frags = [&](int stage, int q, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[buf][i] = opA::read_frag(stage_a(stage), wm * CFG::WM + i * 32 + l32, q, h);
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[buf][j] = opB::read_frag(stage_b(stage), wn * CFG::WN + j * 32 + l32, q, h);
+    };
+
+    // Schedule of one slice (stage `cur` holds it, its first fragments are already in registers):
+    //   q = 0       store the next slice (in registers since the previous iteration) into the other
+    //               stage, ask global memory for the slice after it, read fragments q+1, multiply;
+    //   ...
+    //   q = Q-1     barrier (the other stage is complete; every fragment of this stage was read
+    //               before it), read the first fragments of the next slice, multiply.
+    // So the LDS store, the barrier and the first LDS reads of a slice are all covered by matrix
+    // instructions of the previous one, with a single barrier per slice.  Within a block of matrix
+    // instructions the memory instructions are dealt out one per matrix instruction (scheduling
+    // group barriers below); the steady-state slice is branch-free so that this is one scheduling
+    // region, and the last two slices are peeled.
     const int KT = (K + BK - 1) / BK;
     opA::load_global(A, m0, 0, ra);
     opB::load_global(B, n0, 0, rb);
-    opA::store_lds(sA[0], ra);
-    opB::store_lds(sB[0], rb);
-    __syncthreads();
-
-    for (int kt = 0; kt < KT; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) {
-            opA::load_global(A, m0, (kt + 1) * BK, ra);
-            opB::load_global(B, n0, (kt + 1) * BK, rb);
-        }
-#pragma unroll
-        for (int q = 0; q < BK / 8; q++) {
-            f32x4 fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) fa[i] = opA::read_frag(sA[cur], wm * CFG::WM + i * 32 + l32, q, h);
-#pragma unroll
-            for (int j = 0; j < TN; j++) fb[j] = opB::read_frag(sB[cur], wn * CFG::WN + j * 32 + l32, q, h);
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc.t[i][j], 0, 0, 0);
-        }
-        if (more) {
-            opA::store_lds(sA[cur ^ 1], ra);
-            opB::store_lds(sB[cur ^ 1], rb);
-        }
-        __syncthreads();
+    opA::store_lds(stage_a(0), ra);
+    opB::store_lds(stage_b(0), rb);
+    if (KT > 1) {
+        opA::load_global(A, m0, BK, ra);
+        opB::load_global(B, n0, BK, rb);
     }
+    __syncthreads();
+    read_frags(0, 0, 0);
+
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf][i][s], fb[buf][j][s], acc.t[i][j], 0, 0, 0);
+    };
+    constexpr int MFMAS = 4 * TM * TN;                                   // per fragment set
+    constexpr int FRAG_READS = TM + (CFG::B_KMAJOR ? TN : 2 * TN) + (CFG::A_KMAJOR ? 0 : TM);  // LDS read instructions per set (approx.)
+    // one slice; MORE: another slice follows (already in registers); LOAD: a slice after that exists
+    auto slice = [&](int kt, auto more_c, auto load_c) {
+        constexpr bool MORE = decltype(more_c)::value, LOAD = decltype(load_c)::value;
+        const int cur = kt & 1;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const int buf = q & 1;
+            if (q == 0 && MORE) {
+                opA::store_lds(stage_a(cur ^ 1), ra);
+                opB::store_lds(stage_b(cur ^ 1), rb);
+                if (LOAD) {
+                    opA::load_global(A, m0, (kt + 2) * BK, ra);
+                    opB::load_global(B, n0, (kt + 2) * BK, rb);
+                }
+            }
+            if (q + 1 < Q) {
+                read_frags(cur, q + 1, buf ^ 1);
+            } else {
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                if (MORE) read_frags(cur ^ 1, 0, buf ^ 1);
+            }
+            multiply(buf);
+            // spread the memory instructions of this block between the matrix instructions
+            constexpr int NVS = opA::NV + opB::NV;
+            constexpr int USED_FIRST = (MORE ? NVS : 0) + (MORE && LOAD ? NVS : 0) + FRAG_READS;
+            constexpr int USED_LAST = MORE ? FRAG_READS : 0;
+            if (q == 0 && MORE) {
+#pragma unroll
+                for (int i = 0; i < NVS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+                if (LOAD) {
+#pragma unroll
+                    for (int i = 0; i < NVS; i++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                }
+            }
+            if (q + 1 < Q || MORE) {
+#pragma unroll
+                for (int i = 0; i < FRAG_READS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+            // the remaining matrix instructions of the block (the builtin wants a positive constant)
+            constexpr int REST_FIRST = MFMAS > USED_FIRST ? MFMAS - USED_FIRST : 1;
+            constexpr int REST_LAST = MFMAS > USED_LAST ? MFMAS - USED_LAST : 1;
+            constexpr int REST_MID = MFMAS > FRAG_READS ? MFMAS - FRAG_READS : 1;
+            if (q == 0) { if (MFMAS > USED_FIRST) __builtin_amdgcn_sched_group_barrier(0x008, REST_FIRST, 0); }
+            else if (q + 1 == Q) { if (MFMAS > USED_LAST) __builtin_amdgcn_sched_group_barrier(0x008, REST_LAST, 0); }
+            else { if (MFMAS > FRAG_READS) __builtin_amdgcn_sched_group_barrier(0x008, REST_MID, 0); }
+        }
+    };
+    int kt = 0;
+    for (; kt + 2 < KT; kt++) slice(kt, std::true_type(), std::true_type());
+    if (kt + 1 < KT) { slice(kt, std::true_type(), std::false_type()); kt++; }
+    if (kt < KT) slice(kt, std::false_type(), std::false_type());
+    // the next call may overwrite stage 0 while a slow wavefront still multiplies: its fragments are
+    // in registers, and the barrier above ordered every LDS read of this call before that
 }
 
 // Hands every element of the tile to the epilogue: epi(row, col, value).
