@@ -8,11 +8,15 @@
 // (A) or column (B); lanes 0-31 take k = 0..7 of the step, lanes 32-63 take k = 8..15.
 //   * A slice [BM][BK] is stored as [BK/8][BM][8 bf16]: a 16-byte global load is a 16-byte LDS
 //     store, and one 16-byte LDS read is a lane's whole MFMA operand.
-//   * B slice [BK][BN] is stored as k-pairs, [BK/2][BN][2 bf16]: a thread loads two rows of 8
-//     columns, interleaves them in registers (one 32-bit word per (k pair, n)) and stores 32
-//     bytes; a lane assembles its operand from four conflict-free 4-byte reads (lanes read
-//     consecutive words).
-// Whole tiles only: M % BM == 0, N % BN == 0, K % BK == 0, rows 16-byte aligned (the emitter checks).
+//   * B slice [BK][BN] is stored the same way, [BK/8][BN][8 bf16], which needs a transposition: a
+//     thread loads 8 rows (k) of 4 columns (8 bytes each, lanes on consecutive columns), builds for
+//     each column the four (k, k+1) words with byte permutes and stores 16 bytes per column.  Column n
+//     of a k-group sits at position n ^ ((n / 8) % 8), which makes these stores conflict-free (lanes
+//     write every fourth column) and keeps the reads conflict-free.
+//   * Row m of k-group kq of A sits at position m ^ swz(kq) for the same reason (the lanes that
+//     store the k-groups of one row are 4096 bytes apart).
+// Whole tiles only: M % BM == 0, N % BN == 0, K % BK == 0, rows of A 16-byte and rows of B 8-byte
+// aligned (the emitter checks).
 #ifndef TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
 #define TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
 #include "gemm_mfma.hip.h"
@@ -21,6 +25,7 @@ namespace tgemm {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2), aligned(4)));
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
 struct config_bf16 {
@@ -29,12 +34,13 @@ struct config_bf16 {
     static constexpr int NT = 64 * WGM * WGN;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int A_WORDS = (BK / 8) * BM * 4;    // 32-bit words per stage
-    static constexpr int B_WORDS = (BK / 2) * BN;
+    static constexpr int B_WORDS = (BK / 8) * BN * 4;
     static constexpr int STAGE_WORDS = A_WORDS + B_WORDS;
     static constexpr int LDS_BYTES = 2 * STAGE_WORDS * 4;
     static constexpr int NVA = BM * (BK / 8) / NT;       // 16-byte loads of A per thread and slice
-    static constexpr int NVB = (BK / 2) * (BN / 8) / NT; // (two-row x 8-column) units of B per thread and slice
-    static_assert(BM * (BK / 8) % NT == 0 && (BK / 2) * (BN / 8) % NT == 0, "tile must split evenly over the threads");
+    static constexpr int UNITS_B = (BK / 8) * (BN / 4);  // (8-row x 4-column) units of B per slice
+    static constexpr int NVB = (UNITS_B + NT - 1) / NT;  // units per thread and slice
+    static_assert(BM * (BK / 8) % NT == 0, "tile must split evenly over the threads");
     static_assert(BK % 16 == 0, "BK must be a multiple of 16");
 };
 
@@ -43,83 +49,150 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
                                                      const uint16_t *__restrict__ B, long ldb, int K, int m0, int n0,
                                                      uint32_t *lds) {
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK, BM = CFG::BM, BN = CFG::BN, NT = CFG::NT;
+    constexpr int NVA = CFG::NVA, NVB = CFG::NVB;
+    constexpr int Q = BK / 16;                      // MFMA steps (fragment sets) per slice
+    static_assert(Q >= 2 && Q % 2 == 0, "the pipeline needs an even number of MFMA steps per slice");
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
 
-    u32x4 ra[CFG::NVA], rb0[CFG::NVB], rb1[CFG::NVB];
-    uint32_t *sA[2] = {lds, lds + CFG::STAGE_WORDS};
-    uint32_t *sB[2] = {lds + CFG::A_WORDS, lds + CFG::STAGE_WORDS + CFG::A_WORDS};
+    u32x4 ra[NVA];
+    u32x2 rb[NVB][8];
+    // stage addresses are computed from `lds` (never selected between pointers) so that every
+    // access stays an LDS instruction
+    auto stage_a = [&](int stage) -> uint32_t * { return lds + stage * CFG::STAGE_WORDS; };
+    auto stage_b = [&](int stage) -> uint32_t * { return lds + stage * CFG::STAGE_WORDS + CFG::A_WORDS; };
+    // row m of k-group kq sits at position m ^ swz(kq): the lanes that store the k-groups of one row
+    // (4096 bytes apart) then hit different 16-byte bank groups
+    auto swz = [](int kq) -> int { return (BK / 8 >= 8) ? (kq & 7) : 2 * (kq & 3); };
 
-    auto load = [&](int k0) {
+    auto load_a = [&](int k0) {
 #pragma unroll
-        for (int v = 0; v < CFG::NVA; v++) {
+        for (int v = 0; v < NVA; v++) {
             const int idx = t + NT * v, kq = idx % (BK / 8), m = idx / (BK / 8);
             ra[v] = *reinterpret_cast<const u32x4 *>(A + (long)(m0 + m) * lda + k0 + 8 * kq);
         }
+    };
+    auto col_pos = [](int n) -> int { return n ^ ((n >> 3) & 7); };
+    auto load_b = [&](int k0) {
 #pragma unroll
-        for (int v = 0; v < CFG::NVB; v++) {
-            const int idx = t + NT * v, n8 = idx % (BN / 8), kp = idx / (BN / 8);
-            const uint16_t *p = B + (long)(k0 + 2 * kp) * ldb + n0 + 8 * n8;
-            rb0[v] = *reinterpret_cast<const u32x4 *>(p);
-            rb1[v] = *reinterpret_cast<const u32x4 *>(p + ldb);
+        for (int v = 0; v < NVB; v++) {
+            const int idx = t + NT * v, n4 = idx % (BN / 4), kq = idx / (BN / 4);
+            if (CFG::UNITS_B % NT == 0 || idx < CFG::UNITS_B) {
+                const uint16_t *p = B + (long)(k0 + 8 * kq) * ldb + n0 + 4 * n4;
+#pragma unroll
+                for (int i = 0; i < 8; i++) rb[v][i] = *reinterpret_cast<const u32x2 *>(p + i * ldb);
+            }
         }
     };
-    auto store = [&](int stage) {
+    auto store_a = [&](int stage) {
 #pragma unroll
-        for (int v = 0; v < CFG::NVA; v++) {
+        for (int v = 0; v < NVA; v++) {
             const int idx = t + NT * v, kq = idx % (BK / 8), m = idx / (BK / 8);
-            *reinterpret_cast<u32x4 *>(sA[stage] + (kq * BM + m) * 4) = ra[v];
+            *reinterpret_cast<u32x4 *>(stage_a(stage) + (kq * BM + (m ^ swz(kq))) * 4) = ra[v];
         }
+    };
+    auto store_b = [&](int stage) {
 #pragma unroll
-        for (int v = 0; v < CFG::NVB; v++) {
-            const int idx = t + NT * v, n8 = idx % (BN / 8), kp = idx / (BN / 8);
-            // word j of the output = (row0[j], row1[j]) as (low, high) halves
-            u32x4 lo, hi;
+        for (int v = 0; v < NVB; v++) {
+            const int idx = t + NT * v, n4 = idx % (BN / 4), kq = idx / (BN / 4);
+            if (CFG::UNITS_B % NT == 0 || idx < CFG::UNITS_B) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t a = rb0[v][i], b = rb1[v][i];
-                const uint32_t even = (a & 0xffffu) | (b << 16), odd = (a >> 16) | (b & 0xffff0000u);
-                if (i < 2) { lo[2 * i] = even; lo[2 * i + 1] = odd; }
-                else       { hi[2 * (i - 2)] = even; hi[2 * (i - 2) + 1] = odd; }
+                for (int c = 0; c < 4; c++) {
+                    // word p of column c = (row 2p, row 2p+1) as (low, high) halves
+                    u32x4 w;
+#pragma unroll
+                    for (int pp = 0; pp < 4; pp++)
+                        w[pp] = __builtin_amdgcn_perm(rb[v][2 * pp + 1][c >> 1], rb[v][2 * pp][c >> 1],
+                                                      (c & 1) ? 0x07060302u : 0x05040100u);
+                    *reinterpret_cast<u32x4 *>(stage_b(stage) + (kq * BN + col_pos(4 * n4 + c)) * 4) = w;
+                }
             }
-            uint32_t *q = sB[stage] + kp * BN + 8 * n8;
-            *reinterpret_cast<u32x4 *>(q) = lo;
-            *reinterpret_cast<u32x4 *>(q + 4) = hi;
         }
+    };
+    bf16x8 fa[2][TM], fb[2][TN];                    // fragments: one set in use, one in flight
+    auto read_frags = [&](int stage, int s, int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int kq = 2 * s + h, m = wm * CFG::WM + i * 32 + l32;
+            const u32x4 w = *reinterpret_cast<const u32x4 *>(stage_a(stage) + (kq * BM + (m ^ swz(kq))) * 4);
+            fa[buf][i] = __builtin_bit_cast(bf16x8, w);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int kq = 2 * s + h, n = wn * CFG::WN + j * 32 + l32;
+            const u32x4 w = *reinterpret_cast<const u32x4 *>(stage_b(stage) + (kq * BN + col_pos(n)) * 4);
+            fb[buf][j] = __builtin_bit_cast(bf16x8, w);
+        }
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc.t[i][j], 0, 0, 0);
     };
 
+    // Same schedule as the fp32 loop (gemm_mfma.hip.h): while the matrix cores work through the
+    // Q fragment sets of one slice, the next slice (in registers since the previous iteration) is
+    // stored into the other stage -- A during set 0, B during set 1 -- each followed by the global
+    // loads of the slice after it; the barrier sits before the last set, whose matrix instructions
+    // cover the first fragment reads of the next slice.  Memory instructions are dealt out between
+    // the matrix instructions with scheduling groups.
     const int KT = K / BK;
-    load(0);
-    store(0);
-    __syncthreads();
-    for (int kt = 0; kt < KT; kt++) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) load((kt + 1) * BK);
-#pragma unroll
-        for (int s = 0; s < BK / 16; s++) {
-            bf16x8 fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-                const u32x4 w = *reinterpret_cast<const u32x4 *>(sA[cur] + ((2 * s + h) * BM + wm * CFG::WM + i * 32 + l32) * 4);
-                fa[i] = __builtin_bit_cast(bf16x8, w);
-            }
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const uint32_t *p = sB[cur] + (8 * s + 4 * h) * BN + wn * CFG::WN + j * 32 + l32;
-                const u32x4 w = {p[0], p[BN], p[2 * BN], p[3 * BN]};
-                fb[j] = __builtin_bit_cast(bf16x8, w);
-            }
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc.t[i][j], 0, 0, 0);
-        }
-        if (more) store(cur ^ 1);
-        __syncthreads();
+    load_a(0);
+    load_b(0);
+    store_a(0);
+    store_b(0);
+    if (KT > 1) {
+        load_a(BK);
+        load_b(BK);
     }
+    __syncthreads();
+    read_frags(0, 0, 0);
+
+    constexpr int MFMAS = TM * TN;
+    constexpr int FRAG_READS = TM + TN;             // LDS read instructions per set
+    auto slice = [&](int kt, auto more_c, auto load_c) {
+        constexpr bool MORE = decltype(more_c)::value, LOAD = decltype(load_c)::value;
+        const int cur = kt & 1;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const int buf = q & 1;
+            if (q == 0 && MORE) {
+                store_a(cur ^ 1);
+                if (LOAD) load_a((kt + 2) * BK);
+            }
+            if (q == (Q > 2 ? 1 : 0) && MORE) {
+                store_b(cur ^ 1);
+                if (LOAD) load_b((kt + 2) * BK);
+            }
+            if (q + 1 < Q) {
+                read_frags(cur, q + 1, buf ^ 1);
+            } else {
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                if (MORE) read_frags(cur ^ 1, 0, buf ^ 1);
+            }
+            multiply(buf);
+            if (q + 1 < Q || MORE) {
+#pragma unroll
+                for (int i = 0; i < MFMAS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (q + 1 < Q && MORE) {
+                        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                        if (LOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                    if (i < FRAG_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt + 2 < KT; kt++) slice(kt, std::true_type(), std::true_type());
+    if (kt + 1 < KT) { slice(kt, std::true_type(), std::false_type()); kt++; }
+    if (kt < KT) slice(kt, std::false_type(), std::false_type());
 }
 
 }  // namespace tgemm

@@ -625,7 +625,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     if (bf16) {
         // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
         if (!lit) return reject(24);
-        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 32 == 0) { BM = BN = 256; BK = 32; }
+        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 64 == 0) { BM = BN = 256; BK = 64; }
         else if (Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0) { BM = BN = 64; BK = 64; }
         else return reject(24);
         WGM = WGN = 2;
@@ -811,7 +811,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         const int rowA = operands[0].first.kmajor ? (BK / 4) * (BM + PADX) * 4 : BK * BM;
         const int rowB = operands[0].second.kmajor ? (BK / 4) * (BN + PADX) * 4 : BK * BN;
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
-        if (bf16) k.lds_bytes = std::to_string(2 * ((BK / 8) * BM * 4 + (BK / 2) * BN) * 4);
+        if (bf16) k.lds_bytes = std::to_string(2 * (BK / 8) * (BM + BN) * 4 * 4);
     }
     std::ostringstream src;
     src << pre.str();
