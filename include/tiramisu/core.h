@@ -126,6 +126,19 @@ public:
     int gpu_thread_position(const std::string &comp, int level) const;
 
     // ---- the code generation pipeline (reference: tiramisu_function.cpp:2540-2562) ----
+    /** CPU buffer name -> the GPU buffer declared as its counterpart (the last argument of the
+      * buffer constructor); reference: core.h:903-911. */
+    std::map<std::string, buffer *> mapping;
+    const std::map<std::string, buffer *> &get_mapping() const { return mapping; }
+    void add_mapping(std::pair<std::string, buffer *> p) { mapping.insert(p); }
+    /** First / last computation of the ordering chain (reference: tiramisu_function.cpp:1141-1165). */
+    computation *get_first_cpt();
+    computation *get_last_cpt();
+    /** Insert the host-to-device copies of mapped input buffers before \p c1 and the device-to-host
+      * copies of mapped output buffers after \p c2 (reference: tiramisu_function.cpp:379-435).
+      * Called by codegen() for a GPU target when the function has mapped buffers. */
+    void Automatic_communication(computation *c1, computation *c2);
+
     void set_arguments(const std::vector<buffer *> &buffer_vec);
     /** Turn the ordering graph into static schedule dimensions (reference :2231-2295). */
     void gen_ordering_schedules();
@@ -175,6 +188,11 @@ class buffer {
 
 public:
     memory_location location = memory_location::host;
+    /** Whether codegen() inserts the copies between this GPU buffer and its CPU counterpart
+      * (reference: core.h:1467-1470). */
+    bool automatic_gpu_copy = true;
+    bool get_automatic_gpu_copy() const { return automatic_gpu_copy; }
+    void set_automatic_gpu_copy(bool v) { automatic_gpu_copy = v; }
 
     /** Reference: tiramisu_core.cpp:6762-6781. */
     buffer(std::string name, std::vector<expr> dim_sizes, primitive_t type, argument_t argt,
@@ -335,6 +353,7 @@ public:
     computation &then(computation &next_computation, int L);
     void fuse_after(var lev, computation &comp) { after(comp, lev); }
     computation *get_predecessor();
+    computation *get_successor();
 
     // ---- loop transformations ----
     virtual void split(var L0, int sizeX);

@@ -60,6 +60,12 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
 void *tiramisu_hip_module_load(const void *image, uint64_t size);
 /* Look a kernel up by name; exits with status 1 if the module does not define it. */
 void *tiramisu_hip_module_get_function(void *module, const char *kernel_name);
+/* Device address of a global variable of the module (a __constant__ array holding a buffer tagged
+ * tag_gpu_constant()); exits with status 1 if the module does not define it or it is smaller
+ * than `bytes`.  Replaces the `<buffer>_get_symbol()` host function the reference emits into its
+ * .cu file (src/tiramisu_codegen_cuda.cpp:817-823); its result is what
+ * tiramisu_hip_memcpy_to_symbol() takes as destination. */
+void *tiramisu_hip_module_get_global(void *module, const char *name, uint64_t bytes);
 /* Launch on the current stream.  args[i] points to the i-th kernel argument. */
 int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3],
                         uint32_t dynamic_lds_bytes, void **args);

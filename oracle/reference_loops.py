@@ -92,6 +92,18 @@ def heat2d(grid, steps, boundary_other=None):
     return planes
 
 
+def row_filter(image, taps):
+    """out[r, c] = sum_t image[r, c + t] * taps[t] in fp32, products added left to right: the loop
+    nest of tests/programs/taps_in_constant_memory.cpp (a one-dimensional pass of the reference's
+    benchmarks/halide/gaussiangpu_tiramisu.cpp:46-57)."""
+    n = taps.shape[0]
+    width = image.shape[1] - n + 1
+    acc = image[:, 0:width] * taps[0]
+    for t in range(1, n):
+        acc = acc + image[:, t:t + width] * taps[t]
+    return acc.astype(np.float32)
+
+
 def _shifted(plane, r, dy, dx):
     """View of the interior (margin r) of `plane` displaced by (dy, dx)."""
     ny, nx = plane.shape

@@ -57,6 +57,24 @@ def test_gemm_register_tile(programs_dir):
     assert np.array_equal(C, C_cpu)
 
 
+def test_taps_in_constant_memory_with_automatic_copies(programs_dir):
+    # host buffers in, host buffer out: every copy (one of them to a constant-memory symbol) is
+    # inserted by codegen() from the CPU/GPU buffer mapping
+    rng = np.random.RandomState(61)
+    img, taps = ints(rng, (70, 100)), ints(rng, (5,))
+    out = np.full((70, 96), -1.0, np.float32)
+    out_cpu = out.copy()
+    cpu_variant(programs_dir, "taps_in_constant_memory")(img, taps, out_cpu)
+    prog = runtime.load(programs_dir, "taps_in_constant_memory")
+    prog(img, taps, out)
+    assert np.array_equal(out, ref.row_filter(img, taps))
+    assert np.array_equal(out, out_cpu)
+    # the symbol keeps no state between calls: new taps, new result
+    taps2 = ints(np.random.RandomState(62), (5,))
+    prog(img, taps2, out)
+    assert np.array_equal(out, ref.row_filter(img, taps2))
+
+
 def test_alloc_in_time_loop(programs_dir):
     P = np.zeros((3, 24, 24), np.int32)
     Q = np.zeros((3, 40, 40), np.int32)

@@ -63,6 +63,31 @@ def test_cpu_gemm_register_tile():
     assert np.array_equal(C, expected)
 
 
+def test_row_filter_restatement_pins():
+    # a single unit tap is a shifted copy; all-ones taps on all-ones pixels count the taps
+    img = ints(np.random.RandomState(3), (6, 12))
+    for t in range(5):
+        taps = np.zeros(5, np.float32)
+        taps[t] = 1.0
+        assert np.array_equal(ref.row_filter(img, taps), img[:, t:t + 8])
+    assert np.all(ref.row_filter(np.ones((4, 9), np.float32), np.ones(5, np.float32)) == 5.0)
+    # against plain loops
+    taps = ints(np.random.RandomState(4), (5,))
+    loops = np.zeros((6, 8), np.float32)
+    for r in range(6):
+        for c in range(8):
+            loops[r, c] = sum(float(img[r, c + t]) * float(taps[t]) for t in range(5))
+    assert np.array_equal(ref.row_filter(img, taps), loops)
+
+
+def test_cpu_taps_in_constant_memory():
+    rng = np.random.RandomState(61)
+    img, taps = ints(rng, (70, 100)), ints(rng, (5,))
+    out = np.zeros((70, 96), np.float32)
+    cpu_program("taps_in_constant_memory")(img, taps, out)
+    assert np.array_equal(out, ref.row_filter(img, taps))
+
+
 def test_cpu_alloc_in_time_loop():
     P = np.zeros((3, 24, 24), np.int32)
     Q = np.zeros((3, 40, 40), np.int32)

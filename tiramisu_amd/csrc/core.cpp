@@ -273,9 +273,57 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
             gen_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu);
 }
 
+computation *function::get_first_cpt() {
+    computation *c = nullptr;
+    if (!sched_graph.empty()) c = sched_graph.begin()->first;
+    else
+        for (auto q : body)
+            if (q->should_schedule_this_computation()) { c = q; break; }
+    while (c && c->get_predecessor()) c = c->get_predecessor();
+    return c;
+}
+
+computation *function::get_last_cpt() {
+    computation *c = nullptr;
+    if (!sched_graph.empty()) c = sched_graph.begin()->first;
+    else
+        for (auto q : body)
+            if (q->should_schedule_this_computation()) { c = q; break; }
+    while (c && c->get_successor()) c = c->get_successor();
+    return c;
+}
+
+void function::Automatic_communication(computation *c1, computation *c2) {
+    if (!c1 || !c2) ERROR("automatic CPU/GPU copies need a first and a last computation", true);
+    if (c1->get_predecessor()) ERROR("Automatic_communication: " + c1->get_name() + " has a predecessor", true);
+    if (c2->get_successor()) ERROR("Automatic_communication: " + c2->get_name() + " has a successor", true);
+    computation *first = c1, *last = c2;
+    int n = 1;
+    for (auto &kv : mapping) {
+        buffer *cpu = buffers_list.at(kv.first), *gpu = kv.second;
+        if (gpu->get_argument_type() != a_temporary)
+            ERROR("buffer " + gpu->get_name() + ": the GPU counterpart of a CPU buffer must be a temporary", true);
+        if (!gpu->get_automatic_gpu_copy()) continue;     // the program copies by hand
+        const bool to_constant = gpu->get_location() == memory_location::constant;
+        if (cpu->get_argument_type() == a_input) {
+            computation *c = new computation("cpt" + std::to_string(n++), {}, memcpy(*cpu, *gpu));
+            c->then(*first, computation::root);
+            first = c;
+        }
+        if (!to_constant && cpu->get_argument_type() == a_output) {
+            computation *c = new computation("cpt" + std::to_string(n++), {}, memcpy(*gpu, *cpu));
+            last->then(*c, computation::root);
+            last = c;
+        }
+    }
+}
+
 void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename_in,
                        hardware_architecture_t arch) {
     if (arch == hardware_architecture_t::arch_nvidia_gpu) arch = hardware_architecture_t::arch_amd_gpu;
+    // mapped buffers get their copies inserted for a GPU target (reference: tiramisu_function.cpp:2542-2549)
+    if (arch == hardware_architecture_t::arch_amd_gpu && !mapping.empty())
+        Automatic_communication(get_first_cpt(), get_last_cpt());
     std::string obj_filename = obj_filename_in;
     // TIRAMISU_FORCE_ARCH=cpu compiles a GPU program for the host instead (GPU-mapped loops run
     // serially) and writes <name>_cpu.o: how the parity tests obtain CPU-generated code for the
@@ -318,13 +366,18 @@ lir::program &function::get_lowered_program() {
 // ------------------------------------------------------------------ buffer
 
 buffer::buffer(std::string nm, std::vector<expr> sizes, primitive_t t, argument_t argt, function *f,
-               std::string)
+               std::string corr)
     : name(nm), dim_sizes(std::move(sizes)), type(t), argtype(argt), fct(f) {
     if (!fct) ERROR("declare a function (tiramisu::init) before declaring buffers", true);
     if (name.empty()) ERROR("a buffer needs a name", true);
     for (auto &e : dim_sizes)
         if (!e.is_defined()) ERROR("undefined size expression for buffer " + name, true);
     fct->add_buffer({name, this});
+    if (!corr.empty()) {
+        // this is the GPU counterpart of CPU buffer `corr` (reference: tiramisu_core.cpp:6775-6779)
+        if (!fct->get_buffers().count(corr)) ERROR("buffer " + name + ": no CPU buffer named " + corr, true);
+        fct->add_mapping({corr, this});
+    }
 }
 
 bool buffer::has_constant_extents() const {
@@ -903,8 +956,13 @@ computation &computation::then(computation &next, var L) { next.after(*this, L);
 computation &computation::then(computation &next, int L) { next.after(*this, L); return next; }
 
 computation *computation::get_predecessor() {
-    auto &r = fct->sched_graph_reversed[this];
-    return r.empty() ? nullptr : r.begin()->first;
+    auto it = fct->sched_graph_reversed.find(this);
+    return (it == fct->sched_graph_reversed.end() || it->second.empty()) ? nullptr : it->second.begin()->first;
+}
+
+computation *computation::get_successor() {
+    auto it = fct->sched_graph.find(this);
+    return (it == fct->sched_graph.end() || it->second.empty()) ? nullptr : it->second.begin()->first;
 }
 
 // Static dimensions before the fuse level are copied from the predecessor; the one right

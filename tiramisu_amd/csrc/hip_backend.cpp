@@ -259,7 +259,10 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
             ERROR("buffer " + nm + " is used inside a GPU kernel but lives in host memory; tag it with tag_gpu_global() "
                   "and copy it with memcpy()", true);
         case memory_location::constant:
-            ERROR("buffer " + nm + ": constant memory is not provided by this back-end; use tag_gpu_global()", true);
+            // a file-scope __constant__ array of the code object: not a parameter
+            // (reference: tiramisu_codegen_cuda.cpp:811-829, :1192-1193)
+            ctx.constant_buffers.insert(nm);
+            break;
         default:
             if (!g.declared.count(nm)) top_decls.push_back(g.declaration(b));
         }
@@ -397,9 +400,16 @@ struct host_gen {
         case leaf_kind::sync: return;
         case leaf_kind::copy: {
             buffer *s = n->copy_from, *d = n->copy_to;
-            bool sg = s->get_location() == memory_location::global, dg = d->get_location() == memory_location::global;
+            auto on_device = [](const buffer *b) {
+                return b->get_location() == memory_location::global || b->get_location() == memory_location::constant;
+            };
+            for (const buffer *b : {s, d})
+                if (b->get_location() != memory_location::host && !on_device(b))
+                    ERROR("memcpy computation " + n->comp->get_name() + ": buffer " + b->get_name() + " lives inside a kernel", true);
+            bool sg = on_device(s), dg = on_device(d);
             std::string bytes = "(uint64_t)(" + hp.element_count(s) + ") * sizeof(" + primitive_c_name(s->get_elements_type()) + ")";
-            const char *fn = (!sg && dg) ? "tiramisu_hip_memcpy_to_device" : (sg && !dg) ? "tiramisu_hip_memcpy_to_host"
+            const char *fn = (!sg && d->get_location() == memory_location::constant) ? "tiramisu_hip_memcpy_to_symbol"
+                             : (!sg && dg) ? "tiramisu_hip_memcpy_to_device" : (sg && !dg) ? "tiramisu_hip_memcpy_to_host"
                              : (sg && dg) ? "tiramisu_hip_memcpy_device_to_device" : nullptr;
             if (fn) out << pad(ind) << fn << "((void *)" << d->get_name() << ", (void *)" << s->get_name() << ", " << bytes << ");\n";
             else out << pad(ind) << "memcpy((void *)" << d->get_name() << ", (void *)" << s->get_name() << ", " << bytes << ");\n";
@@ -521,6 +531,13 @@ public:
                 } else {
                     body << "    " << t << " *" << b->get_name() << " = nullptr;\n";
                 }
+            } else if (b->get_location() == memory_location::constant) {
+                // its storage is a __constant__ array of the code object; the host only needs its address
+                // (the reference's <name>_get_symbol(), tiramisu_codegen_cuda.cpp:817-823)
+                if (!b->has_constant_extents()) ERROR("constant-memory buffer " + b->get_name() + " needs constant extents", true);
+                ctx.constant_buffers.insert(b->get_name());
+                body << "    " << t << " *" << b->get_name() << " = (" << t << " *)tiramisu_hip_module_get_global(_tiramisu_module(), \""
+                     << b->get_name() << "\", " << bytes << ");\n";
             } else if (b->get_location() == memory_location::host) {
                 if (b->get_auto_allocate()) {
                     body << "    " << t << " *" << b->get_name() << " = (" << t << " *)malloc(" << bytes << ");\n";
@@ -537,16 +554,25 @@ public:
 
         // ---- kernel file
         const std::string hip_file = obj + ".hip", hsaco = obj + ".hsaco", host_file = obj + ".host.cpp";
-        if (!ctx.kernels.empty() && !std::getenv("HIP_NO_OVERWRITE")) {
+        const bool device_code = !ctx.kernels.empty() || !ctx.constant_buffers.empty();
+        if (device_code && !std::getenv("HIP_NO_OVERWRITE")) {
             std::ofstream k(hip_file);
             if (!k) ERROR("cannot write " + hip_file, true);
             k << "// Generated by the Tiramisu HIP back-end for gfx950.  Function: " << f.get_name() << "\n";
             k << "#include <hip/hip_runtime.h>\n#include <stdint.h>\n";
             k << ctx.includes;
             k << c_prelude(true) << "\n";
+            for (auto &nm : ctx.constant_buffers) {
+                const buffer *b = f.get_buffers().at(nm);
+                long cnt = 1;
+                for (auto &d : b->get_dim_sizes()) cnt *= lir::simplify(d).get_int_val();
+                if (cnt * (long)primitive_size(b->get_elements_type()) > 65536)
+                    ERROR("constant-memory buffer " + nm + " exceeds 64 KiB", true);
+                k << "__constant__ " << primitive_c_name(b->get_elements_type()) << " " << nm << "[" << cnt << "];\n";
+            }
             for (auto &kr : ctx.kernels) k << "// " << kr.name << ": " << kr.how << "\n" << kr.source << "\n";
         }
-        if (!ctx.kernels.empty()) {
+        if (device_code) {
             const char *hipcc = std::getenv("HIPCC_PATH");
             const char *arch = std::getenv("TIRAMISU_HIP_ARCH");
             const char *flags = std::getenv("TIRAMISU_HIP_FLAGS");
@@ -569,7 +595,7 @@ public:
             h << "#include <tiramisu_hip_wrappers.h>\n";
             h << halide_buffer_definition() << c_prelude(false) << "\n";
             for (auto &d : hg.extern_decls) h << d << "\n";
-            if (!ctx.kernels.empty()) {
+            if (device_code) {
                 char *abs_path = realpath(hsaco.c_str(), nullptr);
                 const std::string hsaco_abs = abs_path ? abs_path : hsaco;
                 free(abs_path);

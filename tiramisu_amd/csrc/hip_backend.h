@@ -47,6 +47,7 @@ struct context {
     std::vector<kernel> kernels;        // all kernels of the function, in emission order
     std::string includes;               // extra text at the top of the kernel file
     std::set<std::string> include_once;
+    std::set<std::string> constant_buffers;   // buffers living in the code object's constant memory
     int next_kernel_id();
 };
 

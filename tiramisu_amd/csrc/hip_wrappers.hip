@@ -225,6 +225,18 @@ void *tiramisu_hip_module_get_function(void *module, const char *kernel_name) {
     return (void *)f;
 }
 
+void *tiramisu_hip_module_get_global(void *module, const char *name, uint64_t bytes) {
+    hipDeviceptr_t ptr = nullptr;
+    size_t size = 0;
+    check(hipModuleGetGlobal(&ptr, &size, (hipModule_t)module, name), __FUNCTION__);
+    if (size < bytes) {
+        fprintf(stderr, "Error at %s: symbol %s holds %zu bytes, %llu needed\n", __FUNCTION__, name, size,
+                (unsigned long long)bytes);
+        exit(1);
+    }
+    return (void *)ptr;
+}
+
 int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3], uint32_t dynamic_lds_bytes,
                         void **args) {
     if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return 0;  // empty iteration space
