@@ -16,7 +16,7 @@ from tiramisu_amd import runtime
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
-SMALL = [(256, 256, 64), (128, 192, 96), (100, 70, 50), (33, 17, 9)]
+SMALL = [(256, 256, 64), (128, 192, 96), (100, 70, 50), (33, 17, 9), (64, 256, 512)]
 RTOL = 1e-4
 
 

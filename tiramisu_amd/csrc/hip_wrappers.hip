@@ -98,7 +98,7 @@ void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K
     else if (bm == 128)
         launch_mfma<tgemm::config<128, 128, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
     else
-        launch_mfma<tgemm::config<64, 64, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+        launch_mfma<tgemm::config<64, 64, 32, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
 }
 
 template <bool AK, bool BK_>

@@ -127,17 +127,22 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tm,
     tn = (id % per_group) / gsize;
 }
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_, int PAD_ = 1>
+// WGM x WGN wavefronts tile the block in M and N; WGK > 1 adds groups of wavefronts that each take
+// 1/WGK of every K-slice for the same C tile (for problems with too few C tiles to fill the chip);
+// their partial sums are added through LDS by tile_reduce_k before the epilogue.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_, int PAD_ = 1, int WGK_ = 1>
 struct config {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, WGK = WGK_;
     static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, EDGE = EDGE_;
-    static constexpr int NT = 64 * WGM * WGN;
+    static constexpr int NT = 64 * WGM * WGN * WGK;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     typedef operand_tile<BM, BK, NT, A_KMAJOR, EDGE, PAD_> opA;
     typedef operand_tile<BN, BK, NT, B_KMAJOR, EDGE, PAD_> opB;
     static constexpr int STAGE_FLOATS = opA::LDS_FLOATS + opB::LDS_FLOATS;
     static constexpr int LDS_BYTES = 2 * STAGE_FLOATS * 4;
     static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be made of 32x32 MFMA tiles");
+    static_assert((BK / 8) % WGK == 0, "the K-slice must split evenly over the K groups");
+    static_assert(WGK == 1 || (WGK - 1) * WGM * WGN * TM * TN * 16 * 64 <= 2 * STAGE_FLOATS, "LDS too small for the K reduction");
 };
 
 // Accumulator tiles of one wavefront.
@@ -166,7 +171,8 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     typedef typename CFG::opB opB;
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
+    const int wk = wave / (CFG::WGM * CFG::WGN), wmn = wave % (CFG::WGM * CFG::WGN);
+    const int wm = wmn / CFG::WGN, wn = wmn % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
 
     f32x4 ra[opA::NV], rb[opB::NV];
@@ -174,15 +180,15 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     // access stays an LDS instruction
     auto stage_a = [&](int stage) -> float * { return lds + stage * CFG::STAGE_FLOATS; };
     auto stage_b = [&](int stage) -> float * { return lds + stage * CFG::STAGE_FLOATS + opA::LDS_FLOATS; };
-    constexpr int Q = BK / 8;                       // 16-byte fragment reads per slice
+    constexpr int Q = BK / 8 / CFG::WGK;            // 16-byte fragment reads per slice (of this wavefront's K group)
     static_assert(Q >= 2 && Q % 2 == 0, "the pipeline needs an even number of fragment reads per slice");
     f32x4 fa[2][TM], fb[2][TN];                     // fragments: one set in use, one in flight
 
     auto read_frags = [&](int stage, int q, int buf) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) fa[buf][i] = opA::read_frag(stage_a(stage), wm * CFG::WM + i * 32 + l32, q, h);
+        for (int i = 0; i < TM; i++) fa[buf][i] = opA::read_frag(stage_a(stage), wm * CFG::WM + i * 32 + l32, wk * Q + q, h);
 #pragma unroll
-        for (int j = 0; j < TN; j++) fb[buf][j] = opB::read_frag(stage_b(stage), wn * CFG::WN + j * 32 + l32, q, h);
+        for (int j = 0; j < TN; j++) fb[buf][j] = opB::read_frag(stage_b(stage), wn * CFG::WN + j * 32 + l32, wk * Q + q, h);
     };
 
     // Schedule of one slice (stage `cur` holds it, its first fragments are already in registers):
@@ -285,10 +291,52 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     // in registers, and the barrier above ordered every LDS read of this call before that
 }
 
-// Hands every element of the tile to the epilogue: epi(row, col, value).
+// Adds the partial sums of the WGK groups of wavefronts into group 0 (through `lds`, the buffer
+// tile_accumulate used: its last barrier ordered every read of it before this).  Returns whether the
+// calling wavefront holds the sums, i.e. should run the epilogue.  All threads must call it.
+template <class CFG>
+__device__ __forceinline__ bool tile_reduce_k(accumulators<CFG> &acc, float *lds) {
+    if (CFG::WGK == 1) return true;
+    constexpr int WMN = CFG::WGM * CFG::WGN, REGS4 = CFG::TM * CFG::TN * 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wk = wave / WMN, wmn = wave % WMN;
+    // slot of (K group g >= 1, wavefront wmn, register quad r): 64 lanes x 16 bytes, conflict-free
+    auto slot = [&](int g, int r) -> f32x4 * {
+        return reinterpret_cast<f32x4 *>(lds) + (((g - 1) * WMN + wmn) * REGS4 + r) * 64 + lane;
+    };
+    if (wk > 0) {
+#pragma unroll
+        for (int i = 0; i < CFG::TM; i++)
+#pragma unroll
+            for (int j = 0; j < CFG::TN; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const f32x4 v = {acc.t[i][j][4 * r], acc.t[i][j][4 * r + 1], acc.t[i][j][4 * r + 2], acc.t[i][j][4 * r + 3]};
+                    *slot(wk, (i * CFG::TN + j) * 4 + r) = v;
+                }
+    }
+    __syncthreads();
+    if (wk > 0) return false;
+#pragma unroll
+    for (int g = 1; g < CFG::WGK; g++)
+#pragma unroll
+        for (int i = 0; i < CFG::TM; i++)
+#pragma unroll
+            for (int j = 0; j < CFG::TN; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const f32x4 v = *slot(g, (i * CFG::TN + j) * 4 + r);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc.t[i][j][4 * r + e] += v[e];
+                }
+    return true;
+}
+
+// Hands every element of the tile to the epilogue: epi(row, col, value).  With WGK > 1 only the
+// wavefronts for which tile_reduce_k returned true may call it.
 template <class CFG, class EPI>
 __device__ __forceinline__ void tile_epilogue(const accumulators<CFG> &acc, int M, int N, int m0, int n0, EPI epi) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % (CFG::WGM * CFG::WGN);
     const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
     // accumulator register r of a lane holds row 8*(r/4) + 4*h + r%4, column lane%32 of its tile
@@ -313,7 +361,7 @@ __device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long 
     linear_source<CFG::A_KMAJOR, CFG::EDGE> sa{A, lda, M, K, vec_ok};
     linear_source<CFG::B_KMAJOR, CFG::EDGE> sb{B, ldb, N, K, vec_ok};
     tile_accumulate<CFG>(acc, sa, sb, K, m0, n0, lds);
-    tile_epilogue<CFG>(acc, M, N, m0, n0, epi);
+    if (tile_reduce_k<CFG>(acc, lds)) tile_epilogue<CFG>(acc, M, N, m0, n0, epi);
 }
 
 struct axpby_epilogue {

@@ -364,6 +364,21 @@ bool literal_value(const expr &e, long &v) {
     return true;
 }
 
+// Is the integer expression provably a multiple of m (whatever its variables are)?
+bool multiple_of(const expr &e_in, long m) {
+    const expr e = lir::simplify(e_in);
+    if (e.is_integer_literal()) return e.get_int_val() % m == 0;
+    if (e.get_expr_type() != e_op) return false;
+    switch (e.get_op_type()) {
+    case o_add:
+    case o_sub: return multiple_of(e.get_operand(0), m) && multiple_of(e.get_operand(1), m);
+    case o_mul: return multiple_of(e.get_operand(0), m) || multiple_of(e.get_operand(1), m);
+    case o_minus:
+    case o_cast: return multiple_of(e.get_operand(0), m);
+    default: return false;
+    }
+}
+
 bool reject(int where) {
     if (std::getenv("TIRAMISU_HIP_REPORT")) std::cout << "[tiramisu-hip] contraction check " << where << " failed" << std::endl;
     return false;
@@ -615,13 +630,22 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const expr Me = GM.total, Ne = GN.total, Ke = GK.total;
     long Ml = -1, Nl = -1, Kl = -1;
     const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
-    int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2;
+    int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2, WGK = 1;
     if (lit) {
         if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0) { BM = BN = 256; PADX = 0; }
         else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256 && Ml >= 128) { BM = BN = 128; }
         else if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
     }
+    if (BM == 64 && BN == 64) BK = 32;   // one 32x32 tile per wavefront: longer slices, fewer barriers per flop
+    // few C tiles but a long reduction (a batch-sized M against wide weights, as in recurrent cells):
+    // 64x32 tiles, and 8 groups of wavefronts share the K range of each tile
+    if (lit && !bf16 && BM == 64 && BN == 64 && Ml <= 64 && ((Nl + 63) / 64) <= 64 && Nl % 32 == 0 && Kl % 128 == 0 && Kl >= 256 &&
+        !std::getenv("TIRAMISU_MFMA_NO_SPLITK")) {
+        BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
+    }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
+    if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
     if (bf16) {
         // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
         if (!lit) return reject(24);
@@ -641,7 +665,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         for (const operand_info *g : {&o.first, &o.second}) {
             long v;
             if (g->linear && (!literal_value(g->ld, v) || v % 4 != 0)) edge = true;
-            if (g->linear && (!literal_value(g->base, v) || v % 4 != 0)) edge = true;
+            if (g->linear && !multiple_of(g->base, 4)) edge = true;
         }
 
     // ---- kernel text
@@ -683,8 +707,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     std::ostringstream pre, body;
     const std::string cfg = "tgemm::config<" + std::to_string(BM) + ", " + std::to_string(BN) + ", " + std::to_string(BK) + ", " +
                             std::to_string(WGM) + ", " + std::to_string(WGN) + ", " + (operands[0].first.kmajor ? "true" : "false") + ", " +
-                            (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ">";
-    const int NT = 64 * WGM * WGN;
+                            (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ", " + std::to_string(WGK) + ">";
+    const int NT = 64 * WGM * WGN * WGK;
     if (bf16) {
         body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
         body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
@@ -745,6 +769,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _B, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
         term++;
     }
+    if (WGK > 1) body << "    if (tgemm::tile_reduce_k<CFG>(_acc, _lds))\n";
     body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, [&](int _r, int _c, float _sum) {\n";
     body << digits(GM, "_r", "        ", true) << digits(GN, "_c", "        ", true);
     std::vector<expr> acc_index;

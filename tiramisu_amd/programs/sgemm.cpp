@@ -81,5 +81,6 @@ int main()
     generate(128, 192, 96);
     generate(100, 70, 50);        // ragged: guarded tile edges
     generate(33, 17, 9);
+    generate(64, 256, 512);       // few C tiles, long reduction: wavefront groups split K inside a workgroup
     return 0;
 }
