@@ -130,9 +130,12 @@ __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tm,
 // WGM x WGN wavefronts tile the block in M and N; WGK > 1 adds groups of wavefronts that each take
 // 1/WGK of every K-slice for the same C tile (for problems with too few C tiles to fill the chip);
 // their partial sums are added through LDS by tile_reduce_k before the epilogue.
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_, int PAD_ = 1, int WGK_ = 1>
+// DEPTH is the number of K-slices a thread keeps in flight in registers (1: the next slice only);
+// latency-bound problems (few, short slices per workgroup) ask for all their slices at once.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool A_KMAJOR_, bool B_KMAJOR_, bool EDGE_, int PAD_ = 1, int WGK_ = 1,
+          int DEPTH_ = 1>
 struct config {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, WGK = WGK_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, WGK = WGK_, DEPTH = DEPTH_;
     static constexpr bool A_KMAJOR = A_KMAJOR_, B_KMAJOR = B_KMAJOR_, EDGE = EDGE_;
     static constexpr int NT = 64 * WGM * WGN * WGK;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
@@ -175,7 +178,8 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     const int wm = wmn / CFG::WGN, wn = wmn % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
 
-    f32x4 ra[opA::NV], rb[opB::NV];
+    constexpr int D = CFG::DEPTH;
+    f32x4 ra[D][opA::NV], rb[D][opB::NV];           // slice s travels in slot s % D
     // stage addresses are computed from `lds` (never selected between pointers) so that every
     // access stays an LDS instruction
     auto stage_a = [&](int stage) -> float * { return lds + stage * CFG::STAGE_FLOATS; };
@@ -203,14 +207,16 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     // group barriers below); the steady-state slice is branch-free so that this is one scheduling
     // region, and the last two slices are peeled.
     const int KT = (K + BK - 1) / BK;
-    opA::load_global(A, m0, 0, ra);
-    opB::load_global(B, n0, 0, rb);
-    opA::store_lds(stage_a(0), ra);
-    opB::store_lds(stage_b(0), rb);
-    if (KT > 1) {
-        opA::load_global(A, m0, BK, ra);
-        opB::load_global(B, n0, BK, rb);
-    }
+    opA::load_global(A, m0, 0, ra[0]);
+    opB::load_global(B, n0, 0, rb[0]);
+    opA::store_lds(stage_a(0), ra[0]);
+    opB::store_lds(stage_b(0), rb[0]);
+#pragma unroll
+    for (int s = 1; s <= D; s++)
+        if (s < KT) {
+            opA::load_global(A, m0, s * BK, ra[s % D]);
+            opB::load_global(B, n0, s * BK, rb[s % D]);
+        }
     __syncthreads();
     read_frags(0, 0, 0);
 
@@ -225,19 +231,20 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
     };
     constexpr int MFMAS = 4 * TM * TN;                                   // per fragment set
     constexpr int FRAG_READS = TM + (CFG::B_KMAJOR ? TN : 2 * TN) + (CFG::A_KMAJOR ? 0 : TM);  // LDS read instructions per set (approx.)
-    // one slice; MORE: another slice follows (already in registers); LOAD: a slice after that exists
-    auto slice = [&](int kt, auto more_c, auto load_c) {
+    // one slice; MORE: another slice follows (in register slot `slot`); LOAD: the slice D after that
+    // one exists and takes its place in the slot
+    auto slice = [&](int kt, int slot, auto more_c, auto load_c) {
         constexpr bool MORE = decltype(more_c)::value, LOAD = decltype(load_c)::value;
         const int cur = kt & 1;
 #pragma unroll
         for (int q = 0; q < Q; q++) {
             const int buf = q & 1;
             if (q == 0 && MORE) {
-                opA::store_lds(stage_a(cur ^ 1), ra);
-                opB::store_lds(stage_b(cur ^ 1), rb);
+                opA::store_lds(stage_a(cur ^ 1), ra[slot]);
+                opB::store_lds(stage_b(cur ^ 1), rb[slot]);
                 if (LOAD) {
-                    opA::load_global(A, m0, (kt + 2) * BK, ra);
-                    opB::load_global(B, n0, (kt + 2) * BK, rb);
+                    opA::load_global(A, m0, (kt + 1 + D) * BK, ra[slot]);
+                    opB::load_global(B, n0, (kt + 1 + D) * BK, rb[slot]);
                 }
             }
             if (q + 1 < Q) {
@@ -283,10 +290,24 @@ __device__ __forceinline__ void tile_accumulate(accumulators<CFG> &acc, const SR
             else { if (MFMAS > FRAG_READS) __builtin_amdgcn_sched_group_barrier(0x008, REST_MID, 0); }
         }
     };
-    int kt = 0;
-    for (; kt + 2 < KT; kt++) slice(kt, std::true_type(), std::true_type());
-    if (kt + 1 < KT) { slice(kt, std::true_type(), std::false_type()); kt++; }
-    if (kt < KT) slice(kt, std::false_type(), std::false_type());
+    if (D == 1) {
+        int kt = 0;
+        for (; kt + 2 < KT; kt++) slice(kt, 0, std::true_type(), std::true_type());
+        if (kt + 1 < KT) { slice(kt, 0, std::true_type(), std::false_type()); kt++; }
+        if (kt < KT) slice(kt, 0, std::false_type(), std::false_type());
+    } else {
+        // unrolled by D so that every register slot index is a constant
+        for (int kt0 = 0; kt0 < KT; kt0 += D) {
+#pragma unroll
+            for (int d = 0; d < D; d++) {
+                const int kt = kt0 + d;
+                if (kt >= KT) break;
+                if (kt + 1 + D < KT) slice(kt, (d + 1) % D, std::true_type(), std::true_type());
+                else if (kt + 1 < KT) slice(kt, (d + 1) % D, std::true_type(), std::false_type());
+                else slice(kt, (d + 1) % D, std::false_type(), std::false_type());
+            }
+        }
+    }
     // the next call may overwrite stage 0 while a slow wavefront still multiplies: its fragments are
     // in registers, and the barrier above ordered every LDS read of this call before that
 }

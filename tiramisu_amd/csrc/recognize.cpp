@@ -630,7 +630,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const expr Me = GM.total, Ne = GN.total, Ke = GK.total;
     long Ml = -1, Nl = -1, Kl = -1;
     const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
-    int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2, WGK = 1;
+    int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2, WGK = 1, DEPTH = 1;
     if (lit) {
         if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0) { BM = BN = 256; PADX = 0; }
         else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256 && Ml >= 128) { BM = BN = 128; }
@@ -642,6 +642,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     if (lit && !bf16 && BM == 64 && BN == 64 && Ml <= 64 && ((Nl + 63) / 64) <= 64 && Nl % 32 == 0 && Kl % 128 == 0 && Kl >= 256 &&
         !std::getenv("TIRAMISU_MFMA_NO_SPLITK")) {
         BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
+        DEPTH = (int)std::min<long>(4, std::max<long>(1, Kl / BK - 1));   // latency-bound: ask for (up to) all slices at once
     }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
     if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
@@ -707,7 +708,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     std::ostringstream pre, body;
     const std::string cfg = "tgemm::config<" + std::to_string(BM) + ", " + std::to_string(BN) + ", " + std::to_string(BK) + ", " +
                             std::to_string(WGM) + ", " + std::to_string(WGN) + ", " + (operands[0].first.kmajor ? "true" : "false") + ", " +
-                            (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ", " + std::to_string(WGK) + ">";
+                            (operands[0].second.kmajor ? "true" : "false") + ", " + (edge ? "true" : "false") + ", " + std::to_string(PADX) + ", " + std::to_string(WGK) + ", " + std::to_string(DEPTH) + ">";
     const int NT = 64 * WGM * WGN * WGK;
     if (bf16) {
         body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
