@@ -720,7 +720,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     body << "    const int _M = " << dev.print(Me) << ", _N = " << dev.print(Ne) << ", _K = " << dev.print(Ke) << ";\n";
     body << "    int _tm, _tn;\n    tgemm::tile_of_block((_M + CFG::BM - 1) / CFG::BM, (_N + CFG::BN - 1) / CFG::BN, _tm, _tn);\n";
     body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
-    int term = 0;
+    int term = 0, ktab_words = 0;
     const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
     for (auto &o : operands) {
         body << "    {\n";
@@ -747,13 +747,33 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
             } else {
                 // gather source: offsets are separable sums over the digits of the row and k indices
                 const std::string sname = kname + "_src" + std::to_string(term) + (which == 0 ? "a" : "b");
-                pre << "struct " << sname << " {\n    const float *__restrict__ base;\n    int XE, KE;\n";
-                pre << "    __device__ __forceinline__ long offset(int _x, int _k) const {\n";
-                pre << digits(rowg, "_x", "        ", false) << digits(GK, "_k", "        ", false);
-                pre << "        return 0";
-                for (const group_info *gg : std::vector<const group_info *>{&rowg, &GK})
-                    for (int p : gg->dims) pre << " + (long)" << U.dims[p].kvar << " * " << dev.print(g->coef.at(p));
+                // 32-bit offsets when the buffer is small enough
+                bool small = g->buf->has_constant_extents();
+                if (small) {
+                    double cnt = 1;
+                    for (auto &d : g->buf->get_dim_sizes()) cnt *= (double)lir::simplify(d).get_int_val();
+                    small = cnt < 2147483648.0;
+                }
+                const std::string OT = small ? "int32_t" : "long";
+                // the k part of the offset (divisions by the extents of the reduction dimensions) is
+                // tabulated in LDS once per workgroup when the table is small: one LDS read per load
+                // instead of the digit arithmetic
+                const bool tabulate = small && lit && Kl * 4 <= 32768 && ktab_words == 0 && !std::getenv("TIRAMISU_MFMA_NO_KTAB");
+                pre << "struct " << sname << " {\n    const float *__restrict__ base;\n    int XE, KE;\n    const int32_t *ktab;\n";
+                pre << "    static __device__ __forceinline__ " << OT << " koff(int _k) {\n" << digits(GK, "_k", "        ", false) << "        return 0";
+                for (int p : GK.dims) pre << " + (" << OT << ")" << U.dims[p].kvar << " * " << dev.print(g->coef.at(p));
                 pre << ";\n    }\n";
+                pre << "    __device__ __forceinline__ " << OT << " offset(int _x, int _k) const {\n";
+                pre << digits(rowg, "_x", "        ", false);
+                pre << "        return " << (tabulate ? "ktab[_k]" : "koff(_k)");
+                for (int p : rowg.dims) pre << " + (" << OT << ")" << U.dims[p].kvar << " * " << dev.print(g->coef.at(p));
+                pre << ";\n    }\n";
+                if (tabulate) {
+                    ktab_words = (int)((Kl + 3) / 4 * 4);
+                    body << "        int32_t *_ktab = reinterpret_cast<int32_t *>(_lds) + CFG::LDS_BYTES / 4;\n";
+                    body << "        for (int _k = threadIdx.x; _k < _K; _k += CFG::NT) _ktab[_k] = " << sname << "::koff(_k);\n";
+                    body << "        __syncthreads();\n";
+                }
                 pre << "    __device__ __forceinline__ tgemm::f32x4 load4(int x, int k) const {\n";
                 const char *full = g->gather_kdir ? "(x < XE && k + 3 < KE)" : "(k < KE && x + 3 < XE)";
                 if (g->gather_vec)
@@ -763,7 +783,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
                 pre << "        for (int e = 0; e < 4; e++) {\n            const int xx = " << (g->kmajor ? "x" : "x + e") << ", kk = " << (g->kmajor ? "k + e" : "k")
                     << ";\n            if (xx < XE && kk < KE) r[e] = base[offset(xx, kk)];\n        }\n        return r;\n    }\n};\n";
                 body << "        const " << sname << " " << nm << "{" << g->buf->get_name() << " + (" << dev.print(g->base) << "), " << (which == 0 ? "_M" : "_N")
-                     << ", _K};\n";
+                     << ", _K, " << (tabulate ? "_ktab" : "nullptr") << "};\n";
             }
             which++;
         }
@@ -838,6 +858,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         const int rowB = operands[0].second.kmajor ? (BK / 4) * (BN + PADX) * 4 : BK * BN;
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
         if (bf16) k.lds_bytes = std::to_string(2 * (BK / 8) * (BM + BN) * 4 * 4);
+        else if (ktab_words) k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4 + ktab_words * 4);
     }
     std::ostringstream src;
     src << pre.str();
