@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|heat2d|sgemm1024|sgemm4096|...]
 
-Prints ONE JSON line.  The headline is BASELINE config 2 (heat2d 8192x8192, 32 time steps,
+Prints ONE JSON line.  The headline is benchmark configuration 2 (heat2d 8192x8192, 32 time steps,
 the configuration the HBM-roofline target is quoted on): `value` is algorithmic HBM GB/s of the
 whole compiled Tiramisu function with its buffers already resident in HBM.  A "step" is one
 call of the compiled function (32 stencil time steps).  The other configurations that exist
@@ -308,12 +308,12 @@ def main():
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if head_name == "sgemm4096_bf16" else "f32", "warmup_extra_steps": head.get("warmup_extra_steps", 0),
         "data": "synthetic (seeded uniform inputs, already resident in HBM)",
-        "config": {"workload": {"heat2d": "heat2d 5-point stencil, fp32 grid 8192x8192, 32 time steps (BASELINE configs[1])",
-                                "sgemm1024": "sgemm fp32 1024^3 (BASELINE configs[0])",
-                                "sgemm4096": "sgemm fp32 4096^3 (BASELINE configs[2])",
-                                "sgemm4096_bf16": "sgemm bf16-in/fp32-acc 4096^3 (BASELINE configs[2], bf16 variant)",
-                                "conv2d": "conv2d+bias+ReLU N32 C64->64 112x112 3x3 (BASELINE configs[3])",
-                                "lstm": "4-layer LSTM B64 H512 S100 (BASELINE configs[4])"}.get(head_name, head_name)},
+        "config": {"workload": {"heat2d": "heat2d 5-point stencil, fp32 grid 8192x8192, 32 time steps (benchmark configs[1])",
+                                "sgemm1024": "sgemm fp32 1024^3 (benchmark configs[0])",
+                                "sgemm4096": "sgemm fp32 4096^3 (benchmark configs[2])",
+                                "sgemm4096_bf16": "sgemm bf16-in/fp32-acc 4096^3 (benchmark configs[2], bf16 variant)",
+                                "conv2d": "conv2d+bias+ReLU N32 C64->64 112x112 3x3 (benchmark configs[3])",
+                                "lstm": "4-layer LSTM B64 H512 S100 (benchmark configs[4])"}.get(head_name, head_name)},
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
         "workloads": {k: v for k, v in results.items() if k != head_name},

@@ -73,7 +73,7 @@ def heat2d(grid, steps, boundary_other=None):
     ping-pong planes; returns both planes as the un-tiled program leaves them (plane t % 2 holds
     step t).  Association and rounding follow the program text in tiramisu_amd/programs/heat2d.cpp
     -- ((((c+n)+s)+w)+e)*0.2f in fp32 -- which is the 5-point form of the reference's
-    benchmarks/halide/heat2d_tiramisu.cpp:52-86 with BASELINE's coefficients, iterated in time like
+    benchmarks/halide/heat2d_tiramisu.cpp:52-86 with the benchmark configuration's coefficients, iterated in time like
     benchmarks/halide/heat3d_tiramisu.cpp:27-45.  `boundary_other` is the initial content of
     plane 1 (its boundary cells are read by even steps); zeros if omitted."""
     g = grid.astype(np.float32)

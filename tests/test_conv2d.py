@@ -1,4 +1,4 @@
-"""conv2d + bias + ReLU (BASELINE config 4): oracle pins, CPU-generated code vs the oracle, and
+"""conv2d + bias + ReLU (benchmark configuration 4): oracle pins, CPU-generated code vs the oracle, and
 the implicit-GEMM MFMA kernel vs both.
 
 Tolerance: bit-exact for integer-valued data; for uniform data max |gpu - ref| <= 1e-4 * max |ref|

@@ -1,4 +1,4 @@
-"""heat2d (BASELINE config 2): oracle pins, CPU-generated code vs the oracle, and the time-tiled
+"""heat2d (benchmark configuration 2): oracle pins, CPU-generated code vs the oracle, and the time-tiled
 HIP stencil kernel vs both -- bit for bit (the sweep has no reassociation freedom: every cell
 is the same five fp32 additions and one multiplication on every path)."""
 import ctypes
@@ -105,7 +105,7 @@ def test_gpu_boundaries_of_both_planes_are_respected():
 
 @pytest.mark.gpu
 def test_gpu_full_size_matches_cpu_generated_code():
-    # BASELINE size: 8192 x 8192, 32 steps; the CPU-generated code (parallelize y, vectorize x)
+    # benchmark size: 8192 x 8192, 32 steps; the CPU-generated code (parallelize y, vectorize x)
     # is the checker.  Both planes are compared.
     n, steps = 8192, 32
     g = initial_grid(n, 8192)

@@ -1,4 +1,4 @@
-"""Stacked LSTM (BASELINE config 5): oracle pins, CPU-generated code vs the oracle, and the GPU
+"""Stacked LSTM (benchmark configuration 5): oracle pins, CPU-generated code vs the oracle, and the GPU
 program (MFMA gate GEMMs + fused element-wise kernel per cell) vs both.
 
 Tolerance: max |gpu - ref| <= 1e-4 * max |ref| on the output sequence y (fp32; the MFMA kernel

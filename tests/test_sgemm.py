@@ -1,4 +1,4 @@
-"""sgemm (BASELINE configs 1 and 3): CPU-generated code vs the numpy restatement, and the MFMA
+"""sgemm (benchmark configurations 1 and 3): CPU-generated code vs the numpy restatement, and the MFMA
 contraction kernel vs both.
 
 Tolerances (from the parity statement): bit-exact when inputs are small integers (every partial

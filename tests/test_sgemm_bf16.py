@@ -1,4 +1,4 @@
-"""bf16-input / fp32-accumulate sgemm (the bf16 variant of BASELINE config 3).
+"""bf16-input / fp32-accumulate sgemm (the bf16 variant of benchmark configuration 3).
 
 The reference has no bf16 type, so the oracle is the fp32 result on bf16-rounded inputs
 (round to nearest even), as computed by the CPU-generated code of the same program and by
