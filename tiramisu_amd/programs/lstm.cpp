@@ -8,11 +8,18 @@
 // structure (merged 4H gate rows, h/c buffers indexed [m+1][l+1]) is that of
 // benchmarks/DNN/blocks/LSTM/cpu/generator.cpp:31-60, and sigmoid is 1 / (1 + exp(-x)) (:43).
 //
-// GPU schedule: time steps and layers are host loops; per cell, the bias initialisation and the
-// two-product reduction are fused in one nest (proved a contraction -> one MFMA kernel with
-// K = 2H split over the two weight matrices), and the nine element-wise computations are fused
-// in a second nest (one kernel).  All tensors are GPU-resident.
-// CPU schedule (-DTIRAMISU_TARGET_CPU): the reference's unscheduled program
+// The input half of the gates does not depend on the recurrence, so it is computed for all time
+// steps of a layer at once (gin = bias + W * h_below, one contraction with M = S*B rows), as the
+// reference's library variant does for batches of time steps (gpu_lib/generator.cpp, GEMM_BATCH);
+// the recurrent half then starts from it: gates(m) = gin(m) + R * h(m-1).
+//
+// GPU schedule: layers and time steps are host loops (layer outermost); per layer one MFMA kernel
+// for gin (the bias initialisation fused in, time mapped to workgroups); per cell the copy of gin
+// and the recurrent reduction are fused in one nest (a contraction with K = H), and the nine
+// element-wise computations are fused in a second nest (one kernel).  All tensors are GPU-resident;
+// h is laid out [layer][time][batch][hidden] so that the rows of the layer-wide contraction are
+// contiguous.
+// CPU schedule (-DTIRAMISU_TARGET_CPU): the same computations in the reference's unscheduled order
 // (cpu/generator.cpp:59-75) with the batch loop parallelized.
 // One generated function per shape: lstm_<L>x<B>x<H>x<S>.
 #include <tiramisu/tiramisu.h>
@@ -32,43 +39,49 @@ static void generate(int L, int B, int H, int S)
     buffer buf_biases("buf_biases", {L, 4 * H}, p_float32, a_input);
     buffer buf_x("buf_x", {S, B, H}, p_float32, a_input);
     buffer buf_y("buf_y", {S, B, H}, p_float32, a_output);
+    buffer buf_gin("buf_gin", {S, B, 4 * H}, p_float32, a_temporary);
     buffer buf_gates("buf_gates", {B, 4 * H}, p_float32, a_temporary);
     buffer buf_i("buf_i", {B, H}, p_float32, a_temporary);
     buffer buf_f("buf_f", {B, H}, p_float32, a_temporary);
     buffer buf_z("buf_z", {B, H}, p_float32, a_temporary);
     buffer buf_o("buf_o", {B, H}, p_float32, a_temporary);
-    buffer buf_h("buf_h", {S + 1, L + 1, B, H}, p_float32, a_temporary);
-    buffer buf_c("buf_c", {S + 1, L, B, H}, p_float32, a_temporary);
+    buffer buf_h("buf_h", {L + 1, S + 1, B, H}, p_float32, a_temporary);
+    buffer buf_c("buf_c", {L, S + 1, B, H}, p_float32, a_temporary);
 
     input W("W", {l, g, j}, p_float32);
     input R("R", {l, g, j}, p_float32);
     input bias("bias", {l, g}, p_float32);
     input x("x", {m, k, i}, p_float32);
 
-    computation h("h", {m, l, k, i}, p_float32);
-    computation c("c", {m, l, k, i}, p_float32);
+    computation h("h", {l, m, k, i}, p_float32);
+    computation c("c", {l, m, k, i}, p_float32);
     computation h_init("h_init", {l, k, i}, expr((float)0));
     computation c_init("c_init", {l, k, i}, expr((float)0));
     computation h_copy_x("h_copy_x", {m, k, i}, x(m, k, i));
-    computation gates_init("gates_init", {m, l, k, g}, bias(l, g));
-    computation gates("gates", {m, l, k, g, j}, p_float32);
-    gates.set_expression(gates(m, l, k, g, 0) + W(l, g, j) * h(m, l - 1, k, j) + R(l, g, j) * h(m - 1, l, k, j));
-    computation sig_i("sig_i", {m, l, k, i}, sigmoid(gates(m, l, k, i, 0)));
-    computation sig_f("sig_f", {m, l, k, i}, sigmoid(gates(m, l, k, i + H, 0)));
-    computation tnh_z("tnh_z", {m, l, k, i}, expr(o_tanh, gates(m, l, k, i + 2 * H, 0)));
-    computation sig_o("sig_o", {m, l, k, i}, sigmoid(gates(m, l, k, i + 3 * H, 0)));
-    computation mul_iz("mul_iz", {m, l, k, i}, sig_i(m, l, k, i) * tnh_z(m, l, k, i));
-    computation mul_fc("mul_fc", {m, l, k, i}, sig_f(m, l, k, i) * c(m - 1, l, k, i));
-    c.set_expression(mul_iz(m, l, k, i) + mul_fc(m, l, k, i));
-    computation tnh_c("tnh_c", {m, l, k, i}, expr(o_tanh, c(m, l, k, i)));
-    h.set_expression(tnh_c(m, l, k, i) * sig_o(m, l, k, i));
-    computation y("y", {m, k, i}, h(m, L - 1, k, i));
+    computation gin_init("gin_init", {l, m, k, g}, bias(l, g));
+    computation gin("gin", {l, m, k, g, j}, p_float32);
+    gin.set_expression(gin(l, m, k, g, 0) + W(l, g, j) * h(l - 1, m, k, j));
+    computation gates_init("gates_init", {l, m, k, g}, gin(l, m, k, g, 0));
+    computation gates("gates", {l, m, k, g, j}, p_float32);
+    gates.set_expression(gates(l, m, k, g, 0) + R(l, g, j) * h(l, m - 1, k, j));
+    computation sig_i("sig_i", {l, m, k, i}, sigmoid(gates(l, m, k, i, 0)));
+    computation sig_f("sig_f", {l, m, k, i}, sigmoid(gates(l, m, k, i + H, 0)));
+    computation tnh_z("tnh_z", {l, m, k, i}, expr(o_tanh, gates(l, m, k, i + 2 * H, 0)));
+    computation sig_o("sig_o", {l, m, k, i}, sigmoid(gates(l, m, k, i + 3 * H, 0)));
+    computation mul_iz("mul_iz", {l, m, k, i}, sig_i(l, m, k, i) * tnh_z(l, m, k, i));
+    computation mul_fc("mul_fc", {l, m, k, i}, sig_f(l, m, k, i) * c(l, m - 1, k, i));
+    c.set_expression(mul_iz(l, m, k, i) + mul_fc(l, m, k, i));
+    computation tnh_c("tnh_c", {l, m, k, i}, expr(o_tanh, c(l, m, k, i)));
+    h.set_expression(tnh_c(l, m, k, i) * sig_o(l, m, k, i));
+    computation y("y", {m, k, i}, h(L - 1, m, k, i));
 
     W.store_in(&buf_weights, {l, 0, g, j});
     R.store_in(&buf_weights, {l, 1, g, j});
     bias.store_in(&buf_biases, {l, g});
     x.store_in(&buf_x);
     y.store_in(&buf_y);
+    gin_init.store_in(&buf_gin, {m, k, g});
+    gin.store_in(&buf_gin, {m, k, g});
     gates_init.store_in(&buf_gates, {k, g});
     gates.store_in(&buf_gates, {k, g});
     sig_i.store_in(&buf_i, {k, i});
@@ -78,43 +91,53 @@ static void generate(int L, int B, int H, int S)
     mul_iz.store_in(&buf_i, {k, i});
     mul_fc.store_in(&buf_f, {k, i});
     tnh_c.store_in(&buf_i, {k, i});
-    h.store_in(&buf_h, {m + 1, l + 1, k, i});
-    c.store_in(&buf_c, {m + 1, l, k, i});
-    h_init.store_in(&buf_h, {0, l + 1, k, i});
-    c_init.store_in(&buf_c, {0, l, k, i});
-    h_copy_x.store_in(&buf_h, {m + 1, 0, k, i});
+    h.store_in(&buf_h, {l + 1, m + 1, k, i});
+    c.store_in(&buf_c, {l, m + 1, k, i});
+    h_init.store_in(&buf_h, {l + 1, 0, k, i});
+    c_init.store_in(&buf_c, {l, 0, k, i});
+    h_copy_x.store_in(&buf_h, {0, m + 1, k, i});
 
 #ifdef TIRAMISU_TARGET_CPU
-    for (computation *q : {&gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
+    for (computation *q : {&gin_init, &gin, &gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
         q->parallelize(k);
     h_init.then(c_init, computation::root)
           .then(h_copy_x, computation::root)
-          .then(gates_init, computation::root)
-          .then(gates, l)
-          .then(sig_i, l)
-          .then(sig_f, l)
-          .then(tnh_z, l)
-          .then(sig_o, l)
-          .then(mul_iz, l)
-          .then(mul_fc, l)
-          .then(c, l)
-          .then(tnh_c, l)
-          .then(h, l)
+          .then(gin_init, computation::root)
+          .then(gin, l)
+          .then(gates_init, l)
+          .then(gates, m)
+          .then(sig_i, m)
+          .then(sig_f, m)
+          .then(tnh_z, m)
+          .then(sig_o, m)
+          .then(mul_iz, m)
+          .then(mul_fc, m)
+          .then(c, m)
+          .then(tnh_c, m)
+          .then(h, m)
           .then(y, computation::root);
     tiramisu::codegen({&buf_weights, &buf_biases, &buf_x, &buf_y}, "build/" + name + "_cpu.o", false);
 #else
-    for (buffer *q : {&buf_weights, &buf_biases, &buf_x, &buf_y, &buf_gates, &buf_i, &buf_f, &buf_z, &buf_o, &buf_h, &buf_c})
+    for (buffer *q : {&buf_weights, &buf_biases, &buf_x, &buf_y, &buf_gin, &buf_gates, &buf_i, &buf_f, &buf_z, &buf_o, &buf_h, &buf_c})
         q->tag_gpu_global();
     var kb("kb"), kt("kt"), ib("ib"), it("it"), gb("gb"), gt("gt");
     for (computation *q : {&h_init, &c_init, &h_copy_x, &y, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
         q->gpu_tile(k, i, 16, 16, kb, ib, kt, it);
+    // the layer-wide contraction: loops l | m kb gb | kt gt | j, time and the tile loops on workgroups
+    for (computation *q : {&gin_init, &gin}) {
+        q->tile(k, g, 16, 16, kb, gb, kt, gt);
+        q->tag_gpu_block_level(1, 2, 3);
+        q->tag_gpu_thread_level(4, 5);
+    }
     gates_init.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
     gates.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
     h_init.then(c_init, computation::root)
           .then(h_copy_x, computation::root)
-          .then(gates_init, computation::root)
+          .then(gin_init, computation::root)
+          .then(gin, gt)
+          .then(gates_init, l)
           .then(gates, gt)
-          .then(sig_i, l)
+          .then(sig_i, m)
           .then(sig_f, it)
           .then(tnh_z, it)
           .then(sig_o, it)
