@@ -33,10 +33,10 @@ PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
 # HBM bytes per launch of the dominant heat2d kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); see profiles/.
-HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # by time steps per launch; KiB counters x calibration factor
-    7: (180694.2 * 2.000 + 262333.1 * 1.000) * 1024,
-    3: (150888.7 * 2.000 + 264412.5 * 1.000) * 1024,
-    1: (137641.8 * 2.000 + 265178.7 * 1.000) * 1024,
+HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # interior-tile kernel, by time steps per launch; KiB counters x calibration factor
+    7: (128858.1 * 2.000 + 250674.5 * 1.000) * 1024,
+    3: (127622.7 * 2.000 + 252906.8 * 1.000) * 1024,
+    1: (127512.8 * 2.000 + 254771.8 * 1.000) * 1024,
 }
 
 
@@ -100,12 +100,20 @@ def cpu_threads():
 
 # ---------------------------------------------------------------- workloads
 
-def stencil_steps_per_launch(kernel_source):
-    """{kernel name: time steps fused in one launch}, read from the emitted kernel source."""
+def stencil_kernels(kernel_source, domain_cells):
+    """{kernel name: (time steps fused in one launch, cells advanced per launch)}, read from the
+    emitter's description of each kernel in the generated kernel source: the kernel for interior
+    tiles advances tiles x tile extent cells, its companion the rest of the iteration domain."""
     import re
     text = open(kernel_source).read()
-    return {m.group(1): int(m.group(2))
-            for m in re.finditer(r"#define ST_NAME (\w+)\n(?:#define (?!ST_R )\w+ .*\n)*#define ST_R (\d+)", text)}
+    out = {}
+    for m in re.finditer(r"// (\w+): stencil: (\d+) time step\(s\) per launch, radius \d+, tile (\d+)x(\d+) in registers, "
+                         r".*?, (\d+) interior tiles", text):
+        out[m.group(1)] = (int(m.group(2)), int(m.group(3)) * int(m.group(4)) * int(m.group(5)))
+    for m in re.finditer(r"// (\w+): stencil: the \d+ tiles of (\w+)'s launch", text):
+        steps, cells = out[m.group(2)]
+        out[m.group(1)] = (steps, domain_cells - cells)
+    return out
 
 
 def bench_heat2d(steps, warmup, with_cpu):
@@ -124,15 +132,16 @@ def bench_heat2d(steps, warmup, with_cpu):
     prof = kernel_profile(lambda: prog(buf), steps)
     # dominant kernel: the one with the largest total time per call
     dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
-    fused_steps = stencil_steps_per_launch(os.path.join(PROGRAMS, "build", name + ".o.hip"))[dom[0]]
-    per_launch_bytes = fused_steps * 2.0 * n * n * 4
+    # algorithmic bytes of one launch: every cell the kernel advances is read once and written once per step
+    fused_steps, cells = stencil_kernels(os.path.join(PROGRAMS, "build", name + ".o.hip"), (n - 2) * (n - 2))[dom[0]]
+    per_launch_bytes = fused_steps * 2.0 * cells * 4
     achieved = per_launch_bytes / (dom[1][0] * 1e-3) / 1e9
     out = {
         "value": alg_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": HEAT2D_TRAFFIC_BYTES_PER_LAUNCH.get(fused_steps),
                      "kernel": dom[0], "kernel_ms": dom[1][0], "launches_per_step": dom[1][1],
-                     "time_steps_per_launch": fused_steps},
+                     "time_steps_per_launch": fused_steps, "cells_per_launch": cells},
         "kernels": {k: {"ms": v[0], "launches_per_step": v[1]} for k, v in prof.items()},
     }
     if with_cpu:

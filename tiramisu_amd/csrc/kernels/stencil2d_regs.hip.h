@@ -18,11 +18,14 @@
 // the shrinking valid part are computed from stale data and never used.
 //
 // Cells outside the iteration domain (the fixed boundary) are never written.  When a step needs
-// their value it takes the one their plane holds at that step's parity, read from global memory
-// (no launch ever writes those cells), so the two planes may hold different boundary values,
-// exactly as in the un-tiled program.  Only workgroups whose region touches the boundary run
-// that path; the choice is uniform over the workgroup.  Reading plane `src` and writing plane
-// `1-src` requires ST_R to be odd; the host code composes the time loop from odd chunks.
+// their value it takes the one their plane holds at that step's parity, so the two planes may hold
+// different boundary values, exactly as in the un-tiled program: a thread whose strip contains
+// fixed cells keeps the other plane's values of its strip in registers (read once; no launch ever
+// writes those cells) and swaps the two values of a fixed cell at every step.  That costs registers
+// and checks, so each launch is split in two kernels: ST_NAME for the tiles whose staged region
+// lies inside the iteration domain (no checks at all), ST_NAME_EDGE for the others.  Both read
+// plane `src` and write plane `1-src` (disjoint cells), which requires ST_R to be odd; the host
+// code composes the time loop from odd chunks.
 //
 // Macros supplied by the emitter before this file is included:
 //   ST_NAME            kernel name
@@ -33,6 +36,11 @@
 //   ST_W               wavefronts per workgroup
 //   ST_RPT             rows per thread
 //   ST_EXPR            expression of the new value in terms of ST_AT(dy, dx)
+//   ST_NAME_EDGE       name of the kernel for the tiles that touch the fixed boundary
+//   ST_GX, ST_GY       number of tiles along x and y
+//   ST_IBX0, ST_IBX1, ST_IBY0, ST_IBY1   inclusive ranges of interior tiles (ST_IBY0 = ST_GY and
+//                      ST_IBY1 = ST_GY - 1 when there is none); launch ST_NAME with one workgroup
+//                      per interior tile and ST_NAME_EDGE with one per remaining tile
 // The tile extents follow: ST_TH = ST_W*ST_RPT - 2*ST_R*ST_RAD, ST_TW = 256 - 2*roundup4(ST_R*ST_RAD).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -96,9 +104,12 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     const int gx = bx * ST_TW - ST_HX + 4 * lane;         // plane column of my quads
     const int wave_up = wave > 0 ? wave - 1 : 0, wave_dn = wave < ST_W - 1 ? wave + 1 : ST_W - 1;
 
-    st_f4 cur[ST_RPT];
+    st_f4 cur[ST_RPT], other[EDGE ? ST_RPT : 1];   // other: the other plane's values (fixed cells only)
 #pragma unroll
-    for (int r = 0; r < ST_RPT; r++) cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
+    for (int r = 0; r < ST_RPT; r++) {
+        cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
+        if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(dst, gy0 + r, gx);
+    }
 
     // xch[parity][wave][top|bottom][row][lane]
     auto slot = [&](int parity, int w, int side, int i) -> st_f4 * {
@@ -147,21 +158,18 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
                     w[dy + ST_RAD][ST_RAD + 4 + i] = rt[j][i];
                 }
             }
-            st_f4 fixed = {0.f, 0.f, 0.f, 0.f};
-            bool row_in = true;
-            if (EDGE) {
-                // a fixed cell shows the value of the plane that step s lives in
-                fixed = st_load_quad<true, ST_NY, ST_NX>(parity ? dst : src, gy0 + r, gx);
-                row_in = gy0 + r >= ST_Y0 && gy0 + r <= ST_Y1;
-            }
+            const bool row_in = !EDGE || (gy0 + r >= ST_Y0 && gy0 + r <= ST_Y1);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
 #define ST_AT(dy, dx) w[(dy) + ST_RAD][e + (dx) + ST_RAD]
                 const float computed = (ST_EXPR);
 #undef ST_AT
                 if (EDGE) {
+                    // a fixed cell shows the value of the plane that step s lives in: swap
                     const bool in_dom = row_in && gx + e >= ST_X0 && gx + e <= ST_X1;
-                    cur[r][e] = in_dom ? computed : fixed[e];
+                    const float before = ext[ST_RAD + r][e], there = other[r][e];
+                    cur[r][e] = in_dom ? computed : there;
+                    other[r][e] = in_dom ? there : before;
                 } else {
                     cur[r][e] = computed;
                 }
@@ -187,6 +195,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     }
 }
 
+// Interior tiles: one workgroup per tile of the rectangle [ST_IBX0, ST_IBX1] x [ST_IBY0, ST_IBY1].
 extern "C" __global__ void __launch_bounds__(64 * ST_W)
 #if ST_OCC > 0
 __attribute__((amdgpu_waves_per_eu(ST_OCC)))
@@ -200,19 +209,42 @@ ST_NAME(float *__restrict__ planes, const int src_plane)
     float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a band
     // of consecutive tiles (row-major), so that tiles running together share their halos in L2.
-    const int nb = gridDim.x * gridDim.y, b = blockIdx.y * gridDim.x + blockIdx.x;
+    constexpr int IW = ST_IBX1 - ST_IBX0 + 1;
+    const int nb = gridDim.x, b = blockIdx.x;
 #if ST_XCD
     const int xcd = b % 8, per = nb / 8, extra = nb % 8;
     const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / 8;
 #else
     const int tile = b;
 #endif
-    const int bx = tile % gridDim.x, by = tile / gridDim.x;
-    const int ty0 = by * ST_TH - ST_HY, tx0 = bx * ST_TW - ST_HX;
-    // does the staged region lie inside the iteration domain?
-    const bool interior = ty0 >= ST_Y0 && ty0 + ST_LH - 1 <= ST_Y1 && tx0 >= ST_X0 && tx0 + ST_LW - 1 <= ST_X1;
-    if (interior) ST_CAT(ST_NAME, _sweep)<false>(src, dst, xch, bx, by);
-    else ST_CAT(ST_NAME, _sweep)<true>(src, dst, xch, bx, by);
+    ST_CAT(ST_NAME, _sweep)<false>(src, dst, xch, ST_IBX0 + tile % IW, ST_IBY0 + tile / IW);
+}
+
+// The other tiles, in the order: full tile rows above the interior rectangle, full rows below it,
+// then the tiles left and right of it row by row.
+extern "C" __global__ void __launch_bounds__(64 * ST_W)
+ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
+{
+    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
+    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
+    constexpr int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
+    constexpr int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
+    int e = blockIdx.x, bx, by;
+    if (e < TOP) {
+        by = e / ST_GX;
+        bx = e % ST_GX;
+    } else if (e < TOP + BOTTOM) {
+        e -= TOP;
+        by = ST_IBY1 + 1 + e / ST_GX;
+        bx = e % ST_GX;
+    } else {
+        e -= TOP + BOTTOM;
+        const int c = e % (SIDE > 0 ? SIDE : 1);
+        by = ST_IBY0 + e / (SIDE > 0 ? SIDE : 1);
+        bx = c < ST_IBX0 ? c : ST_IBX1 + 1 + (c - ST_IBX0);
+    }
+    ST_CAT(ST_NAME, _sweep)<true>(src, dst, xch, bx, by);
 }
 
 #undef ST_HY

@@ -203,36 +203,56 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     dev.fct = f;
     dev.device = true;
     const std::string point_text = dev.print(point);
-    std::map<int, kernel> by_steps;
+    std::map<int, std::pair<kernel, kernel>> by_steps;   // (interior tiles, tiles on the fixed boundary)
     std::ostringstream host;
+    auto ceil_div = [](long a, long b) { return a >= 0 ? (a + b - 1) / b : -((-a) / b); };
+    auto floor_div = [](long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); };
     for (auto &ch : chunks) {
         if (!by_steps.count(ch.second)) {
-            kernel k;
+            kernel k, ke;
             k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
+            ke.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
             const int HY = ch.second * radius, HX = (ch.second * radius + 3) / 4 * 4;
             const int TH = LH - 2 * HY, TW = LW - 2 * HX;
+            const long GX = (NX + TW - 1) / TW, GY = (NY + TH - 1) / TH;
+            // tiles whose staged region [b*T - H, b*T - H + L) lies inside the iteration domain
+            long bx0 = std::max<long>(0, ceil_div(lo[2] + HX, TW)), bx1 = std::min<long>(GX - 1, floor_div(hi[2] - LW + 1 + HX, TW));
+            long by0 = std::max<long>(0, ceil_div(lo[1] + HY, TH)), by1 = std::min<long>(GY - 1, floor_div(hi[1] - LH + 1 + HY, TH));
+            if (bx0 > bx1 || by0 > by1) { by0 = GY; by1 = GY - 1; bx0 = 0; bx1 = GX - 1; }   // no interior tile
+            const long interior = (bx1 - bx0 + 1) * (by1 - by0 + 1), edge_tiles = GX * GY - interior;
             k.how = "stencil: " + std::to_string(ch.second) + " time step(s) per launch, radius " + std::to_string(radius) +
                     ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + " in registers, " + std::to_string(WAVES) +
-                    " wavefronts x " + std::to_string(ROWS) + " rows";
+                    " wavefronts x " + std::to_string(ROWS) + " rows, " + std::to_string(interior) + " interior tiles";
+            ke.how = "stencil: the " + std::to_string(edge_tiles) + " tiles of " + k.name + "'s launch that touch the fixed boundary";
             std::ostringstream s;
-            s << "#define ST_NAME " << k.name << "\n#define ST_NY " << NY << "\n#define ST_NX " << NX << "\n#define ST_Y0 " << lo[1]
-              << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2] << "\n#define ST_W " << WAVES
-              << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0) << "\n#define ST_RPT " << ROWS << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius
+            s << "#define ST_NAME " << k.name << "\n#define ST_NAME_EDGE " << ke.name << "\n#define ST_NY " << NY << "\n#define ST_NX " << NX
+              << "\n#define ST_Y0 " << lo[1] << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2]
+              << "\n#define ST_GX " << GX << "\n#define ST_GY " << GY << "\n#define ST_IBX0 " << bx0 << "\n#define ST_IBX1 " << bx1
+              << "\n#define ST_IBY0 " << by0 << "\n#define ST_IBY1 " << by1 << "\n#define ST_W " << WAVES
+              << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0)
+              << "\n#define ST_RPT " << ROWS << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius
               << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
-              << "#undef ST_NAME\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n#undef ST_W\n#undef ST_OCC\n#undef ST_XCD\n"
-              << "#undef ST_RPT\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
-            k.source = s.str();
-            k.params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}};
-            k.grid[0] = std::to_string((NX + TW - 1) / TW);
-            k.grid[1] = std::to_string((NY + TH - 1) / TH);
-            k.block[0] = std::to_string(64 * WAVES);
-            by_steps[ch.second] = k;
+              << "#undef ST_NAME\n#undef ST_NAME_EDGE\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n"
+              << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n"
+              << "#undef ST_XCD\n#undef ST_RPT\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
+            k.source = s.str();            // both kernels come from the one inclusion
+            ke.source = "";
+            for (kernel *q : {&k, &ke}) {
+                q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}};
+                q->block[0] = std::to_string(64 * WAVES);
+            }
+            k.grid[0] = std::to_string(interior);
+            ke.grid[0] = std::to_string(edge_tiles);
+            by_steps[ch.second] = {k, ke};
         }
         const long src = (((ch.first - 1) % 2) + 2) % 2;
-        host << "    {\n        const int32_t _st_src = " << src << ";  // steps " << ch.first << ".." << ch.first + ch.second - 1 << "\n"
-             << launch_text(by_steps[ch.second], "        ") << "    }\n";
+        auto &pr = by_steps[ch.second];
+        host << "    {\n        const int32_t _st_src = " << src << ";  // steps " << ch.first << ".." << ch.first + ch.second - 1 << "\n";
+        if (pr.first.grid[0] != "0") host << launch_text(pr.first, "        ");
+        if (pr.second.grid[0] != "0") host << launch_text(pr.second, "        ");
+        host << "    }\n";
     }
-    for (auto &kv : by_steps) plan.kernels.push_back(kv.second);
+    for (auto &kv : by_steps) { plan.kernels.push_back(kv.second.first); plan.kernels.push_back(kv.second.second); }
     plan.host_code = host.str();
     return true;
 }
