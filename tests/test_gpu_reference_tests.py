@@ -75,6 +75,39 @@ def test_taps_in_constant_memory_with_automatic_copies(programs_dir):
     assert np.array_equal(out, ref.row_filter(img, taps2))
 
 
+@pytest.mark.parametrize("M,N,K", [
+    (100, 70, 50),     # ragged in every direction, rows not 16-byte aligned
+    (64, 64, 64),      # whole tiles
+    (1, 1, 1),
+    (130, 33, 7),      # K smaller than a slice
+    (257, 129, 65),
+    (0, 5, 5), (5, 0, 5),   # empty iteration spaces: nothing is launched, C untouched
+    (5, 5, 0),         # empty reduction: C = beta * C
+])
+@pytest.mark.parametrize("name", ["sgemm_runtime_sizes", "sgemm_runtime_sizes_generic"])
+def test_sgemm_runtime_sizes(programs_dir, name, M, N, K):
+    # one compiled function, sizes read from a buffer at run time; once through the contraction
+    # emitter and once through the schedule-faithful emitter
+    from gpu_util import DeviceArray
+    rng = np.random.RandomState(1000 + M + N + K)
+    A, B, C = ints(rng, (M, K)), ints(rng, (K, N)), ints(rng, (M, N))
+    sizes = np.array([M, N, K], np.int32)
+    scal = np.array([2.0, -1.0], np.float32)
+    expected = ref.sgemm(A, B, C, 2.0, -1.0)
+    C_cpu = C.copy()
+    cpu_variant(programs_dir, name)(sizes, scal, A, B, C_cpu)
+    assert np.array_equal(C_cpu, expected)
+    # device buffers carry a few extra elements so that empty matrices still have an address
+    dA, dB, dC = (DeviceArray(np.concatenate([x.ravel(), np.zeros(4, np.float32)])) for x in (A, B, C))
+    prog = runtime.load(programs_dir, name)
+    w = runtime.wrappers()
+    prog(sizes, scal, runtime.Buffer.from_device(dA.ptr, (M, K), np.float32),
+         runtime.Buffer.from_device(dB.ptr, (K, N), np.float32), runtime.Buffer.from_device(dC.ptr, (M, N), np.float32))
+    w.tiramisu_hip_stream_synchronize(0)
+    out = dC.download()[:M * N].reshape(M, N)
+    assert np.array_equal(out, expected)
+
+
 def test_alloc_in_time_loop(programs_dir):
     P = np.zeros((3, 24, 24), np.int32)
     Q = np.zeros((3, 40, 40), np.int32)
