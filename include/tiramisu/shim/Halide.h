@@ -1,0 +1,114 @@
+// A stand-in for the small part of Halide's run-time buffer API that Tiramisu wrapper programs
+// use (the reference's tests/wrapper_test_*.cpp and benchmark wrappers include "Halide.h" only
+// for Halide::Buffer<T>): a dense host array described by a halide_buffer_t with the pinned
+// layout of generated code (benchmarks/linear_algebra/blas/level1/dot/generated_dot.o.h:1157-1219
+// of the reference).  Dimensions are given and indexed innermost first, as in Halide:
+// Buffer<float> A(K, M) is M rows of K contiguous elements and A(k, m) is element [m][k]
+// ("indices are flipped", benchmarks/linear_algebra/blas/level3/sgemm/gpu/wrapper.cpp:59-62).
+// Put this directory on the include path of a wrapper program instead of Halide's.
+#ifndef TIRAMISU_AMD_HALIDE_SHIM_H
+#define TIRAMISU_AMD_HALIDE_SHIM_H
+#include <cstdint>
+#include <cstring>
+#include <initializer_list>
+#include <memory>
+#include <vector>
+
+#ifndef HALIDE_BUFFER_T_DEFINED
+#define HALIDE_BUFFER_T_DEFINED
+typedef struct halide_dimension_t { int32_t min, extent, stride; uint32_t flags; } halide_dimension_t;
+typedef struct halide_type_t { uint8_t code, bits; uint16_t lanes; } halide_type_t;
+typedef struct halide_buffer_t {
+    uint64_t device;
+    const void *device_interface;
+    uint8_t *host;
+    uint64_t flags;
+    halide_type_t type;
+    int32_t dimensions;
+    halide_dimension_t *dim;
+    void *padding;
+} halide_buffer_t;
+#endif
+
+namespace Halide {
+
+namespace shim {
+template <class T> struct type_code { static constexpr uint8_t value = T(-1) < T(0) ? (T(1) / T(2) != T(0) ? 2 : 0) : 1; };
+template <> struct type_code<bool> { static constexpr uint8_t value = 1; };
+}  // namespace shim
+
+template <class T>
+class Buffer {
+    struct storage {
+        std::vector<T> data;
+        std::vector<halide_dimension_t> dims;
+        halide_buffer_t raw;
+    };
+    std::shared_ptr<storage> s;   // copies share the array, as Halide's do
+
+    void build(const std::vector<int> &extents) {
+        s = std::make_shared<storage>();
+        size_t count = 1;
+        s->dims.resize(extents.empty() ? 1 : extents.size());
+        for (size_t d = 0; d < extents.size(); d++) {
+            s->dims[d] = halide_dimension_t{0, extents[d], (int32_t)count, 0};
+            count *= (size_t)extents[d];
+        }
+        s->data.assign(count, T(0));
+        std::memset(&s->raw, 0, sizeof(s->raw));
+        s->raw.host = reinterpret_cast<uint8_t *>(s->data.data());
+        s->raw.type = halide_type_t{shim::type_code<T>::value, (uint8_t)(8 * sizeof(T)), 1};
+        s->raw.dimensions = (int32_t)extents.size();
+        s->raw.dim = s->dims.data();
+    }
+    size_t offset(std::initializer_list<int> idx) const {
+        size_t o = 0, d = 0;
+        for (int i : idx) o += (size_t)i * (size_t)s->dims[d++].stride;
+        return o;
+    }
+
+public:
+    Buffer() { build({}); }
+    explicit Buffer(int e0) { build({e0}); }
+    Buffer(int e0, int e1) { build({e0, e1}); }
+    Buffer(int e0, int e1, int e2) { build({e0, e1, e2}); }
+    Buffer(int e0, int e1, int e2, int e3) { build({e0, e1, e2, e3}); }
+    explicit Buffer(const std::vector<int> &extents) { build(extents); }
+
+    halide_buffer_t *raw_buffer() { return &s->raw; }
+    const halide_buffer_t *raw_buffer() const { return &s->raw; }
+    T *data() { return s->data.data(); }
+    const T *data() const { return s->data.data(); }
+    T *begin() { return data(); }
+    T *end() { return data() + s->data.size(); }
+    int dimensions() const { return s->raw.dimensions; }
+    int extent(int d) const { return d < dimensions() ? s->dims[d].extent : 1; }
+    int width() const { return extent(0); }
+    int height() const { return extent(1); }
+    int channels() const { return extent(2); }
+    size_t number_of_elements() const { return s->data.size(); }
+    size_t size_in_bytes() const { return s->data.size() * sizeof(T); }
+    void fill(T v) { for (auto &x : s->data) x = v; }
+    void copy_from(const Buffer<T> &o) { s->data = o.s->data; }
+
+    // missing trailing indices are 0, so a 2-D buffer can be read as b(x, y, 0)
+    T &operator()(int i0) { return s->data[offset({i0})]; }
+    T &operator()(int i0, int i1) { return s->data[offset({i0, i1})]; }
+    T &operator()(int i0, int i1, int i2) { return s->data[offset3(i0, i1, i2)]; }
+    T &operator()(int i0, int i1, int i2, int i3) { return s->data[offset({i0, i1, i2, i3})]; }
+    const T &operator()(int i0) const { return s->data[offset({i0})]; }
+    const T &operator()(int i0, int i1) const { return s->data[offset({i0, i1})]; }
+    const T &operator()(int i0, int i1, int i2) const { return s->data[offset3(i0, i1, i2)]; }
+    const T &operator()(int i0, int i1, int i2, int i3) const { return s->data[offset({i0, i1, i2, i3})]; }
+
+private:
+    size_t offset3(int i0, int i1, int i2) const {
+        size_t o = 0;
+        const int idx[3] = {i0, i1, i2};
+        for (int d = 0; d < 3 && d < dimensions(); d++) o += (size_t)idx[d] * (size_t)s->dims[d].stride;
+        return o;
+    }
+};
+
+}  // namespace Halide
+#endif

@@ -126,6 +126,32 @@ def program_sources():
     return out
 
 
+WRAPPER_DIR = os.path.join(ROOT, "tests", "wrappers")
+
+
+def wrapper_library(name):
+    return os.path.join(WRAPPER_DIR, "build", "lib%s.so" % name)
+
+
+def build_wrapper_program(source):
+    """Link a C++ wrapper program (main() + Halide::Buffer arguments, the reference's
+    tests/wrapper_test_*.cpp style) with the generated object named in its first
+    ``// links: <dir>/<object>`` line into a shared library whose entry point is
+    ``tiramisu_wrapper_main`` (the program's main), so that a test can run it in-process."""
+    stem = os.path.splitext(os.path.basename(source))[0]
+    objects = []
+    for line in open(source):
+        if line.startswith("// links:"):
+            objects += [os.path.join(ROOT, o) for o in line[len("// links:"):].split()]
+    os.makedirs(os.path.join(WRAPPER_DIR, "build"), exist_ok=True)
+    entry = os.path.join(WRAPPER_DIR, "build", "entry.h")
+    with open(entry, "w") as f:
+        f.write('extern "C" int tiramisu_wrapper_main(int, char **);\n')
+    _run(["g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-I" + INCLUDE, "-I" + os.path.join(INCLUDE, "tiramisu", "shim"),
+          "-include", entry, "-Dmain=tiramisu_wrapper_main", "-o", wrapper_library(stem), source] + objects +
+         ["-L" + PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(PKG, os.path.join(WRAPPER_DIR, "build"))])
+
+
 def build_all(force=True, verbose=False):
     build_compiler(force)
     build_wrappers(force)
@@ -135,6 +161,10 @@ def build_all(force=True, verbose=False):
         if verbose:
             print("[build] program", os.path.relpath(src, ROOT), flush=True)
         build_program(src, force)
+    if os.path.isdir(WRAPPER_DIR):
+        for f in sorted(os.listdir(WRAPPER_DIR)):
+            if f.endswith(".cpp"):
+                build_wrapper_program(os.path.join(WRAPPER_DIR, f))
 
 
 if __name__ == "__main__":
