@@ -6,4 +6,5 @@
 #include <tiramisu/expr.h>
 #include <tiramisu/core.h>
 #include <tiramisu/block.h>
+#include <tiramisu/macros.h>
 #endif

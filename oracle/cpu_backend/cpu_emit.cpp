@@ -120,6 +120,13 @@ struct cpu_gen {
                 extern_decls.push_back(s + ");");
             }
         });
+        if (n->lkind == leaf_kind::let) {
+            // a scheduled constant: a scalar visible to the rest of this loop body
+            // (reference: LetStmt around the consumer, tiramisu_codegen_halide.cpp:2943-2975)
+            out << pad(ind) << "const " << primitive_c_name(n->comp->get_data_type()) << " " << n->comp->get_name() << " = "
+                << cp.print(n->rhs) << ";\n";
+            return;
+        }
         int i2 = ind;
         const bool scoped = !n->lets.empty() || n->predicate.is_defined();
         if (scoped) { out << pad(ind) << "{\n"; i2++; }

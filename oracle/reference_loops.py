@@ -104,6 +104,30 @@ def row_filter(image, taps):
     return acc.astype(np.float32)
 
 
+def resample_bilinear(src):
+    """The bilinear resampling of tests/programs/resample_bilinear.cpp (the structure of the
+    reference's benchmarks/halide/warp_affinegpu_tiramisu.cpp:55-76: affine sample position, floor,
+    clamped neighbours, two horizontal and one vertical interpolation), in fp32, operation by
+    operation as the program text has them."""
+    f = np.float32
+    h, w = src.shape
+    y = np.arange(h, dtype=np.float32)[:, None]
+    x = np.arange(w, dtype=np.float32)[None, :]
+    fy = (y * f(0.96875) + x * f(0.0625)) - f(1.5)
+    fx = (x * f(0.96875) - y * f(0.0625)) + f(2.25)
+    y0 = np.floor(fy).astype(np.int32)
+    x0 = np.floor(fx).astype(np.int32)
+    wy = fy - np.floor(fy)
+    wx = fx - np.floor(fx)
+    ya, yc = np.clip(y0, 0, h - 1), np.clip(y0 + 1, 0, h - 1)
+    xa, xc = np.clip(x0, 0, w - 1), np.clip(x0 + 1, 0, w - 1)
+    s = src.astype(np.float32)
+    p00, p01, p10, p11 = s[ya, xa], s[ya, xc], s[yc, xa], s[yc, xc]
+    top = p00 + (p01 - p00) * wx
+    bottom = p10 + (p11 - p10) * wx
+    return (top + (bottom - top) * wy).astype(np.float32)
+
+
 def _shifted(plane, r, dy, dx):
     """View of the interior (margin r) of `plane` displaced by (dy, dx)."""
     ny, nx = plane.shape

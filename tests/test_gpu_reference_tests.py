@@ -108,6 +108,21 @@ def test_sgemm_runtime_sizes(programs_dir, name, M, N, K):
     assert np.array_equal(out, expected)
 
 
+def test_resample_bilinear_scheduled_constants(programs_dir):
+    # constants declared at a loop level (scalars in the kernel), clamped data-dependent indices
+    from gpu_util import DeviceArray
+    src = np.random.RandomState(77).randint(0, 256, (90, 132)).astype(np.uint8)
+    d_src, d_dst = DeviceArray(src), DeviceArray(np.zeros((90, 132), np.float32))
+    runtime.load(programs_dir, "resample_bilinear")(d_src.buffer(), d_dst.buffer())
+    out = d_dst.download()
+    out_cpu = np.zeros((90, 132), np.float32)
+    cpu_variant(programs_dir, "resample_bilinear")(src, out_cpu)
+    # every intermediate value is exactly representable (weights are multiples of 1/32), so
+    # the comparison is bit for bit whatever the contraction of multiply-adds
+    assert np.array_equal(out, ref.resample_bilinear(src))
+    assert np.array_equal(out, out_cpu)
+
+
 def test_alloc_in_time_loop(programs_dir):
     P = np.zeros((3, 24, 24), np.int32)
     Q = np.zeros((3, 40, 40), np.int32)

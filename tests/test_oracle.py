@@ -80,6 +80,28 @@ def test_row_filter_restatement_pins():
     assert np.array_equal(ref.row_filter(img, taps), loops)
 
 
+def test_resample_restatement_pins():
+    # a constant image resamples to itself; an image linear in x and y is reproduced exactly where
+    # no neighbour is clamped (bilinear interpolation is exact on such images)
+    assert np.all(ref.resample_bilinear(np.full((20, 30), 7, np.uint8)) == 7.0)
+    h, w = 40, 48
+    yy, xx = np.mgrid[0:h, 0:w]
+    img = (2 * yy + xx).astype(np.uint8)
+    out = ref.resample_bilinear(img)
+    fy = yy * 0.96875 + xx * 0.0625 - 1.5
+    fx = xx * 0.96875 - yy * 0.0625 + 2.25
+    inside = (fy >= 0) & (fy <= h - 2) & (fx >= 0) & (fx <= w - 2)
+    assert inside.sum() > 1000
+    assert np.array_equal(out[inside], (2 * fy + fx)[inside].astype(np.float32))
+
+
+def test_cpu_resample_bilinear():
+    src = np.random.RandomState(77).randint(0, 256, (90, 132)).astype(np.uint8)
+    out = np.zeros((90, 132), np.float32)
+    cpu_program("resample_bilinear")(src, out)
+    assert np.array_equal(out, ref.resample_bilinear(src))
+
+
 def test_cpu_taps_in_constant_memory():
     rng = np.random.RandomState(61)
     img, taps = ints(rng, (70, 100)), ints(rng, (5,))

@@ -232,6 +232,9 @@ struct lowering {
         }
         if (!e.is_defined()) ERROR("computation " + C->get_name() + " is scheduled but has no expression", true);
         n->lkind = (e.get_expr_type() == e_op && e.get_op_type() == o_call) ? leaf_kind::call : leaf_kind::assign;
+        // a scheduled constant declares a scalar visible to what follows it in its loop body
+        // (reference: tiramisu_codegen_cuda.cpp:658-676)
+        if (C->is_let_stmt()) n->lkind = leaf_kind::let;
         for (auto &l : C->get_associated_let_stmts())
             n->lets.push_back({l.first, lower_expr(build, C, n->iterators, l.second)});
         n->rhs = lower_expr(build, C, n->iterators, e);
@@ -247,6 +250,8 @@ struct lowering {
             n->lhs_index = a.get_access();
         } else if (n->lkind == leaf_kind::assign) {
             ERROR("computation " + C->get_name() + " has no buffer to store its result", true);
+        } else if (n->lkind == leaf_kind::let && C->get_predicate().is_defined()) {
+            ERROR("constant " + C->get_name() + " cannot carry a predicate", true);
         }
         return n;
     }
@@ -379,7 +384,7 @@ void function::gen_isl_ast() {
 
     isl_union_map *umap = nullptr;
     for (auto c : body) {
-        if (!c->should_schedule_this_computation() || c->is_let_stmt()) continue;
+        if (!c->should_schedule_this_computation()) continue;   // function-wide constants, inputs
         isl_map *m = isl_map_copy(c->get_schedule());
         m = isl_map_project_out(m, isl_dim_out, 0, 1);  // the duplicate dimension
         isl_set *d = isl_set_copy(c->get_iteration_domain());
@@ -579,6 +584,7 @@ std::string dump(const node_ptr &n, int indent) {
         case leaf_kind::copy: os << "copy " << n->copy_from->get_name() << " -> " << n->copy_to->get_name(); break;
         case leaf_kind::allocate: os << "allocate " << n->target->get_name(); break;
         case leaf_kind::release: os << "free " << n->target->get_name(); break;
+        case leaf_kind::let: os << "let " << n->comp->get_name(); break;
         default:
             if (n->predicate.is_defined()) os << "if " << n->predicate.to_str() << ": ";
             if (n->lhs) os << expr(o_access, n->lhs->get_name(), n->lhs_index, p_none).to_str() << " = ";

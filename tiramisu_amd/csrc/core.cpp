@@ -1214,11 +1214,38 @@ std::vector<var> Input::iterators_from_size_expressions(std::vector<expr> sizes)
 Input::Input(std::string nm, std::vector<expr> sizes, primitive_t t) : input(nm, iterators_from_size_expressions(sizes), t) {}
 
 constant::constant(std::string param_name, const expr &param_expr, primitive_t t, bool function_wide,
-                   computation *, int, function *func) {
-    if (!function_wide)
-        ERROR("constant " + param_name + ": only function-wide constants are provided by this build", true);
+                   computation *with_computation, int at_loop_level, function *func) {
+    if (!func) ERROR("call tiramisu::init() first", true);
+    if (function_wide != (with_computation == nullptr))
+        ERROR("constant " + param_name + ": give a computation exactly when the constant is not function-wide", true);
+    if (!function_wide) {
+        // A scalar recomputed inside the loop nest of `with_computation`, right before it at loop
+        // level `at_loop_level`: its iteration domain is the consumer's projected onto the loops
+        // down to that level (reference: tiramisu_core.cpp:8094-8136).
+        isl_set *iter = isl_set_copy(with_computation->get_iteration_domain());
+        const int keep = at_loop_level + 1, n = isl_set_dim(iter, isl_dim_set);
+        if (at_loop_level < computation::root_dimension || keep > n)
+            ERROR("constant " + param_name + ": loop level out of range", true);
+        iter = isl_set_project_out(iter, isl_dim_set, keep, n - keep);
+        iter = isl_set_set_tuple_name(iter, param_name.c_str());
+        char *str = isl_set_to_str(iter);
+        const std::string domain = str;
+        free(str);
+        isl_set_free(iter);
+        init_computation(domain, func, param_expr, true, t);
+        is_let = true;
+        if (keep == 0) {
+            before(*with_computation, computation::root_dimension);
+        } else if (computation *pred = with_computation->get_predecessor()) {
+            // keep the consumer's place in the order: predecessor, then this, then the consumer
+            const int fused = func->sched_graph[pred][with_computation];
+            between(*pred, fused, *with_computation, at_loop_level);
+        } else {
+            before(*with_computation, at_loop_level);
+        }
+        return;
+    }
     fct = func;
-    if (!fct) ERROR("call tiramisu::init() first", true);
     ctx = fct->get_isl_ctx();
     name = param_name;
     expression = param_expr;

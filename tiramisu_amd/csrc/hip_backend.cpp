@@ -69,8 +69,10 @@ struct generic_kernel_gen {
                 if (n->gpu_block >= 0) loops_per_dim[0][n->gpu_block]++;
                 if (n->gpu_thread >= 0) loops_per_dim[1][n->gpu_thread]++;
             }
-            if (n->kind == node_kind::leaf)
+            if (n->kind == node_kind::leaf) {
                 for (auto &l : n->lets) inner.insert(l.first);
+                if (n->lkind == leaf_kind::let) inner.insert(n->comp->get_name());
+            }
         });
     }
 
@@ -190,6 +192,11 @@ struct generic_kernel_gen {
             return;
         case leaf_kind::release: return;
         case leaf_kind::copy: ERROR("memcpy computation " + n->comp->get_name() + " is scheduled inside a GPU kernel", true);
+        case leaf_kind::let:
+            // visible to the statements that follow in this loop body
+            body << pad(ind) << "const " << primitive_c_name(n->comp->get_data_type()) << " " << n->comp->get_name() << " = "
+                 << dev.print(n->rhs) << ";\n";
+            return;
         default: break;
         }
         int i2 = ind;
@@ -249,6 +256,8 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
         primitive_t t = global::get_loop_iterator_data_type();
         for (auto c : f->get_invariants())
             if (c->get_name() == nm) t = c->get_data_type();
+        for (auto c : f->get_computation_by_name(nm))   // a constant scheduled on the host
+            if (c->is_let_stmt()) t = c->get_data_type();
         k.params.push_back({false, nm, t});
     }
     for (auto &nm : g.used_buffers) {
@@ -434,6 +443,11 @@ struct host_gen {
             return;
         }
         default: break;
+        }
+        if (n->lkind == leaf_kind::let) {
+            out << pad(ind) << "const " << primitive_c_name(n->comp->get_data_type()) << " " << n->comp->get_name() << " = "
+                << hp.print(n->rhs) << ";\n";
+            return;
         }
         // host-side assignment or call
         n->rhs.visit([&](const expr &e) {

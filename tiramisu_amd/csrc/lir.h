@@ -20,7 +20,7 @@ namespace tiramisu {
 namespace lir {
 
 enum class node_kind { block, loop, cond, leaf };
-enum class leaf_kind { assign, sync, copy, allocate, release, call };
+enum class leaf_kind { assign, sync, copy, allocate, release, call, let };   // let: const scalar named after its computation
 
 struct node;
 using node_ptr = std::shared_ptr<node>;
