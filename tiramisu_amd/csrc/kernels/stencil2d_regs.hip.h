@@ -35,6 +35,9 @@
 //   ST_RAD             stencil radius (<= 4, <= ST_RPT)
 //   ST_W               wavefronts per workgroup
 //   ST_RPT             rows per thread
+//   ST_RPT_EDGE        rows per thread in the kernel for boundary tiles (a divisor-sized slice
+//                      of a tile; launch it with ceil(ST_TH / (ST_W*ST_RPT_EDGE - 2*ST_R*ST_RAD))
+//                      workgroups per boundary tile)
 //   ST_EXPR            expression of the new value in terms of ST_AT(dy, dx)
 //   ST_NAME_EDGE       name of the kernel for the tiles that touch the fixed boundary
 //   ST_GX, ST_GY       number of tiles along x and y
@@ -93,20 +96,25 @@ __device__ __forceinline__ st_f4 st_load_quad(const float *__restrict__ plane, i
 }
 #endif
 
-template <bool EDGE>
-__device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int bx, int by) {
+// One workgroup advances the region of ST_W*RPT rows whose centre starts at plane row `oy`, column
+// `ox`, and writes the centre rows below `row_end`.
+template <bool EDGE, int RPT>
+__device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int oy, int ox,
+                                                        int row_end) {
     // values stay in registers from one step to the next: without this the multiply that ends a
     // step would be fused with an add of the next one, and results would differ from the
     // un-tiled program's
 #pragma clang fp contract(off)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int gy0 = by * ST_TH - ST_HY + wave * ST_RPT;   // plane row of my first row
-    const int gx = bx * ST_TW - ST_HX + 4 * lane;         // plane column of my quads
+    constexpr int CENTRE_ROWS = ST_W * RPT - 2 * ST_HY;
+    static_assert(CENTRE_ROWS > 0 && RPT >= ST_RAD, "the halo leaves no rows to write");
+    const int gy0 = oy - ST_HY + wave * RPT;              // plane row of my first row
+    const int gx = ox - ST_HX + 4 * lane;                 // plane column of my quads
     const int wave_up = wave > 0 ? wave - 1 : 0, wave_dn = wave < ST_W - 1 ? wave + 1 : ST_W - 1;
 
-    st_f4 cur[ST_RPT], other[EDGE ? ST_RPT : 1];   // other: the other plane's values (fixed cells only)
+    st_f4 cur[RPT], other[EDGE ? RPT : 1];   // other: the other plane's values (fixed cells only)
 #pragma unroll
-    for (int r = 0; r < ST_RPT; r++) {
+    for (int r = 0; r < RPT; r++) {
         cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
         if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(dst, gy0 + r, gx);
     }
@@ -122,29 +130,29 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
 #pragma unroll
         for (int i = 0; i < ST_RAD; i++) {
             *slot(parity, wave, 0, i) = cur[i];
-            *slot(parity, wave, 1, i) = cur[ST_RPT - ST_RAD + i];
+            *slot(parity, wave, 1, i) = cur[RPT - ST_RAD + i];
         }
         __syncthreads();
         // my rows with ST_RAD rows of the neighbouring wavefronts above and below
-        st_f4 ext[ST_RPT + 2 * ST_RAD];
+        st_f4 ext[RPT + 2 * ST_RAD];
 #pragma unroll
         for (int i = 0; i < ST_RAD; i++) {
             ext[i] = *slot(parity, wave_up, 1, i);
-            ext[ST_RAD + ST_RPT + i] = *slot(parity, wave_dn, 0, i);
+            ext[ST_RAD + RPT + i] = *slot(parity, wave_dn, 0, i);
         }
 #pragma unroll
-        for (int r = 0; r < ST_RPT; r++) ext[ST_RAD + r] = cur[r];
+        for (int r = 0; r < RPT; r++) ext[ST_RAD + r] = cur[r];
         // the ST_RAD cells left and right of every quad, from the adjacent lanes
-        float lf[ST_RPT + 2 * ST_RAD][ST_RAD], rt[ST_RPT + 2 * ST_RAD][ST_RAD];
+        float lf[RPT + 2 * ST_RAD][ST_RAD], rt[RPT + 2 * ST_RAD][ST_RAD];
 #pragma unroll
-        for (int j = 0; j < ST_RPT + 2 * ST_RAD; j++)
+        for (int j = 0; j < RPT + 2 * ST_RAD; j++)
 #pragma unroll
             for (int i = 0; i < ST_RAD; i++) {
                 lf[j][i] = st_from_left(ext[j][4 - ST_RAD + i]);
                 rt[j][i] = st_from_right(ext[j][i]);
             }
 #pragma unroll
-        for (int r = 0; r < ST_RPT; r++) {
+        for (int r = 0; r < RPT; r++) {
             // window of old values around the quad: rows -RAD..RAD, columns -RAD..3+RAD
             float w[2 * ST_RAD + 1][4 + 2 * ST_RAD];
 #pragma unroll
@@ -180,9 +188,9 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     // ---- write the tile centre (cells of the domain only)
     if (4 * lane >= ST_HX && 4 * lane < ST_HX + ST_TW) {
 #pragma unroll
-        for (int r = 0; r < ST_RPT; r++) {
-            const int row = wave * ST_RPT + r, gy = gy0 + r;
-            if (row < ST_HY || row >= ST_HY + ST_TH) continue;
+        for (int r = 0; r < RPT; r++) {
+            const int row = wave * RPT + r, gy = gy0 + r;
+            if (row < ST_HY || row >= ST_HY + CENTRE_ROWS || gy >= row_end) continue;
             if (EDGE && (gy < ST_Y0 || gy > ST_Y1)) continue;
             if ((ST_NX % 4 == 0) && (!EDGE || (gx >= ST_X0 && gx + 3 <= ST_X1))) {
                 *reinterpret_cast<st_f4 *>(dst + (size_t)gy * ST_NX + gx) = cur[r];
@@ -203,7 +211,6 @@ __attribute__((amdgpu_waves_per_eu(ST_OCC)))
 ST_NAME(float *__restrict__ planes, const int src_plane)
 {
     static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
-    static_assert(ST_RPT >= ST_RAD, "a strip must be at least as tall as the stencil radius");
     __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
     const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
     float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
@@ -217,11 +224,16 @@ ST_NAME(float *__restrict__ planes, const int src_plane)
 #else
     const int tile = b;
 #endif
-    ST_CAT(ST_NAME, _sweep)<false>(src, dst, xch, ST_IBX0 + tile % IW, ST_IBY0 + tile / IW);
+    ST_CAT(ST_NAME, _sweep)<false, ST_RPT>(src, dst, xch, (ST_IBY0 + tile / IW) * ST_TH, (ST_IBX0 + tile % IW) * ST_TW, ST_NY);
 }
 
 // The other tiles, in the order: full tile rows above the interior rectangle, full rows below it,
-// then the tiles left and right of it row by row.
+// then the tiles left and right of it row by row.  These tiles are few (one ring), so each is cut
+// into ST_EDGE_SUB horizontal slices of ST_W*ST_RPT_EDGE staged rows, one workgroup each: more and
+// lighter workgroups (the swap registers come on top of the strip) instead of two rounds of one
+// heavy workgroup per CU.
+#define ST_TH_EDGE (ST_W * ST_RPT_EDGE - 2 * ST_HY)
+#define ST_EDGE_SUB ((ST_TH + ST_TH_EDGE - 1) / ST_TH_EDGE)
 extern "C" __global__ void __launch_bounds__(64 * ST_W)
 ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
 {
@@ -230,7 +242,8 @@ ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
     float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
     constexpr int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
     constexpr int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
-    int e = blockIdx.x, bx, by;
+    const int sub = blockIdx.x % ST_EDGE_SUB;
+    int e = blockIdx.x / ST_EDGE_SUB, bx, by;
     if (e < TOP) {
         by = e / ST_GX;
         bx = e % ST_GX;
@@ -244,8 +257,10 @@ ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
         by = ST_IBY0 + e / (SIDE > 0 ? SIDE : 1);
         bx = c < ST_IBX0 ? c : ST_IBX1 + 1 + (c - ST_IBX0);
     }
-    ST_CAT(ST_NAME, _sweep)<true>(src, dst, xch, bx, by);
+    ST_CAT(ST_NAME, _sweep)<true, ST_RPT_EDGE>(src, dst, xch, by * ST_TH + sub * ST_TH_EDGE, bx * ST_TW, (by + 1) * ST_TH);
 }
+#undef ST_TH_EDGE
+#undef ST_EDGE_SUB
 
 #undef ST_HY
 #undef ST_HX
