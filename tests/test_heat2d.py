@@ -83,7 +83,7 @@ def run_on_gpu(n, steps, planes):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n,steps", SMALL + [(1024, 8)])
+@pytest.mark.parametrize("n,steps", SMALL + [(1024, 8), (1030, 9)])
 def test_gpu_matches_oracle(n, steps):
     g = initial_grid(n, 7 * n + steps)
     planes = np.zeros((2, n, n), np.float32)

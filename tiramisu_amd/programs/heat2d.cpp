@@ -41,6 +41,7 @@ int main()
 {
     generate(8192, 32);   // the benchmark configuration
     generate(1024, 8);
+    generate(1030, 9);    // rows not a multiple of 4 elements with interior tiles: unaligned strips
     generate(256, 1);
     generate(130, 4);
     generate(66, 7);
