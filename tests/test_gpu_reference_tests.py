@@ -123,6 +123,15 @@ def test_resample_bilinear_scheduled_constants(programs_dir):
     assert np.array_equal(out, out_cpu)
 
 
+def test_low_level_api_three_dimensional_gpu_tile(programs_dir):
+    # explicit function object, isl-string domain and access, hand-driven pipeline, 3-D gpu_tile
+    from gpu_util import DeviceArray
+    d = DeviceArray(np.full((10, 10), -1, np.int32))
+    runtime.load(programs_dir, "low_level_api")(d.buffer())
+    i, k = np.mgrid[0:10, 0:10]
+    assert np.array_equal(d.download(), (100 * i + k + 7).astype(np.int32))
+
+
 def test_alloc_in_time_loop(programs_dir):
     P = np.zeros((3, 24, 24), np.int32)
     Q = np.zeros((3, 40, 40), np.int32)
