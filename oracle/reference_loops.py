@@ -128,6 +128,42 @@ def resample_bilinear(src):
     return (top + (bottom - top) * wy).astype(np.float32)
 
 
+def ref_cvtcolor_gpu(rgb):
+    """What the reference's benchmarks/halide/cvtcolorgpu_tiramisu.cpp:26-57 computes: planar RGB
+    uint8 [3][M][N] to gray, (r*4899 + g*9617 + b*1868 + 2^13) >> 14 in uint32, cast to uint8."""
+    r, g, b = (rgb[c].astype(np.uint32) for c in range(3))
+    v = r * np.uint32(4899) + g * np.uint32(9617) + b * np.uint32(1868)
+    return ((v + (np.uint32(1) << np.uint32(13))) >> np.uint32(14)).astype(np.uint8)
+
+
+def ref_gaussian_gpu(img, kx, ky):
+    """benchmarks/halide/gaussiangpu_tiramisu.cpp:44-55: out[c][j][i] = uint8(sum_k ky[k] * gx[c][j+k][i])
+    with gx[c][j][i] = sum_k float(img[c][j][i+k]) * kx[k] (inlined), both sums started from 0.f and
+    added in order, for i < N-5, j < M-5 of a uint8 image [C][M][N]."""
+    f = np.float32
+    C, M, N = img.shape
+    x = img.astype(np.float32)
+    gx = np.zeros((C, M, N - 5), np.float32)
+    for k in range(5):
+        gx = gx + x[:, :, k:k + N - 5] * f(kx[k])
+    acc = np.zeros((C, M - 5, N - 5), np.float32)
+    for k in range(5):
+        acc = acc + gx[:, k:k + M - 5, :] * f(ky[k])
+    return acc.astype(np.uint8)
+
+
+def ref_heat2d_gpu(grid):
+    """benchmarks/halide/heat2dgpu_tiramisu.cpp:37-52: one sweep out = 0.3*c + 0.4*(s + e + n + w) on
+    the interior of a square fp32 grid, border cells set to 0 (terms added in the program's order:
+    row below, column right, row above, column left)."""
+    f = np.float32
+    g = grid.astype(np.float32)
+    out = np.zeros_like(g)
+    s = ((g[2:, 1:-1] + g[1:-1, 2:]) + g[:-2, 1:-1]) + g[1:-1, :-2]
+    out[1:-1, 1:-1] = g[1:-1, 1:-1] * f(0.3) + s * f(0.4)
+    return out
+
+
 def _shifted(plane, r, dy, dx):
     """View of the interior (margin r) of `plane` displaced by (dy, dx)."""
     ny, nx = plane.shape

@@ -1,0 +1,80 @@
+"""GPU generator programs of the reference tree, compiled unchanged by this build
+(tests/reference_programs/build_reference_programs.py) and run through their generated functions'
+C ABI with host buffers, compared with numpy restatements of what the programs' text computes
+(oracle/reference_loops.py: ref_*_gpu).  The programs copy to and from the GPU themselves."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from oracle import reference_loops as ref
+from tiramisu_amd import runtime
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def library(name):
+    return os.path.join(HERE, "reference_programs", "build", "lib%s.so" % name)
+
+
+PROGRAMS = {"cvtcolorgpu": "cvtcolorgpu_tiramisu", "gaussiangpu": "gaussiangpu_tiramisu", "heat2dgpu": "heat2dgpu_tiramisu"}
+
+
+def test_restatements_on_closed_forms():
+    # gray of a gray pixel is itself (the three weights sum to 2^14); binomial blur of a constant
+    # image is the constant; the heat sweep of a constant interior gives 0.3 + 4*0.4 = 1.9 times it
+    rgb = np.stack([np.full((4, 5), v, np.uint8) for v in (200, 200, 200)])
+    assert np.all(ref.ref_cvtcolor_gpu(rgb) == 200)
+    k = np.array([1, 4, 6, 4, 1], np.float32)
+    assert np.all(ref.ref_gaussian_gpu(np.full((2, 12, 14), 37, np.uint8), k, k / 256) == 37)
+    g = np.ones((8, 8), np.float32)
+    out = ref.ref_heat2d_gpu(g)
+    assert np.all(out[1:-1, 1:-1] == np.float32(1.0) * np.float32(0.3) + np.float32(4.0) * np.float32(0.4))
+    assert np.all(out[0] == 0) and np.all(out[:, -1] == 0)
+
+
+@pytest.mark.parametrize("name", sorted(PROGRAMS))
+def test_generated_library_exports_its_function(name):
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    assert hasattr(ctypes.CDLL(library(name)), PROGRAMS[name])
+
+
+def load(name):
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    return runtime.Program(library(name), PROGRAMS[name])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(48, 64), (37, 53)])
+def test_reference_cvtcolorgpu(M, N):
+    rgb = np.random.RandomState(M).randint(0, 256, (3, M, N)).astype(np.uint8)
+    out = np.zeros((M, N), np.uint8)
+    load("cvtcolorgpu")(np.array([N, M], np.int32), rgb, out)
+    assert np.array_equal(out, ref.ref_cvtcolor_gpu(rgb))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("C,M,N", [(3, 69, 101), (1, 37, 37)])
+def test_reference_gaussiangpu(C, M, N):
+    # the wrapper's own taps (benchmarks/halide/wrapper_gaussiangpu.cpp:39-40): every value stays exact
+    kx = np.array([1, 4, 6, 4, 1], np.float32)
+    ky = kx / np.float32(256)
+    img = np.random.RandomState(N).randint(0, 256, (C, M, N)).astype(np.uint8)
+    out = np.zeros((C, M - 5, N - 5), np.uint8)
+    load("gaussiangpu")(np.array([N, M, C], np.int32), img, kx, ky, out)
+    assert np.array_equal(out, ref.ref_gaussian_gpu(img, kx, ky))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [62, 92, 47])
+def test_reference_heat2dgpu(n):
+    grid = np.random.RandomState(n).uniform(0, 1, (n, n)).astype(np.float32)
+    out = np.full((n, n), -1.0, np.float32)
+    load("heat2dgpu")(np.array([n, n], np.int32), grid, out)
+    expected = ref.ref_heat2d_gpu(grid)
+    # 0.3*c + 0.4*s may be contracted to a fused multiply-add on the GPU
+    assert np.max(np.abs(out - expected)) <= 1e-6 * np.max(np.abs(expected))

@@ -88,10 +88,14 @@ def program_library(directory, name):
     return os.path.join(directory, "build", "lib%s.so" % name)
 
 
-def build_program(source, force=True, extra_objects=(), defines=()):
+def build_program(source, force=True, extra_objects=(), defines=(), directory=None, shim_headers=False):
     """Compile and run the generator ``source`` (a Tiramisu program), then link every host
-    object it wrote (build/<x>.o) into build/lib<x>.so next to the source."""
-    directory = os.path.dirname(os.path.abspath(source))
+    object it wrote (build/<x>.o) into build/lib<x>.so -- next to the source, or under
+    ``directory`` when the source lies in a tree that must not be written to.  ``shim_headers``
+    adds the stand-ins of include/tiramisu/shim (Halide.h, isl/*.h) to the include path, for
+    programs written against the reference's include set."""
+    source_dir = os.path.dirname(os.path.abspath(source))
+    directory = os.path.abspath(directory) if directory else source_dir
     stem = os.path.splitext(os.path.basename(source))[0]
     bdir = os.path.join(directory, "build")
     os.makedirs(bdir, exist_ok=True)
@@ -100,7 +104,8 @@ def build_program(source, force=True, extra_objects=(), defines=()):
     if not force and _newer(stamp, [source, compiler_library(), wrappers_library()]):
         return
     before = {f: os.path.getmtime(os.path.join(bdir, f)) for f in os.listdir(bdir) if f.endswith(".o")}
-    _run(["g++", "-std=c++17", "-O1", "-I" + INCLUDE, "-I" + directory] + ["-D" + d for d in defines] +
+    shim = ["-I" + os.path.join(INCLUDE, "tiramisu", "shim")] if shim_headers else []
+    _run(["g++", "-std=c++17", "-O1", "-I" + INCLUDE, "-I" + source_dir] + shim + ["-D" + d for d in defines] +
          ["-o", gen, source] + list(extra_objects) +
          ["-L" + PKG, "-ltiramisu", "-Wl,-rpath," + PKG])
     env_out = _run([gen], cwd=directory)

@@ -12,7 +12,7 @@
 #include <cstdint>
 #include <sstream>
 
-#include "isl_api.h"
+#include <tiramisu/isl_api.h>
 #include "lir.h"
 #include "util.h"
 

@@ -7,7 +7,7 @@
 #include <sstream>
 
 #include "hip_backend.h"
-#include "isl_api.h"
+#include <tiramisu/isl_api.h>
 #include "util.h"
 
 namespace tiramisu {
