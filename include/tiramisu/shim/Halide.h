@@ -40,7 +40,8 @@ template <> struct type_code<bool> { static constexpr uint8_t value = 1; };
 template <class T>
 class Buffer {
     struct storage {
-        std::vector<T> data;
+        std::unique_ptr<T[]> data;           // a plain array: Buffer<bool> must hand out bool *
+        size_t count = 0;
         std::vector<halide_dimension_t> dims;
         halide_buffer_t raw;
     };
@@ -54,9 +55,10 @@ class Buffer {
             s->dims[d] = halide_dimension_t{0, extents[d], (int32_t)count, 0};
             count *= (size_t)extents[d];
         }
-        s->data.assign(count, T(0));
+        s->count = count;
+        s->data.reset(new T[count > 0 ? count : 1]());
         std::memset(&s->raw, 0, sizeof(s->raw));
-        s->raw.host = reinterpret_cast<uint8_t *>(s->data.data());
+        s->raw.host = reinterpret_cast<uint8_t *>(s->data.get());
         s->raw.type = halide_type_t{shim::type_code<T>::value, (uint8_t)(8 * sizeof(T)), 1};
         s->raw.dimensions = (int32_t)extents.size();
         s->raw.dim = s->dims.data();
@@ -77,19 +79,19 @@ public:
 
     halide_buffer_t *raw_buffer() { return &s->raw; }
     const halide_buffer_t *raw_buffer() const { return &s->raw; }
-    T *data() { return s->data.data(); }
-    const T *data() const { return s->data.data(); }
+    T *data() { return s->data.get(); }
+    const T *data() const { return s->data.get(); }
     T *begin() { return data(); }
-    T *end() { return data() + s->data.size(); }
+    T *end() { return data() + s->count; }
     int dimensions() const { return s->raw.dimensions; }
     int extent(int d) const { return d < dimensions() ? s->dims[d].extent : 1; }
     int width() const { return extent(0); }
     int height() const { return extent(1); }
     int channels() const { return extent(2); }
-    size_t number_of_elements() const { return s->data.size(); }
-    size_t size_in_bytes() const { return s->data.size() * sizeof(T); }
-    void fill(T v) { for (auto &x : s->data) x = v; }
-    void copy_from(const Buffer<T> &o) { s->data = o.s->data; }
+    size_t number_of_elements() const { return s->count; }
+    size_t size_in_bytes() const { return s->count * sizeof(T); }
+    void fill(T v) { for (size_t i = 0; i < s->count; i++) s->data[i] = v; }
+    void copy_from(const Buffer<T> &o) { for (size_t i = 0; i < s->count && i < o.s->count; i++) s->data[i] = o.s->data[i]; }
 
     // missing trailing indices are 0, so a 2-D buffer can be read as b(x, y, 0)
     T &operator()(int i0) { return s->data[offset({i0})]; }

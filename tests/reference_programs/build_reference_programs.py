@@ -27,8 +27,37 @@ PROGRAMS = [
 ]
 
 
+# The reference's own GPU tests and tutorials: generator and wrapper program, both unchanged.
+# The wrapper (main(): Halide::Buffer inputs, nested-loop expectation, compare_buffers) is linked
+# with the object its generator wrote into build/lib<wrapper>.so and run in-process by the tests.
+# (generator, wrapper) below the reference tree:
+TESTS = [("tests/test_%s.cpp" % n, "tests/wrapper_test_%s.cpp" % n)
+         for n in ("162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + [
+    ("tutorials/developers/tutorial_04gpu/tutorial_04gpu.cpp", "tutorials/developers/tutorial_04gpu/wrapper_tutorial_04gpu.cpp"),
+    ("tutorials/developers/tutorial_04gpu2/tutorial_04gpu2.cpp", "tutorials/developers/tutorial_04gpu2/wrapper_tutorial_04gpu2.cpp"),
+]
+
+
 def library(name):
     return os.path.join(HERE, "build", "lib%s.so" % name)
+
+
+def wrapper_name(wrapper_rel):
+    return os.path.splitext(os.path.basename(wrapper_rel))[0]
+
+
+def build_test(generator_rel, wrapper_rel):
+    bdir = os.path.join(HERE, "build")
+    produced = build.build_program(os.path.join(REFERENCE, generator_rel), directory=HERE, shim_headers=True) or []
+    objects = [os.path.join(bdir, o) for o in produced]
+    entry = os.path.join(bdir, "entry.h")
+    with open(entry, "w") as f:
+        f.write('extern "C" int tiramisu_wrapper_main(int, char **);\n')
+    wrapper = os.path.join(REFERENCE, wrapper_rel)
+    build._run(["g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-I" + build.INCLUDE,
+                "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"), "-I" + os.path.dirname(wrapper),
+                "-include", entry, "-Dmain=tiramisu_wrapper_main", "-o", library(wrapper_name(wrapper_rel)), wrapper] + objects +
+               ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
 def build_all(verbose=False):
@@ -40,6 +69,10 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", rel, flush=True)
         build.build_program(os.path.join(REFERENCE, rel), defines=defines, directory=HERE, shim_headers=True)
+    for generator_rel, wrapper_rel in TESTS:
+        if verbose:
+            print("[reference programs]", generator_rel, "+", os.path.basename(wrapper_rel), flush=True)
+        build_test(generator_rel, wrapper_rel)
     return True
 
 

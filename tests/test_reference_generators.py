@@ -78,3 +78,35 @@ def test_reference_heat2dgpu(n):
     expected = ref.ref_heat2d_gpu(grid)
     # 0.3*c + 0.4*s may be contracted to a fused multiply-add on the GPU
     assert np.max(np.abs(out - expected)) <= 1e-6 * np.max(np.abs(expected))
+
+
+# ---------------------------------------------------------------- the reference's own GPU tests
+
+REFERENCE_TESTS = ["wrapper_test_%s" % n for n in ("162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + \
+                  ["wrapper_tutorial_04gpu", "wrapper_tutorial_04gpu2"]
+
+
+@pytest.mark.parametrize("name", REFERENCE_TESTS)
+def test_reference_test_library_exports_its_entry_point(name):
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    assert hasattr(ctypes.CDLL(library(name)), "tiramisu_wrapper_main")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", REFERENCE_TESTS)
+def test_reference_gpu_test_passes(name):
+    """Generator (tests/test_N.cpp or the tutorial) and wrapper (wrapper_test_N.cpp) of the reference,
+    both unchanged: the wrapper fills Halide::Buffer inputs, calls the generated function, computes
+    its own nested-loop expectation and compares (library GEMM calls in 162-166, gpu_tile and
+    cache_shared GEMMs in 167-171, allocate_at in 197, uint8 GEMMs in the tutorials).  A mismatch
+    ends the process with status 1, as the reference's compare_buffers does."""
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    lib = ctypes.CDLL(library(name))
+    lib.tiramisu_wrapper_main.restype = ctypes.c_int
+    lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    print("running", name, flush=True)
+    assert lib.tiramisu_wrapper_main(0, None) == 0
