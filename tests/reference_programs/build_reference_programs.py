@@ -60,6 +60,26 @@ def build_test(generator_rel, wrapper_rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
+# The reference's tuned GPU sgemm schedule (16x6 register tile per thread, LDS tiles with
+# cache_shared; 3072^3).  Its wrapper needs CUDA headers, so the tests drive the generated function
+# themselves; the program times its kernel through an external get_time(), provided by timer_hook.c.
+SGEMM_TUNED = "benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp"
+
+
+def build_sgemm_tuned():
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, "sgemm_generator3")
+    os.makedirs(work, exist_ok=True)
+    src = os.path.join(REFERENCE, SGEMM_TUNED)
+    gen = os.path.join(work, "gen")
+    build._run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
+                "-I" + os.path.dirname(src), "-o", gen, src, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG])
+    build._run([gen], cwd=work)                      # writes fct.o (function "matmul") into its working directory
+    build._run(["gcc", "-O2", "-fPIC", "-shared", "-o", library("get_time"), os.path.join(HERE, "timer_hook.c")])
+    build._run(["g++", "-shared", "-o", library("sgemm_generator3"), os.path.join(work, "fct.o"), "-L" + build.PKG,
+                "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
+
+
 def build_all(verbose=False):
     if not os.path.isdir(REFERENCE):
         if verbose:
@@ -73,6 +93,9 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", generator_rel, "+", os.path.basename(wrapper_rel), flush=True)
         build_test(generator_rel, wrapper_rel)
+    if verbose:
+        print("[reference programs]", SGEMM_TUNED, flush=True)
+    build_sgemm_tuned()
     return True
 
 

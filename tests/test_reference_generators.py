@@ -110,3 +110,40 @@ def test_reference_gpu_test_passes(name):
     lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
     print("running", name, flush=True)
     assert lib.tiramisu_wrapper_main(0, None) == 0
+
+
+def test_reference_tuned_sgemm_library_exports_its_function():
+    if not os.path.exists(library("sgemm_generator3")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    assert hasattr(ctypes.CDLL(library("sgemm_generator3")), "matmul")
+
+
+@pytest.mark.gpu
+def test_reference_tuned_sgemm_schedule():
+    """benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp, unchanged: 3072^3 with a 16x8
+    register tile per thread, k split by 4 and both operands staged with cache_shared; it copies
+    A, B, C to the GPU, times its kernel with get_time() and copies C back.  Its own wrapper needs
+    CUDA headers, so the generated function is called here; small integer data keeps every sum
+    exact, so the comparison with a float64 product is for equality."""
+    if not os.path.exists(library("sgemm_generator3")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    program = runtime.Program(library("sgemm_generator3"), "matmul")
+    n = 3072
+    rng = np.random.RandomState(3072)
+    A = rng.randint(-2, 3, (n, n)).astype(np.float32)
+    B = rng.randint(-2, 3, (n, n)).astype(np.float32)
+    C0 = rng.randint(-4, 5, (n, n)).astype(np.float32)
+    consts = np.array([3, 2], np.float32)
+    expected = (3.0 * (A.astype(np.float64) @ B.astype(np.float64)) + 2.0 * C0).astype(np.float32)
+    best = None
+    for _ in range(3):
+        C = C0.copy()
+        t0, t1 = np.zeros(1, np.float32), np.zeros(1, np.float32)
+        program(consts, A, B, C, t0, t1)
+        assert np.array_equal(C, expected)
+        ms = float(t1[0] - t0[0])
+        best = ms if best is None else min(best, ms)
+    print("generator3 kernel: %.3f ms, %.1f TFLOP/s" % (best, 2.0 * n ** 3 / best / 1e9), flush=True)
