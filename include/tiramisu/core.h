@@ -255,6 +255,22 @@ protected:
     std::vector<std::pair<std::string, expr>> associated_let_stmts;
     std::vector<var> declared_vars;
 
+public:
+    /** One LDS tile installed by cache_shared(): the input it caches, the tile's shape and origin,
+      * and the computations that declare, fill and fence it. */
+    struct shared_cache {
+        std::string input, access;
+        std::vector<int> shape;
+        std::vector<expr> offsets;
+        int copy_level = -1;
+        std::vector<computation *> apparatus;
+    };
+
+protected:
+    expr uncached_expression;             // expression before cache_shared() redirected loads to LDS tiles
+    std::vector<shared_cache> shared_caches;
+    computation *cache_consumer = nullptr;  // set on the computations that cache_shared() creates
+
     computation() {}
     void init_computation(std::string iteration_space_str, function *f, const expr &e,
                           bool schedule_this_computation, primitive_t t);
@@ -305,6 +321,15 @@ public:
     const std::vector<std::string> &get_iteration_domain_dimension_names() const { return iterator_names_; }
     bool should_schedule_this_computation() const { return schedule_this; }
     bool is_let_stmt() const { return is_let; }
+    /** Expression as written, before cache_shared() redirected loads (undefined when it never did). */
+    const expr &get_uncached_expr() const { return uncached_expression; }
+    const std::vector<shared_cache> &get_shared_caches() const { return shared_caches; }
+    /** The computation whose loads this one serves, when cache_shared() created it. */
+    computation *get_cache_consumer() const { return cache_consumer; }
+    /** True when, under the current schedule, every LDS tile of this computation is proven to
+      * hold exactly the elements that the computation reads through it in each iteration of
+      * the copy level: reading the tile then equals reading the cached input directly. */
+    bool shared_caches_cover_reads() const;
     bool is_inline_computation() const { return inline_; }
     bool has_accesses() const;
     buffer *get_buffer() const;

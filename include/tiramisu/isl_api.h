@@ -127,6 +127,7 @@ isl_map *isl_map_set_tuple_name(isl_map *map, enum isl_dim_type type, const char
 const char *isl_map_get_dim_name(isl_map *map, enum isl_dim_type type, unsigned pos);
 isl_map *isl_map_apply_range(isl_map *a, isl_map *b);
 isl_map *isl_map_apply_domain(isl_map *a, isl_map *b);
+isl_map *isl_map_intersect(isl_map *a, isl_map *b);
 isl_map *isl_map_intersect_domain(isl_map *map, isl_set *set);
 isl_map *isl_map_intersect_range(isl_map *map, isl_set *set);
 isl_map *isl_map_intersect_params(isl_map *map, isl_set *params);
@@ -139,6 +140,9 @@ isl_map *isl_map_fix_si(isl_map *map, enum isl_dim_type type, unsigned pos, int 
 isl_bool isl_map_is_single_valued(isl_map *map);
 isl_bool isl_map_is_empty(isl_map *map);
 isl_bool isl_map_is_equal(isl_map *a, isl_map *b);
+isl_bool isl_map_is_subset(isl_map *a, isl_map *b);
+isl_map *isl_map_range_product(isl_map *a, isl_map *b);
+isl_map *isl_map_equate(isl_map *map, enum isl_dim_type type1, int pos1, enum isl_dim_type type2, int pos2);
 isl_val *isl_map_plain_get_val_if_fixed(isl_map *map, enum isl_dim_type type, unsigned pos);
 isl_space *isl_map_get_space(isl_map *map);
 isl_map *isl_map_coalesce(isl_map *map);

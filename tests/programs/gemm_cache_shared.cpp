@@ -4,18 +4,22 @@
 //  * sgemm_shared_regs: alpha * A * B + beta * C in fp32 with a register tile per thread, a local
 //    accumulator array declared with allocate(), block-wide scheduling commands, constants read
 //    from an input buffer, and both operands cached (A with a padded tile).  Same features as the
-//    reference's benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp.
+//    reference's benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp.  Generated twice:
+//    sgemm_shared_regs (the back-end proves the LDS tiles and the register tile sound and emits
+//    its MFMA kernel) and sgemm_shared_regs_generic (kept as scheduled: cooperative copies,
+//    barriers, per-thread array).
 //  * gemm_u8_shared: uint8 GEMM (wrap-around arithmetic) with both operands cached, reduction
 //    kept in global memory.  Same features as tutorials/developers/tutorial_04gpu2.
+#include <cstdlib>
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
 
-static void sgemm_shared_regs()
+static void sgemm_shared_regs(const std::string &name, bool pattern_emitters)
 {
     const int M = 256, N = 192, K = 64;
     const int T = 16, KB = 8, RI = 4, RJ = 2;
-    tiramisu::init("sgemm_shared_regs");
+    tiramisu::init(name);
 
     var i("i", 0, M), j("j", 0, N), k("k", 0, K);
     var io("io", 0, M / RI), ii("ii", 0, RI), jo("jo", 0, N / RJ), ji("ji", 0, RJ);
@@ -66,7 +70,9 @@ static void sgemm_shared_regs()
     acc.cache_shared(A, ko, {T * RI, KB}, {iob * T * RI, ko * KB}, true);
     acc.cache_shared(B, ko, {KB, T * RJ}, {ko * KB, job * T * RJ});
 
-    tiramisu::codegen({scal.get_buffer(), &host_A, &host_B, &host_C}, "build/sgemm_shared_regs.o", true);
+    if (!pattern_emitters) setenv("TIRAMISU_NO_MFMA", "1", 1);
+    tiramisu::codegen({scal.get_buffer(), &host_A, &host_B, &host_C}, "build/" + name + ".o", true);
+    if (!pattern_emitters) unsetenv("TIRAMISU_NO_MFMA");
 }
 
 static void gemm_u8_shared()
@@ -105,7 +111,8 @@ static void gemm_u8_shared()
 
 int main()
 {
-    sgemm_shared_regs();
+    sgemm_shared_regs("sgemm_shared_regs", true);
+    sgemm_shared_regs("sgemm_shared_regs_generic", false);
     gemm_u8_shared();
     return 0;
 }

@@ -60,23 +60,25 @@ def build_test(generator_rel, wrapper_rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
-# The reference's tuned GPU sgemm schedule (16x6 register tile per thread, LDS tiles with
-# cache_shared; 3072^3).  Its wrapper needs CUDA headers, so the tests drive the generated function
-# themselves; the program times its kernel through an external get_time(), provided by timer_hook.c.
-SGEMM_TUNED = "benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp"
+# The reference's tuned GPU sgemm schedules at 3072^3: generator1 and generator2 stage the operands by
+# hand (explicit LDS copies, double-buffered in generator1; 16x6 register tile), generator3 uses
+# cache_shared (16x8 register tile).  Their wrapper needs CUDA headers, so the tests drive the generated
+# function themselves; each program times its kernel through an external get_time(): timer_hook.c.
+SGEMM_TUNED = ["benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator%d.cpp" % n for n in (1, 2, 3)]
 
 
-def build_sgemm_tuned():
+def build_sgemm_tuned(rel):
     bdir = os.path.join(HERE, "build")
-    work = os.path.join(bdir, "sgemm_generator3")
+    stem = "sgemm_" + os.path.splitext(os.path.basename(rel))[0]
+    work = os.path.join(bdir, stem)
     os.makedirs(work, exist_ok=True)
-    src = os.path.join(REFERENCE, SGEMM_TUNED)
+    src = os.path.join(REFERENCE, rel)
     gen = os.path.join(work, "gen")
     build._run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
                 "-I" + os.path.dirname(src), "-o", gen, src, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG])
     build._run([gen], cwd=work)                      # writes fct.o (function "matmul") into its working directory
     build._run(["gcc", "-O2", "-fPIC", "-shared", "-o", library("get_time"), os.path.join(HERE, "timer_hook.c")])
-    build._run(["g++", "-shared", "-o", library("sgemm_generator3"), os.path.join(work, "fct.o"), "-L" + build.PKG,
+    build._run(["g++", "-shared", "-o", library(stem), os.path.join(work, "fct.o"), "-L" + build.PKG,
                 "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
@@ -93,9 +95,10 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", generator_rel, "+", os.path.basename(wrapper_rel), flush=True)
         build_test(generator_rel, wrapper_rel)
-    if verbose:
-        print("[reference programs]", SGEMM_TUNED, flush=True)
-    build_sgemm_tuned()
+    for rel in SGEMM_TUNED:
+        if verbose:
+            print("[reference programs]", rel, flush=True)
+        build_sgemm_tuned(rel)
     return True
 
 

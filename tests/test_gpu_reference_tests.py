@@ -8,6 +8,7 @@ reference tree), compiled by the HIP back-end, called through the C ABI and comp
 Inputs are small integers, as in the reference's wrappers, so fp32 results are exact and every
 comparison is bit-for-bit."""
 import os
+import re
 
 import numpy as np
 import pytest
@@ -163,14 +164,17 @@ def test_sgemm_library_call(programs_dir, M, N, K, alpha, beta, pad, off):
     assert np.array_equal(C, expected, equal_nan=True)
 
 
-def test_sgemm_cache_shared_register_tile(programs_dir):
-    # generator3-style staged sgemm: LDS tiles via cache_shared, 4x2 register tile, alpha/beta
+@pytest.mark.parametrize("name,kind", [("sgemm_shared_regs", "mfma-contraction"), ("sgemm_shared_regs_generic", "generic")])
+def test_sgemm_cache_shared_register_tile(programs_dir, name, kind):
+    # generator3-style staged sgemm: LDS tiles via cache_shared, 4x2 register tile, alpha/beta;
+    # once through the MFMA kernel (tiles and register tile proven sound), once as scheduled
+    assert re.search(r"^// _kernel_\d+: " + kind, open(os.path.join(programs_dir, "build", name + ".o.hip")).read(), re.M)
     rng = np.random.RandomState(3)
     M, N, K = 256, 192, 64
     A, B, C = ints(rng, (M, K)), ints(rng, (K, N)), ints(rng, (M, N))
     scal = np.array([3.0, 2.0], np.float32)
     expected = ref.sgemm(A, B, C, 3.0, 2.0)
-    runtime.load(programs_dir, "sgemm_shared_regs")(scal, A, B, C)
+    runtime.load(programs_dir, name)(scal, A, B, C)
     assert np.array_equal(C, expected)
 
 

@@ -112,25 +112,35 @@ def test_reference_gpu_test_passes(name):
     assert lib.tiramisu_wrapper_main(0, None) == 0
 
 
-def test_reference_tuned_sgemm_library_exports_its_function():
-    if not os.path.exists(library("sgemm_generator3")):
+TUNED_SGEMM = {"sgemm_generator1": "generic", "sgemm_generator2": "generic", "sgemm_generator3": "mfma-contraction"}
+
+
+@pytest.mark.parametrize("name", sorted(TUNED_SGEMM))
+def test_reference_tuned_sgemm_library(name):
+    """The hand-staged schedules stay as scheduled; the cache_shared one is proven a dense
+    contraction (LDS tiles cover their reads, register tile private) and gets the MFMA kernel."""
+    if not os.path.exists(library(name)):
         pytest.skip("reference tree was absent when the libraries were built")
     runtime.wrappers()
     ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
-    assert hasattr(ctypes.CDLL(library("sgemm_generator3")), "matmul")
+    assert hasattr(ctypes.CDLL(library(name)), "matmul")
+    text = open(os.path.join(HERE, "reference_programs", "build", name, "fct.o.hip")).read()
+    assert ("// _kernel_0: " + TUNED_SGEMM[name]) in text
 
 
 @pytest.mark.gpu
-def test_reference_tuned_sgemm_schedule():
-    """benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp, unchanged: 3072^3 with a 16x8
-    register tile per thread, k split by 4 and both operands staged with cache_shared; it copies
-    A, B, C to the GPU, times its kernel with get_time() and copies C back.  Its own wrapper needs
-    CUDA headers, so the generated function is called here; small integer data keeps every sum
-    exact, so the comparison with a float64 product is for equality."""
-    if not os.path.exists(library("sgemm_generator3")):
+@pytest.mark.parametrize("name", sorted(TUNED_SGEMM))
+def test_reference_tuned_sgemm_schedule(name):
+    """benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator{1,2,3}.cpp, unchanged: 3072^3 with a
+    16x6 (16x8 in generator3) register tile per thread and LDS tiles of both operands, staged by
+    hand in generator1 (double-buffered) and generator2, with cache_shared in generator3.  Each
+    copies A, B, C to the GPU, times its kernel with get_time() and copies C back.  Their wrapper
+    needs CUDA headers, so the generated function is called here; small integer data keeps every
+    sum exact, so the comparison with a float64 product is for equality."""
+    if not os.path.exists(library(name)):
         pytest.skip("reference tree was absent when the libraries were built")
     ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
-    program = runtime.Program(library("sgemm_generator3"), "matmul")
+    program = runtime.Program(library(name), "matmul")
     n = 3072
     rng = np.random.RandomState(3072)
     A = rng.randint(-2, 3, (n, n)).astype(np.float32)
@@ -146,4 +156,4 @@ def test_reference_tuned_sgemm_schedule():
         assert np.array_equal(C, expected)
         ms = float(t1[0] - t0[0])
         best = ms if best is None else min(best, ms)
-    print("generator3 kernel: %.3f ms, %.1f TFLOP/s" % (best, 2.0 * n ** 3 / best / 1e9), flush=True)
+    print("%s kernel: %.3f ms, %.1f TFLOP/s" % (name, best, 2.0 * n ** 3 / best / 1e9), flush=True)

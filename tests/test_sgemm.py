@@ -93,6 +93,23 @@ def test_gpu_uniform_inputs_within_tolerance(M, N, K):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,tile", [(2048, 2048, 48, "128x128x16"), (3072, 3072, 32, "192x192x16"),
+                                        (1024, 1024, 1024, "64x64x32"), (4096, 4096, 4096, "256x256x16")])
+def test_gpu_tile_chosen_for_the_launch(M, N, K, tile):
+    """The C tile is the one whose launch is modelled fastest on 256 compute units; the two
+    sizes that no other test reaches are also checked for exact results on integer data."""
+    text = open(os.path.join(PROGRAMS, "build", name_of(M, N, K) + ".o.hip")).read()
+    assert ("tile " + tile + ",") in text
+    if K > 64:
+        return
+    rng = np.random.RandomState(M + K)
+    A, B, C = ints(rng, (M, K)), ints(rng, (K, N)), ints(rng, (M, N))
+    scal = np.array([3.0, 2.0], np.float32)
+    expected = ref.sgemm(A, B, C, 3.0, 2.0)
+    assert np.array_equal(run_gpu(M, N, K, scal, A, B, C), expected)
+
+
+@pytest.mark.gpu
 def test_gpu_4096_closed_form_and_sampled_rows():
     M = N = K = 4096
     scal = np.array([1.0, 0.0], np.float32)

@@ -29,6 +29,7 @@ struct lowering {
     function *f;
     std::vector<node_ptr> leaves;
     int placeholder_counter = 0;
+    bool as_written = false;   // lower expressions as they were before cache_shared() redirected loads
 
     primitive_t scalar_type(const std::string &nm) const {
         for (auto c : f->get_invariants())
@@ -209,7 +210,7 @@ struct lowering {
             n->iterators[names[i - 1]] = from_isl(a, {});
             isl_ast_expr_free(a);
         }
-        const expr &e = C->get_expr();
+        const expr &e = (as_written && C->get_uncached_expr().is_defined()) ? C->get_uncached_expr() : C->get_expr();
         auto find_buffer = [&](const std::string &bn) {
             auto it = f->get_buffers().find(bn);
             if (it == f->get_buffers().end()) ERROR("unknown buffer " + bn + " in " + C->get_name(), true);
@@ -445,7 +446,7 @@ void function::gen_isl_ast() {
 
 namespace lir {
 
-node_ptr canonical_nest(function &f, computation &c) {
+node_ptr canonical_nest(function &f, computation &c, bool as_written) {
     isl_ctx *ctx = f.get_isl_ctx();
     int n = isl_set_dim(c.get_iteration_domain(), isl_dim_set);
     std::vector<std::string> in;
@@ -457,6 +458,7 @@ node_ptr canonical_nest(function &f, computation &c) {
     m = isl_map_intersect_domain(m, d);
     lowering lw;
     lw.f = &f;
+    lw.as_written = as_written;
     isl_ast_build *build = f.get_program_context() ? isl_ast_build_from_context(isl_set_copy(f.get_program_context()))
                                                    : isl_ast_build_alloc(ctx);
     build = isl_ast_build_set_at_each_domain(build, &at_each_domain, &lw);

@@ -1092,6 +1092,7 @@ computation *computation::cache_shared(computation &inp, const var &level, const
     input *new_access = new input(prefix + "_access", access_vars, inp.get_data_type());
     global::set_auto_data_mapping(saved);
     new_access->store_in(shared, access_exprs);
+    if (!uncached_expression.is_defined()) uncached_expression = expression;
     set_expression(expression.substitute_access(inp.get_name(), new_access->get_name()));
 
     int gpu_level = std::get<0>(thread_dims);
@@ -1168,7 +1169,81 @@ computation *computation::cache_shared(computation &inp, const var &level, const
         if (pred != nullptr) decl->between(*pred, fct->sched_graph[pred][curr], *curr, gpu_level);
         else decl->before(*curr, gpu_level);
     }
+    shared_cache rec;
+    rec.input = inp.get_name();
+    rec.access = new_access->get_name();
+    rec.shape = buffer_shape;
+    rec.offsets = copy_offsets;
+    rec.copy_level = copy_level;
+    rec.apparatus = {decl, copy, sync1, sync2};
+    for (computation *c : rec.apparatus) c->cache_consumer = this;
+    shared_caches.push_back(rec);
     return new_access;
+}
+
+bool computation::shared_caches_cover_reads() const {
+    if (shared_caches.empty()) return true;
+    if (!uncached_expression.is_defined() || predicate.is_defined()) return false;
+    const int nl = (int)level_names.size();
+    // iteration-domain dimensions are renamed: a loop level may carry an iterator's name with another value
+    std::map<std::string, std::string> rename;
+    std::vector<std::string> dom_names;
+    for (size_t d = 0; d < iterator_names_.size(); d++) {
+        dom_names.push_back("_it" + std::to_string(d));
+        rename[iterator_names_[d]] = dom_names.back();
+    }
+    std::map<std::string, expr> rename_subs;
+    for (auto &r : rename) rename_subs[r.first] = expr(var(global::get_loop_iterator_data_type(), r.second));
+    auto renamed = [&](const expr &e) { return e.substitute(rename_subs); };
+    std::vector<std::string> range = {"_dup"};
+    for (int l = 0; l <= nl; l++) {
+        range.push_back("_s" + std::to_string(l));
+        if (l < nl) range.push_back(level_names[l]);
+    }
+    std::set<std::string> params;
+    for (int i = 0; i < (int)isl_set_dim(iteration_domain, isl_dim_param); i++)
+        params.insert(isl_set_get_dim_name(iteration_domain, isl_dim_param, i));
+    std::vector<std::string> bad;
+    for (const shared_cache &sc : shared_caches) {
+        std::vector<std::vector<expr>> reads;
+        uncached_expression.visit([&](const expr &x) {
+            if (x.get_expr_type() == e_op && x.get_op_type() == o_access && x.get_name() == sc.input) reads.push_back(x.get_access());
+        });
+        if (reads.empty()) return false;
+        for (size_t d = 0; d < sc.shape.size(); d++) {
+            // the tile origin may depend on the loop levels down to the copy level only
+            bool names_ok = true;
+            sc.offsets[d].visit([&](const expr &x) {
+                if (x.get_expr_type() != e_var) return;
+                auto it = std::find(level_names.begin(), level_names.end(), x.get_name());
+                if (it == level_names.end() ? !params.count(x.get_name()) : (it - level_names.begin()) > sc.copy_level) names_ok = false;
+            });
+            if (!names_ok) return false;
+            bool ok = true;
+            const std::string off = expr_to_isl_str(sc.offsets[d], ok), n = std::to_string(sc.shape[d]);
+            if (!ok) return false;
+            bad.push_back("(" + off + ") mod " + n + " != 0");
+            for (auto &idx : reads) {
+                if (idx.size() != sc.shape.size()) return false;
+                const std::string at = expr_to_isl_str(renamed(idx[d]), ok);
+                if (!ok) return false;
+                bad.push_back(at + " < " + off);
+                bad.push_back(at + " >= " + off + " + " + n);
+            }
+        }
+    }
+    std::vector<std::string> pv(params.begin(), params.end());
+    const std::string text = params_prefix(pv) + "{ " + name + "[" + join(dom_names, ", ") + "] -> [" + join(range, ", ") + "] : " +
+                             join(bad, " or ") + " }";
+    isl_map *violations = isl_map_read_from_str(ctx, text.c_str());
+    if (!violations) return false;
+    isl_set *dom = isl_set_copy(iteration_domain);
+    if (fct->get_program_context()) dom = isl_set_intersect_params(dom, isl_set_copy(fct->get_program_context()));
+    isl_map *sched = isl_map_intersect_domain(isl_map_copy(schedule), dom);
+    violations = isl_map_intersect(sched, violations);   // positional: dimension names play no part
+    const bool covered = isl_map_is_empty(violations) == isl_bool_true;
+    isl_map_free(violations);
+    return covered;
 }
 
 void computation::gen_time_space_domain() {

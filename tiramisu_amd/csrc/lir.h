@@ -96,8 +96,9 @@ std::string dump(const node_ptr &n, int indent = 0);
   * over the computation's iteration-domain dimensions ("c0", "c1", ... outermost first; a
   * dimension with a single value has no loop) with one leaf whose index expressions and value
   * are written in those iterators: the canonical, schedule-independent form that the pattern
-  * recognisers analyse. */
-node_ptr canonical_nest(function &f, computation &c);
+  * recognisers analyse.  With \p as_written the value is the computation's expression from before
+  * cache_shared() redirected its loads to LDS tiles. */
+node_ptr canonical_nest(function &f, computation &c, bool as_written = false);
 
 /** d e / d v for an expression that is affine in variable \p v (other symbols are constants);
   * sets \p ok to false when e is not affine in v. */

@@ -300,7 +300,7 @@ struct canon {
 bool canonicalize(function *f, const node_ptr &real, const std::set<std::string> &inner, canon &out) {
     out.comp = real->comp;
     out.real = real;
-    node_ptr n = lir::canonical_nest(*f, *real->comp);
+    node_ptr n = lir::canonical_nest(*f, *real->comp, true);
     const auto &names = real->comp->get_iteration_domain_dimension_names();
     out.dims.resize(names.size());
     for (size_t p = 0; p < names.size(); p++) {
@@ -337,6 +337,118 @@ bool canonicalize(function *f, const node_ptr &real, const std::set<std::string>
             if (lir::mentions(it->second, in)) d.in_kernel = true;
     }
     return true;
+}
+
+// ---- per-thread accumulators, proven on the schedule ---------------------------------------
+//
+// A private accumulator (registers, or a per-thread array addressed by tile remainders) ties an
+// initialisation, an update and an epilogue together only through the schedule: statement X
+// belongs with update instance U[...] when both run in the same thread of the same launch and
+// touch the same accumulator element.  The relation is built from the schedules and access
+// relations, so the pairing of dimensions does not depend on how the generated loops are named
+// or nested (register tiles interchanged below the reduction loop, for instance).
+
+// instance -> values of the loop levels from the outermost down to the innermost thread level
+isl_map *thread_of(function *f, computation *c, int &depth) {
+    int last = -1;
+    for (int l = 0; l < c->get_loop_levels_number(); l++)
+        if (f->gpu_thread_position(c->get_name(), l) >= 0) last = l;
+    if (last < 0) return nullptr;
+    depth = last + 1;
+    isl_set *dom = isl_set_copy(c->get_iteration_domain());
+    if (f->get_program_context()) dom = isl_set_intersect_params(dom, isl_set_copy(f->get_program_context()));
+    isl_map *m = isl_map_intersect_domain(isl_map_copy(c->get_schedule()), dom);
+    for (int pos = (int)isl_map_dim(m, isl_dim_out) - 1; pos >= 0; pos--) {
+        const bool keep = pos >= 2 && pos % 2 == 0 && (pos - 2) / 2 <= last;
+        if (!keep) m = isl_map_project_out(m, isl_dim_out, pos, 1);
+    }
+    return m;
+}
+
+// instance of x -> accumulator element: its own store when x writes the accumulator buffer,
+// else the element of the update (or initialisation) instance that its expression reads
+isl_map *accumulator_element_of(computation *x, const std::vector<computation *> &writers, const std::string &acc_buffer) {
+    if (x->get_access_relation() && acc_buffer == isl_map_get_tuple_name(x->get_access_relation(), isl_dim_out))
+        return isl_map_copy(x->get_access_relation());
+    for (computation *w : writers) {
+        std::vector<expr> args;
+        x->get_expr().visit([&](const expr &e) {
+            if (args.empty() && e.get_expr_type() == e_op && e.get_op_type() == o_access && e.get_name() == w->get_name()) args = e.get_access();
+        });
+        if (args.empty() || !w->get_access_relation()) continue;
+        std::vector<std::string> to;
+        bool ok = true;
+        for (auto &a : args) to.push_back(expr_to_isl_str(a, ok));
+        if (!ok) return nullptr;
+        const std::string text = "{ " + x->get_name() + "[" + join(x->get_iteration_domain_dimension_names(), ", ") + "] -> " +
+                                 w->get_name() + "[" + join(to, ", ") + "] }";
+        isl_map *m = isl_map_read_from_str(x->get_ctx(), text.c_str());
+        if (!m) return nullptr;
+        return isl_map_apply_range(m, isl_map_copy(w->get_access_relation()));
+    }
+    return nullptr;
+}
+
+// { x[...] -> u[...] : same thread of the same launch, same accumulator element }
+isl_map *same_thread_same_element(function *f, computation *x, computation *u, const std::vector<computation *> &writers,
+                                  const std::string &acc_buffer) {
+    int dx = 0, du = 0;
+    isl_map *tx = thread_of(f, x, dx), *tu = thread_of(f, u, du);
+    isl_map *ex = accumulator_element_of(x, writers, acc_buffer), *eu = accumulator_element_of(u, writers, acc_buffer);
+    if (!tx || !tu || !ex || !eu || dx != du ||
+        isl_map_dim(ex, isl_dim_out) != isl_map_dim(eu, isl_dim_out) ||
+        std::string(isl_map_get_tuple_name(ex, isl_dim_out)) != isl_map_get_tuple_name(eu, isl_dim_out)) {
+        for (isl_map *m : {tx, tu, ex, eu}) if (m) isl_map_free(m);
+        return nullptr;
+    }
+    return isl_map_apply_range(isl_map_range_product(tx, ex), isl_map_reverse(isl_map_range_product(tu, eu)));
+}
+
+bool forces_equal(isl_map *r, int in_pos, int out_pos) {
+    isl_map *e = isl_map_equate(isl_map_copy(r), isl_dim_in, in_pos, isl_dim_out, out_pos);
+    const bool yes = isl_map_is_subset(r, e) == isl_bool_true;
+    isl_map_free(e);
+    return yes;
+}
+
+// Pairs every in-kernel dimension of x with the dimension of the update that always carries the
+// same value in related instances (pairs[q] = p, or -1 for the other dimensions of x).  Fails
+// when some in-kernel dimension has no partner, when two share one, or when some update
+// instance has no related instance of x.
+bool pair_through_accumulator(function *f, const canon &x, const canon &u, const std::vector<computation *> &writers,
+                              const std::string &acc_buffer, std::vector<int> &pairs) {
+    isl_map *r = same_thread_same_element(f, x.comp, u.comp, writers, acc_buffer);
+    if (!r) return false;
+    bool ok = isl_map_is_empty(r) == isl_bool_false;
+    pairs.assign(x.dims.size(), -1);
+    std::set<int> taken;
+    for (size_t q = 0; q < x.dims.size() && ok; q++) {
+        if (!x.dims[q].in_kernel || !x.dims[q].lo.is_defined()) continue;
+        for (size_t p = 0; p < u.dims.size() && pairs[q] < 0; p++)
+            if (u.dims[p].in_kernel && u.dims[p].lo.is_defined() && !taken.count((int)p) && forces_equal(r, (int)q, (int)p)) pairs[q] = (int)p;
+        if (pairs[q] < 0) ok = false; else taken.insert(pairs[q]);
+    }
+    if (ok) {
+        isl_set *served = isl_map_range(isl_map_copy(r));
+        isl_set *all = isl_set_copy(u.comp->get_iteration_domain());
+        if (f->get_program_context()) all = isl_set_intersect_params(all, isl_set_copy(f->get_program_context()));
+        ok = isl_set_is_subset(all, served) == isl_bool_true;
+        isl_set_free(served);
+        isl_set_free(all);
+    }
+    isl_map_free(r);
+    return ok;
+}
+
+// Within a thread, update instances that share an accumulator element agree on every one of
+// the given dimensions: no two results of the thread live in the same element.
+bool accumulator_elements_are_private(function *f, const canon &u, const std::vector<int> &spatial, const std::string &acc_buffer) {
+    isl_map *r = same_thread_same_element(f, u.comp, u.comp, {u.comp}, acc_buffer);
+    if (!r) return false;
+    bool ok = true;
+    for (int p : spatial) ok = ok && forces_equal(r, p, p);
+    isl_map_free(r);
+    return ok;
 }
 
 void flatten_sum(const expr &e, std::vector<expr> &terms) {
@@ -416,10 +528,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     function *f = ctx.f;
     std::set<std::string> inner;
     std::vector<node_ptr> leaves;
+    // LDS tiles that the schedule installed with cache_shared(): their declaration, cooperative
+    // copy and barriers are left out, and the computation they serve is analysed as written,
+    // once each tile is proven to hold what the computation reads through it.
+    std::set<computation *> cached;
     bool bad = false;
     lir::walk(root, [&](const node_ptr &x) {
         if (x->kind == node_kind::loop) inner.insert(x->iterator);
         if (x->kind != node_kind::leaf) return;
+        if (x->comp && x->comp->get_cache_consumer()) { cached.insert(x->comp->get_cache_consumer()); return; }
         if (x->lkind == leaf_kind::allocate || x->lkind == leaf_kind::release) {
             if (x->target->get_location() == memory_location::global || x->target->get_location() == memory_location::host) bad = true;
             return;
@@ -428,6 +545,13 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         leaves.push_back(x);
     });
     if (bad || leaves.empty() || leaves.size() > 3) return reject(2);
+    for (computation *c : cached) {
+        bool in_nest = false;
+        for (auto &l : leaves) in_nest |= l->comp == c;
+        if (!in_nest || !c->shared_caches_cover_reads()) return reject(26);
+    }
+    for (auto &l : leaves)   // every tile of a cached computation must have been seen in this nest
+        if (!l->comp->get_shared_caches().empty() && !cached.count(l->comp)) return reject(26);
 
     // ---- find the update: own element + products of loads
     int ui = -1;
@@ -485,6 +609,28 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         }
         (is_spatial ? spatial : reduction).push_back((int)p);
     }
+    // register tiles nested differently in the fused statements: pair dimensions on the schedule instead
+    std::map<int, std::vector<int>> paired;   // leaf index -> dimension of that leaf -> dimension of the update
+    if (acc_private && has_init && (spatial.size() < 2 || reduction.empty())) {
+        std::vector<computation *> writers = {U.comp, cs[ii].comp};
+        const std::string acc_name = acc_buf->get_name();
+        std::vector<int> pi;
+        if (!pair_through_accumulator(f, cs[ii], U, writers, acc_name, pi)) return reject(6);
+        spatial.clear();
+        reduction.clear();
+        std::set<int> sp;
+        for (int p : pi) if (p >= 0) sp.insert(p);
+        for (size_t p = 0; p < U.dims.size(); p++)
+            if (U.dims[p].in_kernel && U.dims[p].lo.is_defined()) (sp.count((int)p) ? spatial : reduction).push_back((int)p);
+        if (!accumulator_elements_are_private(f, U, spatial, acc_name)) return reject(6);
+        paired[ii] = pi;
+        const int ei_ = ui + 1;
+        if (ei_ < (int)leaves.size()) {
+            std::vector<int> pe;
+            if (!pair_through_accumulator(f, cs[ei_], U, writers, acc_name, pe)) return reject(6);
+            paired[ei_] = pe;
+        }
+    }
     if (spatial.size() < 2 || reduction.empty()) return reject(6);
 
     // ---- the GEMM view: N dimensions are the spatial dimensions of the factor that involves the
@@ -534,13 +680,18 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
 
     // initialisation / epilogue: their in-kernel dimensions must be spatial dimensions of the update
     auto bind_to_update = [&](canon &c) -> bool {
+        const std::vector<int> *proven = nullptr;
+        for (auto &pr : paired)
+            if (&cs[pr.first] == &c) proven = &pr.second;
         for (size_t p = 0; p < c.dims.size(); p++) {
             canon_dim &d = c.dims[p];
             if (!d.lo.is_defined() || !d.in_kernel) continue;
             const expr mine = lir::simplify(c.real->iterators.at(d.name));
             int match = -1;
-            for (int sp : spatial)
-                if (mine.is_equal(lir::simplify(ureal->iterators.at(U.dims[sp].name)))) match = sp;
+            if (proven) match = (*proven)[p];
+            else
+                for (int sp : spatial)
+                    if (mine.is_equal(lir::simplify(ureal->iterators.at(U.dims[sp].name)))) match = sp;
             if (match < 0) return false;
             if (!lir::simplify(d.lo).is_equal(lir::simplify(U.dims[match].lo)) || !lir::simplify(d.hi).is_equal(lir::simplify(U.dims[match].hi)))
                 return false;
@@ -555,7 +706,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     if (!out_buf) return reject(7);
 
     // the accumulator element is the same in all fused statements (compared in the scheduled program)
-    if (has_init && (leaves[ii]->lhs != acc_buf || !same_element(expr(o_access, acc_buf->get_name(), leaves[ii]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
+    if (has_init && (leaves[ii]->lhs != acc_buf ||
+                     (paired.empty() && !same_element(expr(o_access, acc_buf->get_name(), leaves[ii]->lhs_index, p_float32), acc_buf, ureal->lhs_index))))
         return reject(13);
     if (has_init && reads_buffer(cs[ii].leaf->rhs, acc_buf->get_name())) return reject(14);
 
@@ -657,9 +809,24 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
     int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2, WGK = 1, DEPTH = 1;
     if (lit) {
-        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0) { BM = BN = 256; PADX = 0; }
-        else if (((Ml + 127) / 128) * ((Nl + 127) / 128) >= 256 && Ml >= 128) { BM = BN = 128; }
-        else if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
+        if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
+        else {
+            // square tiles: the one whose launch is modelled fastest.  A compute unit works through
+            // ceil(tiles / 256) tiles, each costing its area over the fraction of the MFMA rate that
+            // a tile of that size sustains (larger tiles re-read less through LDS).  256 and 192
+            // are for whole tiles only; 192 is what makes 3072 = 16 x 192 one tile per compute unit.
+            struct candidate { int tile; double rate; bool whole_only; };
+            const candidate cands[] = {{256, 1.0, true}, {192, 0.9, true}, {128, 0.8, false}, {64, 0.68, false}};
+            double best = 0;
+            for (const candidate &c : cands) {
+                if (c.whole_only && (Ml % c.tile != 0 || Nl % c.tile != 0)) continue;
+                if (c.tile == 128 && Ml < 128) continue;
+                const long tiles = ((Ml + c.tile - 1) / c.tile) * ((Nl + c.tile - 1) / c.tile);
+                const double cost = (double)((tiles + 255) / 256) * c.tile * c.tile / c.rate;
+                if (best == 0 || cost < best) { best = cost; BM = BN = c.tile; }
+            }
+            PADX = BM == 256 ? 0 : 1;
+        }
     }
     if (BM == 64 && BN == 64) BK = 32;   // one 32x32 tile per wavefront: longer slices, fewer barriers per flop
     // few C tiles but a long reduction (a batch-sized M against wide weights, as in recurrent cells):

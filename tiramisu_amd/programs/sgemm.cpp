@@ -82,5 +82,7 @@ int main()
     generate(100, 70, 50);        // ragged: guarded tile edges
     generate(33, 17, 9);
     generate(64, 256, 512);       // few C tiles, long reduction: wavefront groups split K inside a workgroup
+    generate(2048, 2048, 48);     // 256 tiles of 128x128
+    generate(3072, 3072, 32);     // 256 tiles of 192x192 (the size of the reference's GPU sgemm benchmark)
     return 0;
 }
