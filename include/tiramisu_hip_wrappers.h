@@ -70,6 +70,20 @@ void *tiramisu_hip_module_get_global(void *module, const char *name, uint64_t by
 int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3],
                         uint32_t dynamic_lds_bytes, void **args);
 
+/* ---- host loops tagged parallel around GPU work.  The reference lowers such a loop to a Halide
+ *      parallel loop (ForType::Parallel, tiramisu_codegen_halide.cpp:2104-2145): its iterations
+ *      run on pool threads, each on its own per-thread default stream, and the program
+ *      synchronises that stream before the iteration ends
+ *      (benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp:99-100, :133-135).  Here generated host
+ *      code hands the loop body to this call: body(i, closure) runs once for every i in
+ *      [first, last] on up to four pool threads, each with a stream of its own as its current
+ *      stream.  The caller's stream is synchronised before the first iteration starts and every
+ *      pool thread's stream before the call returns, so work before, inside and after the loop
+ *      is ordered as in the serial loop; iterations must be independent of one another.
+ *      Called from inside a parallel iteration, or with a single iteration, it runs the body
+ *      in the calling thread. ---- */
+void tiramisu_hip_parallel_for(int32_t first, int32_t last, void (*body)(int32_t, void *), void *closure);
+
 /* ---- stream and timing helpers for wrappers and benchmarks (the reference's
  *      benchmarks bracket device work with get_time() calls,
  *      benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp:66-69) ---- */
@@ -84,7 +98,7 @@ int tiramisu_hip_event_destroy(void *event);
 int tiramisu_hip_device_count(void);
 
 /* ---- per-launch timing.  Between profile_start and profile_stop every tiramisu_hip_launch
- *      (and GEMM library call) of the calling thread is bracketed by two events on the current
+ *      (and GEMM library call), from any thread, is bracketed by two events on its current
  *      stream; profile_stop waits for them and keeps one (kernel name, milliseconds) record
  *      per launch, readable until the next profile_start.  The reference has no counterpart:
  *      its benchmarks use nvprof (utils/run_gpu_bench.py). ---- */

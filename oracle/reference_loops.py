@@ -306,3 +306,4 @@ def lstm(weights, biases, x):
             below = h
         y[m] = below
     return y
+

@@ -60,25 +60,34 @@ def build_test(generator_rel, wrapper_rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
-# The reference's tuned GPU sgemm schedules at 3072^3: generator1 and generator2 stage the operands by
-# hand (explicit LDS copies, double-buffered in generator1; 16x6 register tile), generator3 uses
-# cache_shared (16x8 register tile).  Their wrapper needs CUDA headers, so the tests drive the generated
-# function themselves; each program times its kernel through an external get_time(): timer_hook.c.
-SGEMM_TUNED = ["benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator%d.cpp" % n for n in (1, 2, 3)]
+# Benchmark generators whose wrapper needs CUDA, cuBLAS or cuDNN headers: the tests drive the
+# generated function themselves.  Each program writes its object into its working directory and
+# (all but the first LSTM) times its kernels through an external get_time(): timer_hook.c.
+#  * sgemm at 3072^3: generator1 and generator2 stage the operands by hand (explicit LDS copies,
+#    double-buffered in generator1; 16x6 register tile), generator3 uses cache_shared (16x8).
+#  * LSTM: gpu/generator.cpp takes its sizes at run time and stages both matrix products through
+#    LDS by hand; gpu_lib/generator.cpp (4 layers, batch 64, 512 features, 100 steps) calls the
+#    library GEMM, batches the input products over 10 steps and walks (layer, step block)
+#    diagonally with skew + interchange under a parallel host loop.
+# (source below the reference tree, library stem, object the program writes):
+SELF_DRIVEN = [("benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator%d.cpp" % n, "sgemm_generator%d" % n, "fct.o")
+               for n in (1, 2, 3)] + [
+    ("benchmarks/DNN/blocks/LSTM/gpu/generator.cpp", "lstm_gpu", "lstm.o"),
+    ("benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp", "lstm_gpu_lib", "lstm.o"),
+]
 
 
-def build_sgemm_tuned(rel):
+def build_self_driven(rel, stem, obj):
     bdir = os.path.join(HERE, "build")
-    stem = "sgemm_" + os.path.splitext(os.path.basename(rel))[0]
     work = os.path.join(bdir, stem)
     os.makedirs(work, exist_ok=True)
     src = os.path.join(REFERENCE, rel)
     gen = os.path.join(work, "gen")
     build._run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
                 "-I" + os.path.dirname(src), "-o", gen, src, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG])
-    build._run([gen], cwd=work)                      # writes fct.o (function "matmul") into its working directory
+    build._run([gen], cwd=work)
     build._run(["gcc", "-O2", "-fPIC", "-shared", "-o", library("get_time"), os.path.join(HERE, "timer_hook.c")])
-    build._run(["g++", "-shared", "-o", library(stem), os.path.join(work, "fct.o"), "-L" + build.PKG,
+    build._run(["g++", "-shared", "-o", library(stem), os.path.join(work, obj), "-L" + build.PKG,
                 "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
@@ -95,10 +104,10 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", generator_rel, "+", os.path.basename(wrapper_rel), flush=True)
         build_test(generator_rel, wrapper_rel)
-    for rel in SGEMM_TUNED:
+    for rel, stem, obj in SELF_DRIVEN:
         if verbose:
             print("[reference programs]", rel, flush=True)
-        build_sgemm_tuned(rel)
+        build_self_driven(rel, stem, obj)
     return True
 
 

@@ -1,0 +1,58 @@
+"""tiramisu_hip_sgemm, the library GEMM behind cublas_gemm() (replaces tiramisu_cublas_sgemm,
+tiramisu_cuda_wrappers.cpp:74-115), called through the C ABI on every kernel configuration it
+dispatches to: the square tiles chosen for the launch (64, 128, 192, 256), guarded edges, the
+64-row split-K configuration with its four prefetch depths, transposed operands, leading
+dimensions and offsets.  Small integer data: every sum is exact, comparison for equality with a
+float64 product."""
+import numpy as np
+import pytest
+
+from tiramisu_amd import runtime
+
+pytestmark = pytest.mark.gpu
+
+
+def run(M, N, K, alpha, beta, tA=False, tB=False, pad=0, off=0, seed=0):
+    from gpu_util import DeviceArray
+    rng = np.random.RandomState(seed + M + N + K)
+    a_rows, a_cols = (K, M) if tA else (M, K)
+    b_rows, b_cols = (N, K) if tB else (K, N)
+    ldA, ldB, ldC = a_cols + pad, b_cols + pad, N + 2 * pad
+    A = rng.randint(-3, 4, a_rows * ldA + off).astype(np.float32)
+    B = rng.randint(-3, 4, b_rows * ldB + off + 4).astype(np.float32)
+    C = rng.randint(-3, 4, M * ldC + off + 8).astype(np.float32)
+    offA, offB, offC = off, off + 4 if off else 0, off + 8 if off else 0
+    a = A[offA:offA + a_rows * ldA].reshape(a_rows, ldA)[:, :a_cols].astype(np.float64)
+    b = B[offB:offB + b_rows * ldB].reshape(b_rows, ldB)[:, :b_cols].astype(np.float64)
+    expected = C.copy()
+    c = expected[offC:offC + M * ldC].reshape(M, ldC)[:, :N]
+    c[:] = alpha * ((a.T if tA else a) @ (b.T if tB else b)) + (beta * c if beta != 0 else 0)
+    dA, dB, dC = DeviceArray(A), DeviceArray(B), DeviceArray(C)
+    packed = pad == 0
+    runtime.wrappers().tiramisu_hip_sgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, alpha, beta, 0 if packed else ldA, 0 if packed else ldB,
+                                          0 if packed else ldC, offA, offB, offC, tA, tB)
+    out = dC.download()
+    assert np.array_equal(out, expected)
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 64, 64), (64, 64, 48), (100, 70, 50), (640, 2048, 512), (2048, 2048, 48),
+                                   (3072, 3072, 32), (4096, 4096, 64), (33, 17, 9), (8, 8, 4)])
+def test_square_tiles(M, N, K):
+    run(M, N, K, 1.0, 0.0)
+    run(M, N, K, 3.0, 2.0, seed=1)
+
+
+@pytest.mark.parametrize("K", [256, 384, 512, 1024])
+@pytest.mark.parametrize("tB", [False, True])
+def test_batch_of_64_rows_splits_k(K, tB):
+    # the recurrent product of an LSTM cell (benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp:76-84)
+    run(64, 2048, K, 1.0, 1.0, tB=tB)
+    run(64, 96, K, 2.0, 0.0, tB=tB, seed=2)
+
+
+@pytest.mark.parametrize("tA,tB", [(False, True), (True, False), (True, True)])
+def test_transposed_operands_padding_and_offsets(tA, tB):
+    run(128, 192, 96, 1.0, 1.0, tA=tA, tB=tB)
+    run(96, 80, 40, 2.0, 1.0, tA=tA, tB=tB, pad=4, off=12)
+    run(64, 2048, 512, 1.0, 1.0, tA=tA, tB=tB, pad=4, off=16)
+    run(50, 30, 20, 1.0, 0.0, tA=tA, tB=tB, pad=3, off=5)

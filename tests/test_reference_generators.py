@@ -157,3 +157,49 @@ def test_reference_tuned_sgemm_schedule(name):
         ms = float(t1[0] - t0[0])
         best = ms if best is None else min(best, ms)
     print("%s kernel: %.3f ms, %.1f TFLOP/s" % (name, best, 2.0 * n ** 3 / best / 1e9), flush=True)
+
+
+def lstm_inputs(L, B, H, S, seed):
+    rng = np.random.RandomState(seed)
+    bound = 1.0 / np.sqrt(H)
+    weights = rng.uniform(-bound, bound, (L, 2, 4 * H, H)).astype(np.float32)
+    biases = rng.uniform(-bound, bound, (L, 4 * H)).astype(np.float32)
+    x = rng.uniform(-1, 1, (S, B, H)).astype(np.float32)
+    return weights, biases, x
+
+
+@pytest.mark.parametrize("name", ["lstm_gpu", "lstm_gpu_lib"])
+def test_reference_lstm_library_exports_its_function(name):
+    """Both GPU LSTM generators compile and generate code unchanged.  Only gpu_lib's function is
+    run: gpu/generator.cpp maps its reads of the previous hidden state to rows {m - 1, l} of the
+    state buffer (:268, :280) while the states are stored at {m + 1, l + 1} (:295), so its first
+    step reads row -1, before the allocation."""
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    assert hasattr(ctypes.CDLL(library(name)), "lstm")
+
+
+@pytest.mark.gpu
+def test_reference_lstm_gpu_lib_generator():
+    """benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp, unchanged, at its own size (4 layers, batch
+    64, 512 features, 100 steps): weights transposed on the GPU, library GEMM calls with offsets
+    (input products batched over 10 steps), (layer, step block) walked diagonally after skew +
+    interchange, nonlinearities in one fused kernel per step.  The program times itself."""
+    if not os.path.exists(library("lstm_gpu_lib")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    L, B, H, S = 4, 64, 512, 100
+    weights, biases, x = lstm_inputs(L, B, H, S, 512)
+    program = runtime.Program(library("lstm_gpu_lib"), "lstm")
+    expected = ref.lstm(weights, biases, x)
+    best = None
+    for _ in range(3):
+        y = np.zeros((S, B, H), np.float32)
+        t0, t1 = np.zeros(1, np.float32), np.zeros(1, np.float32)
+        program(weights, biases, x, y, t0, t1)
+        assert np.max(np.abs(y - expected)) <= 1e-4 * np.max(np.abs(expected))
+        ms = float(t1[0] - t0[0])
+        best = ms if best is None else min(best, ms)
+    print("gpu_lib LSTM generator: %.3f ms" % best, flush=True)

@@ -333,6 +333,22 @@ struct host_gen {
 
     host_gen(context &c) : ctx(c), f(c.f) { hp.fct = f; }
 
+    // A host loop tagged parallel is handed to the runtime's pool when its iterations can run
+    // side by side as emitted: unit stride, not nested in another such loop, and no buffer
+    // allocated or released in its body (those assign variables of the enclosing function).
+    bool in_parallel_loop = false;
+    int parallel_loops = 0;
+    bool runs_in_parallel(const node_ptr &n) const {
+        if (!n->parallel || in_parallel_loop || std::getenv("TIRAMISU_HIP_SERIAL_HOST_LOOPS")) return false;
+        const expr inc = lir::simplify(n->increment);
+        if (!inc.is_integer_literal() || inc.get_int_val() != 1) return false;
+        bool ok = true;
+        lir::walk(n->body, [&](const node_ptr &x) {
+            if (x->kind == node_kind::leaf && (x->lkind == leaf_kind::allocate || x->lkind == leaf_kind::release)) ok = false;
+        });
+        return ok;
+    }
+
     static bool is_gpu_loop(const node_ptr &n) { return n->kind == node_kind::loop && (n->gpu_block >= 0 || n->gpu_thread >= 0); }
 
     void require_host(const buffer *b, const std::string &who) {
@@ -379,6 +395,21 @@ struct host_gen {
                 if (emit_stencil(ctx, nullptr, n, plan)) {
                     for (auto &k : plan.kernels) ctx.kernels.push_back(k);
                     out << plan.host_code;
+                    break;
+                }
+                if (runs_in_parallel(n)) {
+                    // iterations on pool threads, each with a stream of its own (what the reference's
+                    // Halide parallel loop around kernel calls does: tiramisu_codegen_halide.cpp:2104-2145)
+                    const std::string body = "_parallel_body_" + std::to_string(parallel_loops++);
+                    out << pad(ind) << "{\n";
+                    out << pad(ind + 1) << "auto " << body << " = [&](int32_t " << n->iterator << ") {\n";
+                    in_parallel_loop = true;
+                    emit(n->body, ind + 2);
+                    in_parallel_loop = false;
+                    out << pad(ind + 1) << "};\n";
+                    out << pad(ind + 1) << "tiramisu_hip_parallel_for(" << hp.print(n->init) << ", " << hp.print(n->upper)
+                        << ", [](int32_t _i, void *_p) { (*static_cast<decltype(" << body << ") *>(_p))(_i); }, (void *)&" << body << ");\n";
+                    out << pad(ind) << "}\n";
                     break;
                 }
                 out << pad(ind) << "for (int32_t " << n->iterator << " = " << hp.print(n->init) << "; " << n->iterator

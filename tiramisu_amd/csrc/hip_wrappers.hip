@@ -5,12 +5,16 @@
 // build's own MFMA kernel instead of a vendor BLAS.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <atomic>
+#include <condition_variable>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/tiramisu_hip_wrappers.h"
@@ -33,14 +37,14 @@ struct launch_record {
     hipEvent_t start, stop;
     float ms;
 };
-thread_local bool profiling = false;
-thread_local std::vector<launch_record> records;
+std::atomic<bool> profiling{false};
+std::vector<launch_record> records;     // guarded by records_mutex: launches may come from pool threads
+std::mutex records_mutex;
 std::mutex names_mutex;
 std::map<void *, std::string> function_names;
 
 struct scoped_record {
     bool on;
-    size_t idx = 0;
     scoped_record(const std::string &name) : on(profiling) {
         if (!on) return;
         launch_record r;
@@ -49,13 +53,71 @@ struct scoped_record {
         check(hipEventCreate(&r.start), "tiramisu_hip_profile");
         check(hipEventCreate(&r.stop), "tiramisu_hip_profile");
         check(hipEventRecord(r.start, current_stream), "tiramisu_hip_profile");
+        stop = r.stop;
+        std::lock_guard<std::mutex> g(records_mutex);
         records.push_back(r);
-        idx = records.size() - 1;
     }
     ~scoped_record() {
-        if (on) check(hipEventRecord(records[idx].stop, current_stream), "tiramisu_hip_profile");
+        if (on) check(hipEventRecord(stop, current_stream), "tiramisu_hip_profile");
+    }
+    hipEvent_t stop = nullptr;
+};
+
+// ---- pool for host loops tagged parallel.  Threads are created on first use and live until
+// the process ends (the state is never destroyed, so nothing is torn down under a waiting thread).
+struct parallel_pool {
+    static constexpr int WORKERS = 4;   // as many as there are hardware queues per process by default
+    std::mutex m;
+    std::condition_variable wake, done;
+    std::vector<std::thread> threads;
+    // the job being run (one at a time: jobs_mutex serialises callers)
+    std::mutex jobs_mutex;
+    void (*body)(int32_t, void *) = nullptr;
+    void *closure = nullptr;
+    int32_t next = 0, last = -1;
+    long generation = 0;
+    int active = 0;
+
+    void worker() {
+        hipStream_t s;
+        check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "tiramisu_hip_parallel_for");
+        current_stream = s;
+        long seen = 0;
+        std::unique_lock<std::mutex> lk(m);
+        for (;;) {
+            wake.wait(lk, [&] { return generation != seen; });
+            seen = generation;
+            while (next <= last) {
+                const int32_t i = next++;
+                lk.unlock();
+                body(i, closure);
+                lk.lock();
+            }
+            lk.unlock();
+            check(hipStreamSynchronize(s), "tiramisu_hip_parallel_for");
+            lk.lock();
+            if (--active == 0) done.notify_all();
+        }
+    }
+
+    void run(int32_t first, int32_t last_, void (*b)(int32_t, void *), void *c) {
+        std::lock_guard<std::mutex> one(jobs_mutex);
+        std::unique_lock<std::mutex> lk(m);
+        while ((int)threads.size() < WORKERS) {
+            threads.emplace_back([this] { worker(); });
+            threads.back().detach();
+        }
+        body = b;
+        closure = c;
+        next = first;
+        last = last_;
+        active = WORKERS;
+        generation++;
+        wake.notify_all();
+        done.wait(lk, [&] { return active == 0; });
     }
 };
+thread_local bool in_parallel_iteration = false;
 
 // One thread per element of C; any strides, any sizes.  Used for double precision and for
 // shapes the MFMA path does not take.
@@ -80,25 +142,56 @@ void launch_mfma(const float *A, const float *B, float *C, int M, int N, int K, 
     check(hipGetLastError(), "tiramisu_hip_sgemm");
 }
 
-// 256x256 tiles (4 waves of 128x128) once they give every compute unit work; 128x128 tiles
-// (4 waves of 64x64) for mid sizes; 64x64 tiles when larger ones would leave most of the 256
-// compute units idle.
+// The square C tile whose launch is modelled fastest: a compute unit works through
+// ceil(tiles / 256) tiles, each costing its area over the share of the MFMA rate that a tile of
+// that size sustains.  256 and 192 are for whole tiles only (3072 = 16 x 192: one per unit).
 int tile_for(int M, int N) {
-    if ((long)(M / 256) * (N / 256) >= 192 && M % 256 == 0 && N % 256 == 0) return 256;
-    if ((long)((M + 127) / 128) * ((N + 127) / 128) >= 256) return 128;
-    return 64;
+    struct candidate { int tile; double rate; bool whole_only; };
+    const candidate cands[] = {{256, 1.0, true}, {192, 0.9, true}, {128, 0.8, false}, {64, 0.68, false}};
+    double best = 0;
+    int tile = 64;
+    for (const candidate &c : cands) {
+        if (c.whole_only && (M % c.tile != 0 || N % c.tile != 0)) continue;
+        if (c.tile == 128 && M < 128) continue;
+        const long tiles = (long)((M + c.tile - 1) / c.tile) * ((N + c.tile - 1) / c.tile);
+        const double cost = (double)((tiles + 255) / 256) * c.tile * c.tile / c.rate;
+        if (best == 0 || cost < best) { best = cost; tile = c.tile; }
+    }
+    return tile;
 }
 
 template <bool AK, bool BK_, bool EDGE>
 void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
                    float alpha, float beta, bool vec_ok) {
     const int bm = tile_for(M, N);
-    if (bm == 256)
-        launch_mfma<tgemm::config<256, 256, 16, 2, 2, AK, BK_, EDGE, 0>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
-    else if (bm == 128)
+    if constexpr (!EDGE) {
+        if (bm == 256)
+            return launch_mfma<tgemm::config<256, 256, 16, 2, 2, AK, BK_, false, 0>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+        if (bm == 192)
+            return launch_mfma<tgemm::config<192, 192, 16, 2, 2, AK, BK_, false>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+    }
+    if (bm == 128)
         launch_mfma<tgemm::config<128, 128, 16, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
     else
         launch_mfma<tgemm::config<64, 64, 32, 2, 2, AK, BK_, EDGE>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
+}
+
+// Few C tiles but a long reduction (a batch of 64 rows against wide weights, as in recurrent
+// cells): 64x32 tiles, 8 groups of wavefronts share the K range of each tile and reduce through
+// LDS, and up to four K-slices are requested ahead (the launch is latency-bound).
+bool skinny(int M, int N, int K, bool vec_ok, bool transposeA) {
+    return !transposeA && vec_ok && M == 64 && (N + 63) / 64 <= 64 && N % 32 == 0 && K % 128 == 0 && K >= 256;
+}
+
+template <bool BK_>
+void dispatch_skinny(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
+                     float alpha, float beta) {
+    switch (std::min(4, K / 128 - 1)) {
+    case 1: return launch_mfma<tgemm::config<64, 32, 128, 2, 1, true, BK_, false, 0, 8, 1>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, true);
+    case 2: return launch_mfma<tgemm::config<64, 32, 128, 2, 1, true, BK_, false, 0, 8, 2>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, true);
+    case 3: return launch_mfma<tgemm::config<64, 32, 128, 2, 1, true, BK_, false, 0, 8, 3>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, true);
+    default: return launch_mfma<tgemm::config<64, 32, 128, 2, 1, true, BK_, false, 0, 8, 4>>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, true);
+    }
 }
 
 template <bool AK, bool BK_>
@@ -178,8 +271,13 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
         check(hipGetLastError(), __FUNCTION__);
         return 0;
     }
+    if (skinny(m, n, k, vec_ok, transposeA)) {
+        if (transposeB) dispatch_skinny<true>(a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta);
+        else dispatch_skinny<false>(a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta);
+        return 0;
+    }
     const int bm = tile_for(m, n);
-    const bool edge = !(vec_ok && m % bm == 0 && n % bm == 0 && k % 16 == 0);
+    const bool edge = !(vec_ok && m % bm == 0 && n % bm == 0 && k % (bm == 64 ? 32 : 16) == 0);   // K-slice of the tile
     // A is K-contiguous unless transposed; B is K-contiguous only when transposed.
     if (!transposeA && !transposeB) dispatch_edge<true, false>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
     else if (!transposeA && transposeB) dispatch_edge<true, true>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
@@ -245,7 +343,7 @@ int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t b
         exit(1);
     }
     std::string nm;
-    if (profiling) {
+    if (profiling.load()) {
         std::lock_guard<std::mutex> g(names_mutex);
         nm = function_names[function];
     }
@@ -254,6 +352,22 @@ int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t b
                                 dynamic_lds_bytes, current_stream, args, nullptr),
           __FUNCTION__);
     return 0;
+}
+
+void tiramisu_hip_parallel_for(int32_t first, int32_t last, void (*body)(int32_t, void *), void *closure) {
+    if (last < first) return;
+    if (first == last || in_parallel_iteration) {
+        for (int32_t i = first; i <= last; i++) body(i, closure);
+        return;
+    }
+    static parallel_pool *pool = new parallel_pool;
+    struct job { void (*body)(int32_t, void *); void *closure; } j{body, closure};
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);   // what the caller launched so far is complete
+    pool->run(first, last, [](int32_t i, void *p) {
+        in_parallel_iteration = true;
+        static_cast<job *>(p)->body(i, static_cast<job *>(p)->closure);
+        in_parallel_iteration = false;
+    }, &j);
 }
 
 int tiramisu_hip_set_stream(void *stream) {
@@ -287,6 +401,7 @@ int tiramisu_hip_event_destroy(void *event) {
 }
 
 int tiramisu_hip_profile_start(void) {
+    std::lock_guard<std::mutex> g(records_mutex);
     for (auto &r : records) {
         hipEventDestroy(r.start);
         hipEventDestroy(r.stop);
@@ -298,6 +413,7 @@ int tiramisu_hip_profile_start(void) {
 
 int tiramisu_hip_profile_stop(void) {
     profiling = false;
+    std::lock_guard<std::mutex> g(records_mutex);
     for (auto &r : records) {
         check(hipEventSynchronize(r.stop), __FUNCTION__);
         check(hipEventElapsedTime(&r.ms, r.start, r.stop), __FUNCTION__);

@@ -335,6 +335,16 @@ bool canonicalize(function *f, const node_ptr &real, const std::set<std::string>
         if (it == real->iterators.end()) return false;
         for (auto &in : inner)
             if (lir::mentions(it->second, in)) d.in_kernel = true;
+        // A dimension split between host loops and the kernel: one launch covers part of its
+        // range only, which the canonical bounds do not describe.
+        bool partly_outside = false;
+        if (d.in_kernel)
+            it->second.visit([&](const expr &x) {
+                if (x.get_expr_type() != e_var || inner.count(x.get_name())) return;
+                const std::string &nm = x.get_name();
+                if (nm.size() > 1 && nm[0] == 'c' && nm.find_first_not_of("0123456789", 1) == std::string::npos) partly_outside = true;
+            });
+        if (partly_outside) return false;
     }
     return true;
 }
