@@ -307,3 +307,78 @@ def lstm(weights, biases, x):
         y[m] = below
     return y
 
+
+
+def ref_convolution_gpu(img, kernel):
+    """benchmarks/halide/convolutiongpu_tiramisu.cpp:47-56, :69, :95-117: 3x3 filter of a planar uint8
+    image [3][M][N] staged through an 18x18 LDS tile (the staging does not change the values):
+    out[c][j][i] = uint8(0.f + sum over _j, then _i, of float(img[c][j+_j][i+_i]) * kernel[_j][_i]),
+    for i < N-2, j < M-2 (kernel(_i,_j) reads kernel_gpu[_j][_i], a plain copy of the host kernel)."""
+    f = np.float32
+    C, M, N = img.shape
+    x = img.astype(np.float32)
+    acc = np.zeros((C, M - 2, N - 2), np.float32)
+    for _j in range(3):
+        for _i in range(3):
+            acc = acc + x[:, _j:_j + M - 2, _i:_i + N - 2] * f(kernel[_j][_i])
+    return acc.astype(np.uint8)
+
+
+def ref_fusion_gpu(img):
+    """benchmarks/halide/fusiongpu_tiramisu.cpp:36-41: f = 255 - in, g = 2*in, h = f + g, k = f - g on
+    uint8, every value stored as uint8 (arithmetic modulo 256)."""
+    x = img.astype(np.int32)
+    f = (255 - x) % 256
+    g = (2 * x) % 256
+    return f.astype(np.uint8), g.astype(np.uint8), ((f + g) % 256).astype(np.uint8), ((f - g) % 256).astype(np.uint8)
+
+
+def ref_rgbyuv420_gpu(rgb):
+    """benchmarks/halide/rgbyuv420gpu_tiramisu.cpp:37-50: planar RGB uint8 [3][M][N] (M, N even) to a
+    full-resolution y and half-resolution u, v taken at even pixels.  int32 arithmetic as the
+    generated C computes it: % is the remainder of truncating division (sign of the dividend),
+    and the conversion to uint8 is modulo 256."""
+    r, g, b = (rgb[c].astype(np.int32) for c in range(3))
+    y = np.fmod(66 * r + 129 * g + 25 * b + 128, 256) + 16
+    r2, g2, b2 = r[::2, ::2], g[::2, ::2], b[::2, ::2]
+    u = np.fmod(-38 * r2 - 74 * g2 + 112 * b2 + 128, 256) + 128
+    v = np.fmod(112 * r2 - 94 * g2 - 18 * b2 + 128, 256) + 128
+    return tuple((a % 256).astype(np.uint8) for a in (y, u, v))
+
+
+def ref_warp_affine_gpu(img):
+    """benchmarks/halide/warp_affinegpu_tiramisu.cpp:44-80, literally: with every coefficient 0.1f,
+    o_r = 0.1*i + 0.1*j + 0.1 (the program's o_c has the same value), r = c = o_r - floor(o_r), both
+    coordinates are floor(o_r) (:63-64), clamped to [0, N] for rows and [0, M] for columns, and
+    out[j][i] = mix(mix(A00, A01, r), mix(A10, A11, r), c) with mix(x, y, a) = x*(1-a) + y*a and
+    in(r, c) read at img[c][r].  fp32 throughout; img is uint8 [M][N]."""
+    f = np.float32
+    M, N = img.shape
+    j, i = np.meshgrid(np.arange(M, dtype=np.float32), np.arange(N, dtype=np.float32), indexing="ij")
+    o = (f(0.1) * i + f(0.1) * j).astype(np.float32) + f(0.1)
+    fl = np.floor(o).astype(np.float32)
+    frac = (o - fl).astype(np.float32)
+    coord = fl.astype(np.int32)
+    rows = lambda v: np.clip(v, 0, N)
+    cols = lambda v: np.clip(v, 0, M)
+    at = lambda rr, cc: img[cc, rr].astype(np.float32)
+    a00, a01 = at(rows(coord), cols(coord)), at(rows(coord), cols(coord + 1))
+    a10, a11 = at(rows(coord + 1), cols(coord)), at(rows(coord + 1), cols(coord + 1))
+    one = f(1.0)
+    mix = lambda x, y, a: (x * (one - a)).astype(np.float32) + (y * a).astype(np.float32)
+    return mix(mix(a00, a01, frac), mix(a10, a11, frac), frac).astype(np.float32)
+
+
+def ref_edge_gpu(img):
+    """benchmarks/halide/edgegpu_tiramisu.cpp:25-31, :47-49, in place on a planar uint8 image [3][M][N]:
+    R = (ring of the 8 neighbours of the 3x3 window at (i, j)) / 8 in int arithmetic for i < N-2,
+    j < M-2, then Img(i, j) = (R(i+1,j+1) - R(i+2,j)) + (R(i+2,j+1) - R(i+1,j)) stored as uint8.  R is
+    defined for indices below N-2 / M-2 only, so the result is fixed for i < N-4, j < M-4; returns
+    that region, [3][M-4][N-4]."""
+    x = img.astype(np.int32)
+    C, M, N = img.shape
+    s = lambda dj, di: x[:, dj:dj + M - 2, di:di + N - 2]          # Img(i+di, j+dj)
+    R = (s(0, 0) + s(1, 0) + s(2, 0) + s(0, 1) + s(2, 1) + s(0, 2) + s(1, 2) + s(2, 2)) // 8
+    t = lambda dj, di: R[:, dj:dj + M - 4, di:di + N - 4]          # R(i+di, j+dj)
+    out = (t(1, 1) - t(0, 2)) + (t(1, 2) - t(0, 1))
+    return (out % 256).astype(np.uint8)

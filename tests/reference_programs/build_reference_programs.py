@@ -24,6 +24,11 @@ PROGRAMS = [
     ("benchmarks/halide/cvtcolorgpu_tiramisu.cpp", [], "cvtcolorgpu"),
     ("benchmarks/halide/gaussiangpu_tiramisu.cpp", [], "gaussiangpu"),
     ("benchmarks/halide/heat2dgpu_tiramisu.cpp", ["USE_GPU2"], "heat2dgpu"),
+    ("benchmarks/halide/convolutiongpu_tiramisu.cpp", [], "convolutiongpu"),
+    ("benchmarks/halide/fusiongpu_tiramisu.cpp", [], "fusiongpu"),
+    ("benchmarks/halide/rgbyuv420gpu_tiramisu.cpp", [], "rgbyuv420gpu"),
+    ("benchmarks/halide/warp_affinegpu_tiramisu.cpp", [], "warp_affinegpu"),
+    ("benchmarks/halide/edgegpu_tiramisu.cpp", [], "edgegpu"),
 ]
 
 
@@ -69,11 +74,13 @@ def build_test(generator_rel, wrapper_rel):
 #    LDS by hand; gpu_lib/generator.cpp (4 layers, batch 64, 512 features, 100 steps) calls the
 #    library GEMM, batches the input products over 10 steps and walks (layer, step block)
 #    diagonally with skew + interchange under a parallel host loop.
+#  * chain_mm: (A x B) x C, two GEMM nests with the reduction loop interchanged inward.
 # (source below the reference tree, library stem, object the program writes):
 SELF_DRIVEN = [("benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator%d.cpp" % n, "sgemm_generator%d" % n, "fct.o")
                for n in (1, 2, 3)] + [
     ("benchmarks/DNN/blocks/LSTM/gpu/generator.cpp", "lstm_gpu", "lstm.o"),
     ("benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp", "lstm_gpu_lib", "lstm.o"),
+    ("benchmarks/linear_algebra/chain_mm/gpu/generator.cpp", "chain_mm", "fct.o"),
 ]
 
 

@@ -18,7 +18,9 @@ def library(name):
     return os.path.join(HERE, "reference_programs", "build", "lib%s.so" % name)
 
 
-PROGRAMS = {"cvtcolorgpu": "cvtcolorgpu_tiramisu", "gaussiangpu": "gaussiangpu_tiramisu", "heat2dgpu": "heat2dgpu_tiramisu"}
+PROGRAMS = {"cvtcolorgpu": "cvtcolorgpu_tiramisu", "gaussiangpu": "gaussiangpu_tiramisu", "heat2dgpu": "heat2dgpu_tiramisu",
+            "convolutiongpu": "convolutiongpu_tiramisu", "fusiongpu": "fusiongpu_tiramisu",
+            "rgbyuv420gpu": "rgbyuv420gpu_tiramisu", "warp_affinegpu": "warp_affinegpu_tiramisu", "edgegpu": "edge_tiramisu"}
 
 
 def test_restatements_on_closed_forms():
@@ -32,6 +34,20 @@ def test_restatements_on_closed_forms():
     out = ref.ref_heat2d_gpu(g)
     assert np.all(out[1:-1, 1:-1] == np.float32(1.0) * np.float32(0.3) + np.float32(4.0) * np.float32(0.4))
     assert np.all(out[0] == 0) and np.all(out[:, -1] == 0)
+    # identity filter; (255 - x) + 2x = 255 + x; gray pixels: y = (220 v + 128) % 256 + 16 and, the chroma
+    # weights cancelling, u = v = 128 % 256 + 128 = 256, which is 0 as uint8; a constant image warps to itself; the edge filter of a constant is 0
+    img = np.random.RandomState(2).randint(0, 256, (3, 12, 14)).astype(np.uint8)
+    ident = np.zeros((3, 3), np.float32)
+    ident[1, 1] = 1
+    assert np.array_equal(ref.ref_convolution_gpu(img, ident), img[:, 1:-1, 1:-1])
+    f, g2, h, k2 = ref.ref_fusion_gpu(img)
+    assert np.array_equal(h, (img.astype(np.int32) + 255).astype(np.uint8)) and np.array_equal(f, 255 - img)
+    gray = np.stack([img[0]] * 3)
+    y, u, v = ref.ref_rgbyuv420_gpu(gray)
+    assert np.array_equal(y, ((220 * gray[0].astype(np.int32) + 128) % 256 + 16).astype(np.uint8))
+    assert np.all(u == 0) and np.all(v == 0)
+    assert np.allclose(ref.ref_warp_affine_gpu(np.full((20, 24), 77, np.uint8)), 77.0, rtol=1e-6)
+    assert np.all(ref.ref_edge_gpu(np.full((3, 12, 14), 200, np.uint8)) == 0)
 
 
 @pytest.mark.parametrize("name", sorted(PROGRAMS))
@@ -81,6 +97,66 @@ def test_reference_heat2dgpu(n):
 
 
 # ---------------------------------------------------------------- the reference's own GPU tests
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(48, 64), (37, 53)])
+def test_reference_convolutiongpu(M, N):
+    # taps that are multiples of 1/8 and add up to 1: every product and sum is exact and fits uint8
+    kernel = np.array([[0, 0.125, 0], [0.125, 0.25, 0.125], [0, 0.25, 0.125]], np.float32)
+    img = np.random.RandomState(M + N).randint(0, 256, (3, M, N)).astype(np.uint8)
+    out = np.zeros((3, M - 2, N - 2), np.uint8)
+    load("convolutiongpu")(np.array([N, M], np.int32), img, kernel, out)
+    assert np.array_equal(out, ref.ref_convolution_gpu(img, kernel))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(48, 64), (37, 53)])
+def test_reference_fusiongpu(M, N):
+    img = np.random.RandomState(M * N).randint(0, 256, (3, M, N)).astype(np.uint8)
+    outs = [np.zeros((3, M, N), np.uint8) for _ in range(4)]
+    load("fusiongpu")(np.array([N, M], np.int32), img, *outs)
+    for got, want in zip(outs, ref.ref_fusion_gpu(img)):
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(48, 64), (38, 54)])
+def test_reference_rgbyuv420gpu(M, N):
+    img = np.random.RandomState(3 * M + N).randint(0, 256, (3, M, N)).astype(np.uint8)
+    y, u, v = np.zeros((M, N), np.uint8), np.zeros((M // 2, N // 2), np.uint8), np.zeros((M // 2, N // 2), np.uint8)
+    load("rgbyuv420gpu")(np.array([N, M], np.int32), img, y, u, v)
+    ey, eu, ev = ref.ref_rgbyuv420_gpu(img)
+    assert np.array_equal(y, ey) and np.array_equal(u, eu) and np.array_equal(v, ev)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N", [(96, 128), (75, 101)])
+def test_reference_warp_affinegpu(M, N):
+    img = np.random.RandomState(M + 7 * N).randint(0, 256, (M, N)).astype(np.uint8)
+    out = np.zeros((M, N), np.float32)
+    load("warp_affinegpu")(np.array([N, M], np.int32), img, out)
+    expected = ref.ref_warp_affine_gpu(img)
+    # fused multiply-adds may move a source coordinate that lies on an integer by one ulp to the
+    # other side of floor(): such pixels are excused, all others must agree
+    f = np.float32
+    j, i = np.meshgrid(np.arange(M, dtype=np.float32), np.arange(N, dtype=np.float32), indexing="ij")
+    o = (f(0.1) * i + f(0.1) * j).astype(np.float32) + f(0.1)
+    on_integer = np.abs(o - np.round(o)) < 1e-4
+    ok = np.abs(out - expected) <= 1e-4 * 255
+    assert np.all(ok | on_integer)
+    assert np.mean(ok) > 0.85
+
+
+@pytest.mark.gpu
+def test_reference_edgegpu():
+    # the program is written for 8192 x 8192 x 3 in place (edgegpu_tiramisu.cpp:3-4)
+    n = 8192
+    img = np.random.RandomState(8192).randint(0, 256, (3, n, n)).astype(np.uint8)
+    work = img.copy()
+    load("edgegpu")(work)
+    assert np.array_equal(work[:, :n - 4, :n - 4], ref.ref_edge_gpu(img))
+    assert np.array_equal(work[:, n - 2:, :], img[:, n - 2:, :]) and np.array_equal(work[:, :, n - 2:], img[:, :, n - 2:])
+
 
 REFERENCE_TESTS = ["wrapper_test_%s" % n for n in ("162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + \
                   ["wrapper_tutorial_04gpu", "wrapper_tutorial_04gpu2"]
@@ -203,3 +279,30 @@ def test_reference_lstm_gpu_lib_generator():
         ms = float(t1[0] - t0[0])
         best = ms if best is None else min(best, ms)
     print("gpu_lib LSTM generator: %.3f ms" % best, flush=True)
+
+
+def test_reference_chain_mm_library_exports_its_function():
+    if not os.path.exists(library("chain_mm")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    assert hasattr(ctypes.CDLL(library("chain_mm")), "matmul")
+    text = open(os.path.join(HERE, "reference_programs", "build", "chain_mm", "fct.o.hip")).read()
+    assert text.count("mfma-contraction") == 2
+
+
+@pytest.mark.gpu
+def test_reference_chain_mm_generator():
+    """benchmarks/linear_algebra/chain_mm/gpu/generator.cpp, unchanged: O = (A x B) x C with
+    1024x512, 512x128 and 128x256 operands (configuration.h), each product a gpu_tile nest with its
+    zero initialisation fused at the thread level; both become MFMA kernels.  Integer data small
+    enough that every partial sum is exact in fp32."""
+    if not os.path.exists(library("chain_mm")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    rng = np.random.RandomState(1024)
+    A = rng.randint(-2, 3, (1024, 512)).astype(np.float32)
+    B = rng.randint(-2, 3, (512, 128)).astype(np.float32)
+    C = rng.randint(-2, 3, (128, 256)).astype(np.float32)
+    O = np.full((1024, 256), -1, np.float32)
+    runtime.Program(library("chain_mm"), "matmul")(A, B, C, O)
+    expected = ((A.astype(np.float64) @ B.astype(np.float64)) @ C.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(O, expected)
