@@ -157,9 +157,42 @@ def build_wrapper_program(source):
          ["-L" + PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(PKG, os.path.join(WRAPPER_DIR, "build"))])
 
 
+PYTHON_PACKAGE = os.path.join(PKG, "python", "tiramisu")
+PYTHON_PROGRAMS = os.path.join(ROOT, "tests", "python_programs")
+
+
+def python_module():
+    import sysconfig
+    return os.path.join(PYTHON_PACKAGE, "tiramisu" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_python_module():
+    """The pybind11 extension behind ``from tiramisu import *`` (tiramisu_amd/python/tiramisu)."""
+    import sysconfig
+    import pybind11
+    _run(["g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-fvisibility=hidden", "-I" + INCLUDE, "-I" + pybind11.get_include(),
+          "-I" + sysconfig.get_paths()["include"], "-o", python_module(), os.path.join(CSRC, "python_module.cpp"),
+          "-L" + PKG, "-ltiramisu", "-Wl,-rpath,$ORIGIN/../.."])
+    return python_module()
+
+
+def build_python_programs(verbose=False):
+    """Run the Tiramisu programs written in Python (tests/python_programs/*.py): each generates its
+    object and links lib<function>.so under tests/python_programs/build/."""
+    if not os.path.isdir(PYTHON_PROGRAMS):
+        return
+    for f in sorted(os.listdir(PYTHON_PROGRAMS)):
+        if f.endswith(".py"):
+            if verbose:
+                print("[build] python program", f, flush=True)
+            _run([sys.executable, os.path.join(PYTHON_PROGRAMS, f)])
+
+
 def build_all(force=True, verbose=False):
     build_compiler(force)
     build_wrappers(force)
+    build_python_module()
+    build_python_programs(verbose)
     for src in program_sources():
         if "CPU_ONLY_PROGRAM" in open(src).read():
             continue  # needs the CPU back-end, which lives with the oracle
