@@ -62,10 +62,11 @@ struct linear_source {
 // One operand tile of X x BK elements (X = BM for A, BN for B).
 template <int X, int BK, int NT, bool KMAJOR, bool EDGE, int PAD>
 struct operand_tile {
-    static constexpr int NV = X * BK / 4 / NT;                 // 16-byte loads per thread and slice
+    static constexpr int UNITS = X * BK / 4;                      // 16-byte loads per slice
+    static constexpr int NV = (UNITS + NT - 1) / NT;              // ... per thread (the last round may be partial)
+    static constexpr bool PARTIAL = UNITS % NT != 0;
     static constexpr int ROW = KMAJOR ? (X + PAD) * 4 : X;      // LDS floats per k-group / per k
     static constexpr int LDS_FLOATS = KMAJOR ? (BK / 4) * ROW : BK * ROW;
-    static_assert(X * BK / 4 % NT == 0, "tile must split evenly over the threads");
     static_assert(BK % 8 == 0, "BK must be a multiple of 8");
 
     static __device__ __forceinline__ int swizzle(int x, int kq) { return x ^ (2 * (kq & 3)); }
@@ -78,6 +79,7 @@ struct operand_tile {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
             const int idx = t + NT * v;
+            if (PARTIAL && idx >= UNITS) break;
             int x, k;
             if (KMAJOR) { k = 4 * (idx % (BK / 4)); x = idx / (BK / 4); }
             else        { x = 4 * (idx % (X / 4));  k = idx / (X / 4); }
@@ -90,6 +92,7 @@ struct operand_tile {
 #pragma unroll
         for (int v = 0; v < NV; v++) {
             const int idx = t + NT * v;
+            if (PARTIAL && idx >= UNITS) break;
             if (KMAJOR) {
                 const int kq = idx % (BK / 4), x = idx / (BK / 4);
                 *reinterpret_cast<f32x4 *>(lds + kq * ROW + swizzle(x, kq) * 4) = regs[v];

@@ -848,6 +848,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
     if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
     if (bf16) {
         // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
