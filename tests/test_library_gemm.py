@@ -56,3 +56,18 @@ def test_transposed_operands_padding_and_offsets(tA, tB):
     run(96, 80, 40, 2.0, 1.0, tA=tA, tB=tB, pad=4, off=12)
     run(64, 2048, 512, 1.0, 1.0, tA=tA, tB=tB, pad=4, off=16)
     run(50, 30, 20, 1.0, 0.0, tA=tA, tB=tB, pad=3, off=5)
+
+
+def test_seeded_sweep_of_shapes():
+    # 80 shapes up to 300 in each dimension, every transposition, with and without padding / offsets
+    rng = np.random.RandomState(2026)
+    for case in range(80):
+        M, N, K = (int(v) for v in rng.randint(1, 301, 3))
+        if case % 5 == 0:
+            M, N, K = 64 * int(rng.randint(1, 4)), 32 * int(rng.randint(1, 9)), 128 * int(rng.randint(2, 5))
+        tA, tB = bool(rng.randint(2)), bool(rng.randint(2))
+        pad = int(rng.choice([0, 1, 4]))
+        off = int(rng.choice([0, 3, 16]))
+        alpha, beta = float(rng.choice([1.0, 2.0, -1.0])), float(rng.choice([0.0, 1.0, 0.5]))
+        print("case", case, M, N, K, tA, tB, pad, off, alpha, beta, flush=True)
+        run(M, N, K, alpha, beta, tA=tA, tB=tB, pad=pad, off=off, seed=case)
