@@ -71,3 +71,17 @@ def test_seeded_sweep_of_shapes():
         alpha, beta = float(rng.choice([1.0, 2.0, -1.0])), float(rng.choice([0.0, 1.0, 0.5]))
         print("case", case, M, N, K, tA, tB, pad, off, alpha, beta, flush=True)
         run(M, N, K, alpha, beta, tA=tA, tB=tB, pad=pad, off=off, seed=case)
+
+
+@pytest.mark.parametrize("M,N,K,tA,tB", [(70, 50, 30, False, False), (64, 96, 128, True, False), (33, 65, 17, False, True), (128, 128, 64, True, True)])
+def test_double_precision(M, N, K, tA, tB):
+    # tiramisu_hip_dgemm (replaces tiramisu_cublas_dgemm, tiramisu_cuda_wrappers.cpp:117-162)
+    from gpu_util import DeviceArray
+    rng = np.random.RandomState(M * K)
+    A = rng.uniform(-1, 1, (K, M) if tA else (M, K))
+    B = rng.uniform(-1, 1, (N, K) if tB else (K, N))
+    C = rng.uniform(-1, 1, (M, N))
+    expected = 1.5 * ((A.T if tA else A) @ (B.T if tB else B)) + 0.5 * C
+    dA, dB, dC = DeviceArray(A), DeviceArray(B), DeviceArray(C)
+    runtime.wrappers().tiramisu_hip_dgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 1.5, 0.5, 0, 0, 0, 0, 0, 0, tA, tB)
+    assert np.max(np.abs(dC.download() - expected)) <= 1e-12 * K
