@@ -33,10 +33,10 @@ PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
 # HBM bytes per launch of the dominant heat2d kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); see profiles/.
-HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # interior-tile kernel, by time steps per launch; KiB counters x calibration factor
-    7: (128858.1 * 2.000 + 250674.5 * 1.000) * 1024,
-    3: (127622.7 * 2.000 + 252906.8 * 1.000) * 1024,
-    1: (127512.8 * 2.000 + 254771.8 * 1.000) * 1024,
+HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # by time steps per launch; KiB counters x calibration factor
+    7: (154709.4 * 2.000 + 262159.8 * 1.000) * 1024,
+    3: (146714.7 * 2.000 + 263337.0 * 1.000) * 1024,
+    1: (145302.2 * 2.000 + 264923.8 * 1.000) * 1024,
 }
 
 
@@ -103,16 +103,20 @@ def cpu_threads():
 def stencil_kernels(kernel_source, domain_cells):
     """{kernel name: (time steps fused in one launch, cells advanced per launch)}, read from the
     emitter's description of each kernel in the generated kernel source: the kernel for interior
-    tiles advances tiles x tile extent cells, its companion the rest of the iteration domain."""
+    tiles advances tiles x tile extent cells, its companion the rest of the iteration domain --
+    or the one launch all of it, when it carries the boundary slices behind its interior tiles."""
     import re
     text = open(kernel_source).read()
     out = {}
     for m in re.finditer(r"// (\w+): stencil: (\d+) time step\(s\) per launch, radius \d+, tile (\d+)x(\d+) in registers, "
                          r".*?, (\d+) interior tiles", text):
         out[m.group(1)] = (int(m.group(2)), int(m.group(3)) * int(m.group(4)) * int(m.group(5)))
-    for m in re.finditer(r"// (\w+): stencil: the \d+ tiles of (\w+)'s launch", text):
+    for m in re.finditer(r"// (\w+): stencil: the \d+ tiles of (\w+)'s launch[^\n]*", text):
         steps, cells = out[m.group(2)]
-        out[m.group(1)] = (steps, domain_cells - cells)
+        if "carried by" in m.group(0):          # one launch advances the whole iteration domain
+            out[m.group(2)] = (steps, domain_cells)
+        else:
+            out[m.group(1)] = (steps, domain_cells - cells)
     return out
 
 

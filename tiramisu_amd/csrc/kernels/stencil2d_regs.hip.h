@@ -203,47 +203,19 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     }
 }
 
-// Interior tiles: one workgroup per tile of the rectangle [ST_IBX0, ST_IBX1] x [ST_IBY0, ST_IBY1].
-extern "C" __global__ void __launch_bounds__(64 * ST_W)
-#if ST_OCC > 0
-__attribute__((amdgpu_waves_per_eu(ST_OCC)))
-#endif
-ST_NAME(float *__restrict__ planes, const int src_plane)
-{
-    static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
-    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
-    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
-    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
-    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a band
-    // of consecutive tiles (row-major), so that tiles running together share their halos in L2.
-    constexpr int IW = ST_IBX1 - ST_IBX0 + 1;
-    const int nb = gridDim.x, b = blockIdx.x;
-#if ST_XCD
-    const int xcd = b % 8, per = nb / 8, extra = nb % 8;
-    const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / 8;
-#else
-    const int tile = b;
-#endif
-    ST_CAT(ST_NAME, _sweep)<false, ST_RPT>(src, dst, xch, (ST_IBY0 + tile / IW) * ST_TH, (ST_IBX0 + tile % IW) * ST_TW, ST_NY);
-}
-
-// The other tiles, in the order: full tile rows above the interior rectangle, full rows below it,
-// then the tiles left and right of it row by row.  These tiles are few (one ring), so each is cut
-// into ST_EDGE_SUB horizontal slices of ST_W*ST_RPT_EDGE staged rows, one workgroup each: more and
-// lighter workgroups (the swap registers come on top of the strip) instead of two rounds of one
-// heavy workgroup per CU.
+// The tiles outside the interior rectangle, in the order: full tile rows above the interior
+// rectangle, full rows below it, then the tiles left and right of it row by row.  These tiles are
+// few (one ring), so each is cut into ST_EDGE_SUB horizontal slices of ST_W*ST_RPT_EDGE staged
+// rows, one workgroup each: more and lighter workgroups (the swap registers come on top of the
+// strip) instead of one heavy workgroup per tile.  eb is the index of the slice.
 #define ST_TH_EDGE (ST_W * ST_RPT_EDGE - 2 * ST_HY)
 #define ST_EDGE_SUB ((ST_TH + ST_TH_EDGE - 1) / ST_TH_EDGE)
-extern "C" __global__ void __launch_bounds__(64 * ST_W)
-ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
+static __device__ __forceinline__ void ST_CAT(ST_NAME, _edge_slice)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int eb)
 {
-    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
-    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
-    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
     constexpr int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
     constexpr int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
-    const int sub = blockIdx.x % ST_EDGE_SUB;
-    int e = blockIdx.x / ST_EDGE_SUB, bx, by;
+    const int sub = eb % ST_EDGE_SUB;
+    int e = eb / ST_EDGE_SUB, bx, by;
     if (e < TOP) {
         by = e / ST_GX;
         bx = e % ST_GX;
@@ -259,6 +231,53 @@ ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
     }
     ST_CAT(ST_NAME, _sweep)<true, ST_RPT_EDGE>(src, dst, xch, by * ST_TH + sub * ST_TH_EDGE, bx * ST_TW, (by + 1) * ST_TH);
 }
+
+// Interior tiles: one workgroup per tile of the rectangle [ST_IBX0, ST_IBX1] x [ST_IBY0, ST_IBY1],
+// no bounds checks.  With ST_MERGE the launch carries the edge slices as well, after the ST_NI
+// interior workgroups: they are lighter and fill the tail of the launch instead of running as a
+// small launch of their own (the edge path needs fewer registers than the interior one, so the
+// interior tiles keep their occupancy).
+#define ST_NI ((ST_IBY1 >= ST_IBY0 && ST_IBX1 >= ST_IBX0) ? (ST_IBX1 - ST_IBX0 + 1) * (ST_IBY1 - ST_IBY0 + 1) : 0)
+extern "C" __global__ void __launch_bounds__(64 * ST_W)
+#if ST_OCC > 0
+__attribute__((amdgpu_waves_per_eu(ST_OCC)))
+#endif
+ST_NAME(float *__restrict__ planes, const int src_plane)
+{
+    static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
+    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
+    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
+    const int b = blockIdx.x;
+#if ST_MERGE
+    if (b >= ST_NI) {
+        ST_CAT(ST_NAME, _edge_slice)(src, dst, xch, b - ST_NI);
+        return;
+    }
+#endif
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a band
+    // of consecutive tiles (row-major), so that tiles running together share their halos in L2.
+    constexpr int IW = ST_IBX1 - ST_IBX0 + 1;
+    constexpr int nb = ST_NI;
+#if ST_XCD
+    const int xcd = b % 8, per = nb / 8, extra = nb % 8;
+    const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / 8;
+#else
+    const int tile = b;
+#endif
+    ST_CAT(ST_NAME, _sweep)<false, ST_RPT>(src, dst, xch, (ST_IBY0 + tile / IW) * ST_TH, (ST_IBX0 + tile % IW) * ST_TW, ST_NY);
+}
+
+// The edge slices as a launch of their own (used when the launches are not merged).
+extern "C" __global__ void __launch_bounds__(64 * ST_W)
+ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
+{
+    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
+    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
+    ST_CAT(ST_NAME, _edge_slice)(src, dst, xch, blockIdx.x);
+}
+#undef ST_NI
 #undef ST_TH_EDGE
 #undef ST_EDGE_SUB
 

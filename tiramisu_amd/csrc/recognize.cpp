@@ -207,6 +207,8 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     std::ostringstream host;
     auto ceil_div = [](long a, long b) { return a >= 0 ? (a + b - 1) / b : -((-a) / b); };
     auto floor_div = [](long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); };
+    // one launch per chunk: the boundary slices ride behind the interior tiles (TIRAMISU_STENCIL_MERGE=0: two launches)
+    const bool merge = env_int("TIRAMISU_STENCIL_MERGE", 1) != 0;
     for (auto &ch : chunks) {
         if (!by_steps.count(ch.second)) {
             kernel k, ke;
@@ -228,26 +230,27 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
                     ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + " in registers, " + std::to_string(WAVES) +
                     " wavefronts x " + std::to_string(ROWS) + " rows, " + std::to_string(interior) + " interior tiles";
             ke.how = "stencil: the " + std::to_string(edge_tiles) + " tiles of " + k.name + "'s launch that touch the fixed boundary, in " +
-                     std::to_string(edge_sub) + " slice(s) of " + std::to_string(TH_edge) + " rows each";
+                     std::to_string(edge_sub) + " slice(s) of " + std::to_string(TH_edge) + " rows each" +
+                     (merge ? " (carried by " + k.name + "'s launch, after its interior tiles)" : "");
             std::ostringstream s;
             s << "#define ST_NAME " << k.name << "\n#define ST_NAME_EDGE " << ke.name << "\n#define ST_NY " << NY << "\n#define ST_NX " << NX
               << "\n#define ST_Y0 " << lo[1] << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2]
               << "\n#define ST_GX " << GX << "\n#define ST_GY " << GY << "\n#define ST_IBX0 " << bx0 << "\n#define ST_IBX1 " << bx1
               << "\n#define ST_IBY0 " << by0 << "\n#define ST_IBY1 " << by1 << "\n#define ST_W " << WAVES
-              << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0)
+              << "\n#define ST_MERGE " << (merge ? 1 : 0) << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0)
               << "\n#define ST_RPT " << ROWS << "\n#define ST_RPT_EDGE " << rows_edge << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius
               << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
               << "#undef ST_NAME\n#undef ST_NAME_EDGE\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n"
               << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n"
-              << "#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
+              << "#undef ST_MERGE\n#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
             k.source = s.str();            // both kernels come from the one inclusion
             ke.source = "";
             for (kernel *q : {&k, &ke}) {
                 q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}};
                 q->block[0] = std::to_string(64 * WAVES);
             }
-            k.grid[0] = std::to_string(interior);
-            ke.grid[0] = std::to_string(edge_tiles * edge_sub);
+            k.grid[0] = std::to_string(merge ? interior + edge_tiles * edge_sub : interior);
+            ke.grid[0] = std::to_string(merge ? 0 : edge_tiles * edge_sub);
             by_steps[ch.second] = {k, ke};
         }
         const long src = (((ch.first - 1) % 2) + 2) % 2;
