@@ -34,9 +34,9 @@ PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 # HBM bytes per launch of the dominant heat2d kernel measured with rocprofv3 --pmc
 # (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); see profiles/.
 HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # by time steps per launch; KiB counters x calibration factor
-    7: (154709.4 * 2.000 + 262159.8 * 1.000) * 1024,
-    3: (146714.7 * 2.000 + 263337.0 * 1.000) * 1024,
-    1: (145302.2 * 2.000 + 264923.8 * 1.000) * 1024,
+    11: (176981.2 * 2.000 + 262402.5 * 1.000) * 1024,
+    9: (172771.4 * 2.000 + 262401.0 * 1.000) * 1024,
+    1: (144475.0 * 2.000 + 266309.6 * 1.000) * 1024,
 }
 
 

@@ -179,10 +179,10 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     const long T0 = lo[0], T1 = hi[0];
     const long steps = T1 - T0 + 1;
     // region staged by one workgroup: WAVES*ROWS rows by 256 columns (kernels/stencil2d_regs.hip.h)
-    const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", 8);
+    const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", 11);
     if (WAVES < 1 || WAVES > 16 || ROWS < radius || ROWS > 32) return false;
     const int LH = WAVES * ROWS, LW = 256;
-    int rmax = env_int("TIRAMISU_STENCIL_STEPS", 7);
+    int rmax = env_int("TIRAMISU_STENCIL_STEPS", 11);
     // keep at least half of the staged rows and columns as the tile
     while (rmax > 1 && (4 * rmax * radius > LH || 4 * ((rmax * radius + 3) / 4 * 4) > LW)) rmax -= 1;
     if (rmax % 2 == 0) rmax -= 1;
