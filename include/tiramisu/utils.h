@@ -4,6 +4,7 @@
 // tiramisu/shim/Halide.h -- and do not need the compiler library.
 #ifndef TIRAMISU_AMD_UTILS_H
 #define TIRAMISU_AMD_UTILS_H
+#include "Halide.h"      // Halide's own, or tiramisu/shim/Halide.h when that directory is on the include path (reference: utils.h:4)
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
