@@ -77,8 +77,10 @@ struct parallel_pool {
     int32_t next = 0, last = -1;
     long generation = 0;
     int active = 0;
+    int device = 0;        // the device that was current when the pool was first used
 
     void worker() {
+        check(hipSetDevice(device), "tiramisu_hip_parallel_for");
         hipStream_t s;
         check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "tiramisu_hip_parallel_for");
         current_stream = s;
@@ -103,6 +105,7 @@ struct parallel_pool {
     void run(int32_t first, int32_t last_, void (*b)(int32_t, void *), void *c) {
         std::lock_guard<std::mutex> one(jobs_mutex);
         std::unique_lock<std::mutex> lk(m);
+        if (threads.empty()) check(hipGetDevice(&device), "tiramisu_hip_parallel_for");
         while ((int)threads.size() < WORKERS) {
             threads.emplace_back([this] { worker(); });
             threads.back().detach();
