@@ -22,7 +22,10 @@ extern "C" {
 #endif
 
 /* ---- memory (replaces tiramisu_cuda_malloc / tiramisu_cuda_free,
- *      tiramisu_cuda_wrappers.cpp:55-68) ---- */
+ *      tiramisu_cuda_wrappers.cpp:55-68).  Freed blocks are kept for the next request of the
+ *      same size (generated functions allocate and free their temporaries on every call), up to
+ *      TIRAMISU_HIP_POOL_BYTES of idle memory (default 16 GiB, 0 = no pooling); tiramisu_hip_free
+ *      waits for the calling thread's stream before it takes a block back. ---- */
 void *tiramisu_hip_malloc(uint64_t size);
 int tiramisu_hip_free(void *ptr);
 

@@ -122,6 +122,19 @@ struct parallel_pool {
 };
 thread_local bool in_parallel_iteration = false;
 
+// ---- pooled device memory (see tiramisu_hip_malloc)
+std::mutex pool_mutex;
+std::map<uint64_t, std::vector<void *>> pool_free;   // idle blocks by size
+std::map<void *, uint64_t> pool_live;                  // blocks handed out
+uint64_t pool_idle_bytes = 0;
+uint64_t pool_limit() {
+    static const uint64_t limit = [] {
+        const char *e = std::getenv("TIRAMISU_HIP_POOL_BYTES");
+        return e ? (uint64_t)std::strtoull(e, nullptr, 10) : (uint64_t)16 << 30;
+    }();
+    return limit;
+}
+
 // One thread per element of C; any strides, any sizes.  Used for double precision and for
 // shapes the MFMA path does not take.
 template <typename T>
@@ -208,14 +221,52 @@ void dispatch_edge(bool edge, const float *A, const float *B, float *C, int M, i
 
 extern "C" {
 
+// Device memory is pooled: generated functions allocate their temporaries on entry and free
+// them on exit, every call (the reference pays cudaMalloc / cudaFree each time,
+// tiramisu_cuda_wrappers.cpp:55-68).  A freed block is kept, by size, for the next request of that
+// size; blocks beyond TIRAMISU_HIP_POOL_BYTES (default 16 GiB; 0 turns pooling off) go back to HIP.
 void *tiramisu_hip_malloc(uint64_t size) {
+    {
+        std::lock_guard<std::mutex> g(pool_mutex);
+        auto it = pool_free.find(size);
+        if (it != pool_free.end() && !it->second.empty()) {
+            void *p = it->second.back();
+            it->second.pop_back();
+            pool_idle_bytes -= size;
+            pool_live[p] = size;
+            return p;
+        }
+    }
     void *p = nullptr;
     check(hipMalloc(&p, size), __FUNCTION__);
+    std::lock_guard<std::mutex> g(pool_mutex);
+    pool_live[p] = size;
     return p;
 }
 
 int tiramisu_hip_free(void *ptr) {
-    check(hipFree(ptr), __FUNCTION__);
+    if (!ptr) return 0;
+    uint64_t size = 0;
+    bool keep = false;
+    {
+        std::lock_guard<std::mutex> g(pool_mutex);
+        auto it = pool_live.find(ptr);
+        if (it != pool_live.end()) {
+            size = it->second;
+            pool_live.erase(it);
+            keep = pool_idle_bytes + size <= pool_limit();
+        }
+    }
+    if (!keep) {
+        check(hipFree(ptr), __FUNCTION__);
+        return 0;
+    }
+    // work that still uses the block was issued on the calling thread's stream (or on pool
+    // streams that tiramisu_hip_parallel_for has already synchronised)
+    check(hipStreamSynchronize(current_stream), __FUNCTION__);
+    std::lock_guard<std::mutex> g(pool_mutex);
+    pool_free[size].push_back(ptr);
+    pool_idle_bytes += size;
     return 0;
 }
 
