@@ -85,3 +85,18 @@ def test_double_precision(M, N, K, tA, tB):
     dA, dB, dC = DeviceArray(A), DeviceArray(B), DeviceArray(C)
     runtime.wrappers().tiramisu_hip_dgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 1.5, 0.5, 0, 0, 0, 0, 0, 0, tA, tB)
     assert np.max(np.abs(dC.download() - expected)) <= 1e-12 * K
+
+
+def test_freed_device_blocks_are_reused():
+    # the runtime keeps freed blocks by size for the next request (generated functions allocate
+    # and free their temporaries on every call)
+    w = runtime.wrappers()
+    a = w.tiramisu_hip_malloc(3 << 20)
+    b = w.tiramisu_hip_malloc(3 << 20)
+    assert a != b
+    w.tiramisu_hip_free(a)
+    c = w.tiramisu_hip_malloc(5 << 20)
+    d = w.tiramisu_hip_malloc(3 << 20)
+    assert d == a and c not in (a, b)
+    for p in (b, c, d):
+        w.tiramisu_hip_free(p)
