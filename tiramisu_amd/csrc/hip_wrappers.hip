@@ -66,7 +66,12 @@ struct scoped_record {
 // ---- pool for host loops tagged parallel.  Threads are created on first use and live until
 // the process ends (the state is never destroyed, so nothing is torn down under a waiting thread).
 struct parallel_pool {
-    static constexpr int WORKERS = 4;   // as many as there are hardware queues per process by default
+    // as many as there are hardware queues per process by default; TIRAMISU_HIP_POOL_THREADS overrides (1..16)
+    const int WORKERS = [] {
+        const char *e = std::getenv("TIRAMISU_HIP_POOL_THREADS");
+        const int n = e ? std::atoi(e) : 4;
+        return n < 1 ? 1 : n > 16 ? 16 : n;
+    }();
     std::mutex m;
     std::condition_variable wake, done;
     std::vector<std::thread> threads;
