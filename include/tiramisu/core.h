@@ -168,8 +168,15 @@ public:
     const std::vector<std::string> &get_codegen_log() const { return codegen_log; }
     void log(const std::string &s) { codegen_log.push_back(s); }
 
+    /** True when GPU-mapped loops are generated without gen_cuda_stmt() -- the route that, in the
+      * reference, hands the loops to Halide's own GPU target, which moves buffers between host and
+      * device by itself: kernels may then name host buffers, and the host glue copies them around
+      * each launch. */
+    bool copies_host_buffers_implicitly() const { return implicit_gpu_copies; }
+
 private:
     bool hand_driven_gpu = false;
+    bool implicit_gpu_copies = false;
     int name_counter = 0;
     std::vector<std::string> codegen_log;
 };

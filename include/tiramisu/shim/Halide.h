@@ -79,6 +79,12 @@ public:
 
     halide_buffer_t *raw_buffer() { return &s->raw; }
     const halide_buffer_t *raw_buffer() const { return &s->raw; }
+    // Generated functions of this build leave their results in host memory (explicit or
+    // implicit copies), so the calls that wrappers make around Halide's GPU targets have nothing to do.
+    int copy_to_host(void * = nullptr) { return 0; }
+    int device_sync(void * = nullptr) { return 0; }
+    void set_host_dirty(bool = true) {}
+    void set_device_dirty(bool = true) {}
     T *data() { return s->data.get(); }
     const T *data() const { return s->data.get(); }
     T *begin() { return data(); }

@@ -37,7 +37,7 @@ PROGRAMS = [
 # with the object its generator wrote into build/lib<wrapper>.so and run in-process by the tests.
 # (generator, wrapper) below the reference tree:
 TESTS = [("tests/test_%s.cpp" % n, "tests/wrapper_test_%s.cpp" % n)
-         for n in ("162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + [
+         for n in ("17", "18", "19", "162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + [
     ("tutorials/developers/tutorial_04gpu/tutorial_04gpu.cpp", "tutorials/developers/tutorial_04gpu/wrapper_tutorial_04gpu.cpp"),
     ("tutorials/developers/tutorial_04gpu2/tutorial_04gpu2.cpp", "tutorials/developers/tutorial_04gpu2/wrapper_tutorial_04gpu2.cpp"),
 ]

@@ -158,7 +158,7 @@ def test_reference_edgegpu():
     assert np.array_equal(work[:, n - 2:, :], img[:, n - 2:, :]) and np.array_equal(work[:, :, n - 2:], img[:, :, n - 2:])
 
 
-REFERENCE_TESTS = ["wrapper_test_%s" % n for n in ("162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + \
+REFERENCE_TESTS = ["wrapper_test_%s" % n for n in ("17", "18", "19", "162", "164", "165", "166", "167", "168", "169", "170", "171", "197")] + \
                   ["wrapper_tutorial_04gpu", "wrapper_tutorial_04gpu2"]
 
 
@@ -175,8 +175,10 @@ def test_reference_test_library_exports_its_entry_point(name):
 def test_reference_gpu_test_passes(name):
     """Generator (tests/test_N.cpp or the tutorial) and wrapper (wrapper_test_N.cpp) of the reference,
     both unchanged: the wrapper fills Halide::Buffer inputs, calls the generated function, computes
-    its own nested-loop expectation and compares (library GEMM calls in 162-166, gpu_tile and
-    cache_shared GEMMs in 167-171, allocate_at in 197, uint8 GEMMs in the tutorials).  A mismatch
+    its own nested-loop expectation and compares (tag_gpu_level / gpu_tile on host buffers without
+    gen_cuda_stmt in 17-19: the route of Halide's GPU target in the reference, implicit copies here;
+    library GEMM calls in 162-166, gpu_tile and cache_shared GEMMs in 167-171, allocate_at in
+    197, uint8 GEMMs in the tutorials).  A mismatch
     ends the process with status 1, as the reference's compare_buffers does."""
     if not os.path.exists(library(name)):
         pytest.skip("reference tree was absent when the libraries were built")

@@ -352,6 +352,14 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
 void function::gen_halide_obj(const std::string &obj_file_name) {
     hardware_architecture_t arch =
         hand_driven_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu;
+    // GPU-mapped loops without gen_cuda_stmt(): the reference leaves them to Halide's GPU target
+    // (tests/test_17.cpp - test_19.cpp); here they go to the HIP back-end with implicit copies,
+    // unless a CPU back-end is linked in and asked for
+    if (!hand_driven_gpu && !gpu_block_dimensions.empty() && backend::find(hardware_architecture_t::arch_amd_gpu) &&
+        !(std::getenv("TIRAMISU_FORCE_ARCH") && std::string(std::getenv("TIRAMISU_FORCE_ARCH")) == "cpu")) {
+        arch = hardware_architecture_t::arch_amd_gpu;
+        implicit_gpu_copies = true;
+    }
     backend *b = backend::find(arch);
     if (!b) ERROR("no back-end registered for the requested architecture", true);
     if (!ast) gen_isl_ast();

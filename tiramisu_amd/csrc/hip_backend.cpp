@@ -264,9 +264,19 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
         buffer *b = f->get_buffers().at(nm);
         switch (b->get_location()) {
         case memory_location::global: k.params.push_back({true, nm, b->get_elements_type()}); break;
-        case memory_location::host:
-            ERROR("buffer " + nm + " is used inside a GPU kernel but lives in host memory; tag it with tag_gpu_global() "
-                  "and copy it with memcpy()", true);
+        case memory_location::host: {
+            if (!f->copies_host_buffers_implicitly())
+                ERROR("buffer " + nm + " is used inside a GPU kernel but lives in host memory; tag it with tag_gpu_global() "
+                      "and copy it with memcpy()", true);
+            bool written = false;
+            lir::walk(root, [&](const node_ptr &x) {
+                if (x->kind == node_kind::leaf && x->lhs == b) written = true;
+            });
+            k.params.push_back({true, nm, b->get_elements_type()});
+            k.host_mirrors.push_back({nm, primitive_c_name(b->get_elements_type()),
+                                      "(uint64_t)(" + host.element_count(b) + ") * sizeof(" + primitive_c_name(b->get_elements_type()) + ")", written});
+            break;
+        }
         case memory_location::constant:
             // a file-scope __constant__ array of the code object: not a parameter
             // (reference: tiramisu_codegen_cuda.cpp:811-829, :1192-1193)
@@ -301,8 +311,20 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
     return k;
 }
 
-std::string launch_text(const kernel &k, const std::string &ind) {
+std::string launch_text(const kernel &k, const std::string &ind_outer) {
     std::ostringstream os;
+    std::string ind = ind_outer;
+    if (!k.host_mirrors.empty()) {
+        // implicit copies: inside the inner scope the buffer's name means its device copy
+        os << ind << "{\n";
+        for (auto &m : k.host_mirrors) os << ind << "    " << m.ctype << " *" << m.name << "__host = " << m.name << ";\n";
+        os << ind << "    {\n";
+        ind += "        ";
+        for (auto &m : k.host_mirrors) {
+            os << ind << m.ctype << " *" << m.name << " = (" << m.ctype << " *)tiramisu_hip_malloc(" << m.bytes << ");\n";
+            os << ind << "tiramisu_hip_memcpy_to_device((void *)" << m.name << ", (void *)" << m.name << "__host, " << m.bytes << ");\n";
+        }
+    }
     os << ind << "{\n";
     os << ind << "    void *_args[] = {";
     for (size_t i = 0; i < k.params.size(); i++) os << (i ? ", " : "") << "(void *)&" << k.params[i].name;
@@ -315,6 +337,14 @@ std::string launch_text(const kernel &k, const std::string &ind) {
     os << ind << "    static void *_fn = tiramisu_hip_module_get_function(_tiramisu_module(), \"" << k.name << "\");\n";
     os << ind << "    tiramisu_hip_launch(_fn, _grid, _block, (uint32_t)(" << k.lds_bytes << "), _args);\n";
     os << ind << "}\n";
+    if (!k.host_mirrors.empty()) {
+        for (auto &m : k.host_mirrors) {
+            if (m.written)
+                os << ind << "tiramisu_hip_memcpy_to_host((void *)" << m.name << "__host, (void *)" << m.name << ", " << m.bytes << ");\n";
+            os << ind << "tiramisu_hip_free((void *)" << m.name << ");\n";
+        }
+        os << ind_outer << "    }\n" << ind_outer << "}\n";
+    }
     return os.str();
 }
 

@@ -32,6 +32,10 @@ struct kernel {
     std::string block[3] = {"1", "1", "1"};
     std::string lds_bytes = "0";
     std::string how;                    // "generic", "mfma-contraction", "stencil", ...
+    /** Host buffers that the kernel names (only with implicit copies): the launch site gives it
+      * device copies of them, copied in before the launch and, when written, back after it. */
+    struct host_mirror { std::string name, ctype, bytes; bool written; };
+    std::vector<host_mirror> host_mirrors;
 };
 
 /** A launch sequence that replaces one GPU-tagged loop nest. */
