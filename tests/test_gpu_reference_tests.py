@@ -188,3 +188,28 @@ def test_gemm_uint8_cache_shared(programs_dir):
     expected = ((C.astype(np.int64) + A.astype(np.int64) @ B.astype(np.int64)) % 256).astype(np.uint8)
     runtime.load(programs_dir, "gemm_u8_shared")(A, B, C)
     assert np.array_equal(C, expected)
+
+
+@pytest.mark.parametrize("tag,tA,tB,pad,origin", [("nn", False, False, 0, 0), ("nt", False, True, 0, 0), ("tn", True, False, 0, 0),
+                                                  ("tt", True, True, 0, 0), ("pitched", False, True, 3, 2)])
+def test_gemm_operand_layouts(programs_dir, tag, tA, tB, pad, origin):
+    # tests/programs/gemm_operand_layouts.cpp: every storage order of the two operands, and operands
+    # inside larger buffers (pitch and origin not multiples of 4 elements), through the MFMA emitter
+    from gpu_util import DeviceArray
+    M, N, K = 96, 80, 72
+    rng = np.random.RandomState(len(tag) + 7 * pad)
+    a_rows, a_cols = (K, M) if tA else (M, K)
+    b_rows, b_cols = (N, K) if tB else (K, N)
+    bufA, bufB = ints(rng, (a_rows + origin, a_cols + pad)), ints(rng, (b_rows + origin, b_cols + pad))
+    C = ints(rng, (M, N))
+    shift = 1 if pad else 0
+    a = bufA[origin:origin + a_rows, shift:shift + a_cols]
+    b = bufB[origin:origin + b_rows, shift:shift + b_cols]
+    expected = ref.gemm_accumulate(np.ascontiguousarray(a.T if tA else a), np.ascontiguousarray(b.T if tB else b), C)
+    assert re.search(r"^// _kernel_\d+: mfma-contraction", open(os.path.join(programs_dir, "build", "gemm_layout_%s.o.hip" % tag)).read(), re.M)
+    C_cpu = C.copy()
+    cpu_variant(programs_dir, "gemm_layout_" + tag)(bufA, bufB, C_cpu)
+    dA, dB, dC = DeviceArray(bufA), DeviceArray(bufB), DeviceArray(C)
+    runtime.load(programs_dir, "gemm_layout_" + tag)(dA.buffer(), dB.buffer(), dC.buffer())
+    out = dC.download()
+    assert np.array_equal(out, expected) and np.array_equal(out, C_cpu)
