@@ -213,3 +213,24 @@ def test_gemm_operand_layouts(programs_dir, tag, tA, tB, pad, origin):
     runtime.load(programs_dir, "gemm_layout_" + tag)(dA.buffer(), dB.buffer(), dC.buffer())
     out = dC.download()
     assert np.array_equal(out, expected) and np.array_equal(out, C_cpu)
+
+
+def test_gemm_two_products_with_batch(programs_dir):
+    # tests/programs/gemm_two_products.cpp: two products per reduction step, batch on a third block
+    # index (flattened with the rows into M), bias as fused initialisation
+    from gpu_util import DeviceArray
+    NB, M, N, K = 3, 64, 96, 80
+    rng = np.random.RandomState(380)
+    W, R = ints(rng, (N, K)), ints(rng, (N, K))
+    x, h = ints(rng, (NB, M, K)), ints(rng, (NB, M, K))
+    bias = ints(rng, (N,))
+    expected = (bias[None, None, :].astype(np.float64) + x.astype(np.float64) @ W.T.astype(np.float64) +
+                h.astype(np.float64) @ R.T.astype(np.float64)).astype(np.float32)
+    text = open(os.path.join(programs_dir, "build", "gemm_two_products.o.hip")).read()
+    assert "2 product term(s), fused initialisation" in text
+    out_cpu = np.zeros((NB, M, N), np.float32)
+    cpu_variant(programs_dir, "gemm_two_products")(W, R, x, h, bias, out_cpu)
+    devs = [DeviceArray(a) for a in (W, R, x, h, bias, np.full((NB, M, N), -1, np.float32))]
+    runtime.load(programs_dir, "gemm_two_products")(*[d.buffer() for d in devs])
+    out = devs[-1].download()
+    assert np.array_equal(out, expected) and np.array_equal(out_cpu, expected)
