@@ -1,0 +1,144 @@
+"""Time variants of a Tiramisu program on the GPU: the role that evaluation by execution plays for the
+reference's auto-scheduler (src/auto_scheduler/tiramisu_evaluator.cpp: build the candidate, run it,
+keep the time), here for the knobs of the HIP back-end's pattern emitters.
+
+    python -m tiramisu_amd.autotune tiramisu_amd/programs/heat2d.cpp heat2d_8192x32 \\
+        --knob TIRAMISU_STENCIL_STEPS=7,9,11 --knob TIRAMISU_STENCIL_ROWS=8,10,11
+
+builds the generator once, runs it once per combination of knob values (environment variables read
+by the back-end at code-generation time) in a scratch directory, calls the named function on
+seeded inputs shaped after the back-end's description of its arguments, and prints one line per
+variant, fastest first.  Every variant's outputs are compared with the first variant's: a knob must
+not change results (integer-valued inputs, so contraction kernels compare exactly too).
+Knobs: TIRAMISU_STENCIL_STEPS / _ROWS / _WAVES / _MERGE / _XCD, TIRAMISU_MFMA_TILE / _BK / _PAD / _DEPTH,
+TIRAMISU_NO_MFMA, TIRAMISU_NO_STENCIL, TIRAMISU_HIP_SERIAL_HOST_LOOPS."""
+import argparse
+import itertools
+import json
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+from . import build, runtime
+
+
+def variants(knobs):
+    names = [k.split("=", 1)[0] for k in knobs]
+    values = [k.split("=", 1)[1].split(",") for k in knobs]
+    for combo in itertools.product(*values):
+        yield dict(zip(names, combo))
+
+
+def generate(gen, directory, env_overrides):
+    os.makedirs(os.path.join(directory, "build"), exist_ok=True)
+    env = dict(os.environ)
+    env.update(env_overrides)
+    subprocess.run([gen], cwd=directory, env=env, check=True, stdout=subprocess.DEVNULL)
+
+
+def link(directory, function):
+    obj = os.path.join(directory, "build", function + ".o")
+    if not os.path.exists(obj):
+        obj = os.path.join(directory, "build", "generated_fct_" + function + ".o")
+    lib = os.path.join(directory, "build", "lib%s.so" % function)
+    subprocess.run(["g++", "-shared", "-o", lib, obj, "-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath," + build.PKG], check=True)
+    return lib
+
+
+class DeviceBuffer:
+    def __init__(self, host):
+        self.w = runtime.wrappers()
+        self.host = np.ascontiguousarray(host)
+        self.ptr = self.w.tiramisu_hip_malloc(max(self.host.nbytes, 16))
+        self.upload()
+
+    def upload(self):
+        self.w.tiramisu_hip_memcpy_to_device(self.ptr, self.host.ctypes.data, self.host.nbytes)
+
+    def download(self):
+        out = np.empty_like(self.host)
+        self.w.tiramisu_hip_stream_synchronize(0)
+        self.w.tiramisu_hip_memcpy_to_host(out.ctypes.data, self.ptr, out.nbytes)
+        return out
+
+    def free(self):
+        self.w.tiramisu_hip_free(self.ptr)
+
+
+def make_arguments(manifest, seed):
+    rng = np.random.RandomState(seed)
+    args = []
+    for a in manifest["arguments"]:
+        if not all(isinstance(v, int) for v in a["shape"]):
+            raise SystemExit("argument %s has run-time extents %s: the harness needs constant shapes" % (a["name"], a["shape"]))
+        dtype = np.dtype(runtime._C_TYPES[a["type"]])
+        values = rng.randint(0, 4, a["shape"]) if dtype.kind in "iu" else rng.randint(-2, 3, a["shape"])
+        host = values.astype(dtype)
+        args.append(DeviceBuffer(host) if a["memory"] == "device" else host)
+    return args
+
+
+def run_variant(lib, function, manifest, repeat, seed):
+    program = runtime.Program(lib, function)
+    args = make_arguments(manifest, seed)
+
+    def call():
+        program(*[runtime.Buffer.from_device(a.ptr, a.host.shape, a.host.dtype) if isinstance(a, DeviceBuffer) else a for a in args])
+    call()
+    outputs = [(a.download() if isinstance(a, DeviceBuffer) else a.copy())
+               for a, m in zip(args, manifest["arguments"]) if m["kind"] == "output"]
+    for _ in range(max(3, repeat // 2)):
+        call()
+    times = []
+    for _ in range(repeat):
+        with runtime.DeviceTimer() as t:
+            call()
+        times.append(t.ms)
+    for a in args:
+        if isinstance(a, DeviceBuffer):
+            a.free()
+    return float(np.median(times)), outputs
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\\n\\n")[0])
+    ap.add_argument("source")
+    ap.add_argument("function")
+    ap.add_argument("--knob", action="append", default=[], help="NAME=v1,v2,...")
+    ap.add_argument("--repeat", type=int, default=20)
+    ap.add_argument("--keep", help="directory to keep the generated variants in")
+    a = ap.parse_args(argv)
+    if runtime.wrappers().tiramisu_hip_device_count() < 1:
+        raise SystemExit("no HIP device visible")
+    scratch = a.keep or tempfile.mkdtemp(prefix="tiramisu_autotune_")
+    os.makedirs(scratch, exist_ok=True)
+    gen = os.path.join(scratch, "generator")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.dirname(os.path.abspath(a.source)), "-o", gen,
+                    a.source, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG], check=True)
+    results, first = [], None
+    for n, env in enumerate(variants(a.knob)):
+        directory = os.path.join(scratch, "v%d" % n)
+        generate(gen, directory, env)
+        lib = link(directory, a.function)
+        manifest = runtime.manifest_of(lib, a.function)
+        ms, outputs = run_variant(lib, a.function, manifest, a.repeat, seed=1)
+        same = True
+        if first is None:
+            first = outputs
+        else:
+            same = all(np.array_equal(x, y) for x, y in zip(first, outputs))
+        results.append({"knobs": env, "ms": ms, "same_as_first": same, "kernels": [k["how"].split(",")[0] for k in manifest["kernels"]]})
+    results.sort(key=lambda r: r["ms"])
+    for r in results:
+        print(json.dumps(r))
+    if not a.keep:
+        shutil.rmtree(scratch, ignore_errors=True)
+    return results
+
+
+if __name__ == "__main__":
+    main()

@@ -691,6 +691,34 @@ public:
             std::string cmd = std::string(cxx ? cxx : "g++") + " -std=c++17 -O2 -fPIC -I" + inc + " -c " + host_file + " -o " + obj;
             if (run(cmd) != 0) ERROR("host compiler failed on " + host_file, true);
         }
+        // ---- manifest: what a harness needs to call the function and to know what was emitted
+        {
+            auto quoted = [](const std::string &t) {
+                std::string r = "\"";
+                for (char c : t) { if (c == '"' || c == '\\') r += '\\'; r += c; }
+                return r + "\"";
+            };
+            c_printer mp;
+            mp.fct = &f;
+            std::ofstream m(obj + ".json");
+            m << "{\n  \"function\": " << quoted(f.get_name()) << ",\n  \"arguments\": [";
+            for (size_t i = 0; i < args.size(); i++) {
+                const buffer *b = args[i];
+                m << (i ? "," : "") << "\n    {\"name\": " << quoted(b->get_name()) << ", \"type\": " << quoted(primitive_c_name(b->get_elements_type()))
+                  << ", \"kind\": " << quoted(b->get_argument_type() == a_input ? "input" : b->get_argument_type() == a_output ? "output" : "temporary")
+                  << ", \"memory\": " << quoted(b->get_location() == memory_location::host ? "host" : "device") << ", \"shape\": [";
+                for (size_t d = 0; d < b->get_dim_sizes().size(); d++) {
+                    const expr e = lir::simplify(b->get_dim_sizes()[d]);
+                    m << (d ? ", " : "");
+                    if (e.is_integer_literal()) m << e.get_int_val(); else m << quoted(mp.print(e));
+                }
+                m << "]}";
+            }
+            m << "\n  ],\n  \"kernels\": [";
+            for (size_t i = 0; i < ctx.kernels.size(); i++)
+                m << (i ? "," : "") << "\n    {\"name\": " << quoted(ctx.kernels[i].name) << ", \"how\": " << quoted(ctx.kernels[i].how) << "}";
+            m << "\n  ]\n}\n";
+        }
         for (auto &k : ctx.kernels) f.log(k.name + ": " + k.how);
         if (debug_level() >= 1 || std::getenv("TIRAMISU_HIP_REPORT"))
             for (auto &k : ctx.kernels) std::cout << "[tiramisu-hip] " << f.get_name() << " " << k.name << ": " << k.how << std::endl;

@@ -44,6 +44,7 @@ class Buffer:
     def __init__(self, shape, dtype, host_ptr=0, device_ptr=0, keepalive=None):
         dtype = np.dtype(dtype)
         self.keepalive = keepalive
+        self.shape, self.dtype, self.on_device = tuple(int(v) for v in shape), dtype, bool(device_ptr)
         nd = len(shape)
         self.dims = (halide_dimension_t * max(nd, 1))()
         stride = 1
@@ -113,9 +114,35 @@ def wrappers():
     return _wrappers
 
 
+_C_TYPES = {"float": "float32", "double": "float64", "int8_t": "int8", "int16_t": "int16", "int32_t": "int32", "int64_t": "int64",
+            "uint8_t": "uint8", "uint16_t": "uint16", "uint32_t": "uint32", "uint64_t": "uint64", "bool": "bool",
+            "tiramisu_bf16_t": "uint16"}
+
+
+def manifest_of(library_path, function_name):
+    """The description the HIP back-end writes next to each object (``<object>.json``: arguments
+    with type, shape and memory space, kernels emitted) for the object that ``lib<stem>.so`` was
+    linked from (``<stem>.o`` or ``generated_fct_<stem>.o`` in the same directory), or None."""
+    import json
+    directory, base = os.path.split(os.path.abspath(library_path))
+    stem = base[3:-3] if base.startswith("lib") and base.endswith(".so") else base
+    for name in (stem + ".o.json", "generated_fct_" + stem + ".o.json"):
+        path = os.path.join(directory, name)
+        if os.path.exists(path):
+            try:
+                m = json.load(open(path))
+            except ValueError:
+                return None
+            return m if m.get("function") == function_name else None
+    return None
+
+
 class Program:
     """One compiled Tiramisu function: ``Program(path, "test_167")(A, B, C)`` with numpy arrays
-    and/or ``Buffer`` objects as arguments."""
+    and/or ``Buffer`` objects as arguments.  When the back-end's description of the function is
+    found next to the library, arguments are checked against it before the call (count, element
+    type, constant extents, host or device memory): a wrong buffer would otherwise be a
+    out-of-bounds access on the GPU."""
 
     def __init__(self, library_path, function_name, needs_gpu_runtime=True):
         if not os.path.exists(library_path):
@@ -125,9 +152,31 @@ class Program:
         self.lib = ctypes.CDLL(library_path)
         self.fn = getattr(self.lib, function_name)
         self.fn.restype = ctypes.c_int
+        self.name = function_name
+        self.manifest = manifest_of(library_path, function_name) if needs_gpu_runtime else None
+
+    def check(self, bufs):
+        expected = self.manifest["arguments"]
+        if len(bufs) != len(expected):
+            raise ValueError("%s takes %d buffers, %d given" % (self.name, len(expected), len(bufs)))
+        for b, e in zip(bufs, expected):
+            if np.dtype(_C_TYPES.get(e["type"], b.dtype)) != b.dtype:
+                raise ValueError("%s: buffer %s holds %s, %s given" % (self.name, e["name"], e["type"], b.dtype))
+            if (e["memory"] == "device") != b.on_device:
+                raise ValueError("%s: buffer %s lives in %s memory" % (self.name, e["name"], e["memory"]))
+            # a host input may be declared larger than what the program reads of it (the reference's
+            # sgemm generators declare their two scalars over the row range); anything the GPU
+            # touches, and every output, must have the declared number of elements
+            strict = e["memory"] == "device" or e["kind"] != "input"
+            if strict and all(isinstance(v, int) for v in e["shape"]):
+                want = int(np.prod(e["shape"])) if e["shape"] else 1
+                if int(np.prod(b.shape)) != want:
+                    raise ValueError("%s: buffer %s has shape %s, %s given" % (self.name, e["name"], e["shape"], list(b.shape)))
 
     def __call__(self, *args):
         bufs = [a if isinstance(a, Buffer) else Buffer.from_numpy(a) for a in args]
+        if self.manifest is not None:
+            self.check(bufs)
         rc = self.fn(*[b.pointer() for b in bufs])
         if rc != 0:
             raise RuntimeError("Tiramisu function returned %d" % rc)
