@@ -382,3 +382,17 @@ def ref_edge_gpu(img):
     t = lambda dj, di: R[:, dj:dj + M - 4, di:di + N - 4]          # R(i+di, j+dj)
     out = (t(1, 1) - t(0, 2)) + (t(1, 2) - t(0, 1))
     return (out % 256).astype(np.uint8)
+
+
+def lstm_gpu_packing(weights, biases, x):
+    """The stacked LSTM of lstm() on buffers packed the way the reference's GPU generators pack them
+    (benchmarks/DNN/blocks/LSTM/gpu/reference_generator.cpp:100-111 and gpu/generator.cpp:123-126, :256-257):
+    weight slot 0 holds the recurrent matrices R and slot 1 the input matrices W, and the 4H rows
+    are ordered i, z, o, f.  Restated by re-packing into lstm()'s layout (slot 0 = W, slot 1 = R;
+    rows i, f, z, o).  Pinned by the reference's own naive program, compiled unchanged
+    (tests/test_reference_generators.py: test_naive_lstm_program_pins_the_packing)."""
+    H = weights.shape[3]
+    blocks = [0, 3, 1, 2]                      # lstm()'s i, f, z, o taken from i, z, o, f
+    rows = np.concatenate([np.arange(b * H, (b + 1) * H) for b in blocks])
+    repacked = np.ascontiguousarray(weights[:, ::-1][:, :, rows, :])
+    return lstm(repacked, np.ascontiguousarray(biases[:, rows]), x)

@@ -98,6 +98,27 @@ def build_self_driven(rel, stem, obj):
                 "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
+# The reference's naive restatement of its LSTM (a CPU program: codegen without the GPU flag), compiled
+# unchanged through the oracle's CPU emitter: the pin of the numpy LSTM oracle's packing and gate order
+# for the reference's GPU generator (slot 0 = R, rows i, z, o, f).
+LSTM_NAIVE = "benchmarks/DNN/blocks/LSTM/gpu/reference_generator.cpp"
+
+
+def build_lstm_naive():
+    from oracle import build as oracle_build
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, "lstm_ref")
+    os.makedirs(work, exist_ok=True)
+    src = os.path.join(REFERENCE, LSTM_NAIVE)
+    gen = os.path.join(work, "gen")
+    cpu_dir = os.path.dirname(oracle_build.CPU_BACKEND)
+    build._run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"), "-o", gen, src,
+                "-L" + build.PKG, "-ltiramisu", "-Wl,--no-as-needed", "-L" + cpu_dir, "-ltiramisu_cpu_backend", "-Wl,--as-needed",
+                "-Wl,-rpath," + build.PKG, "-Wl,-rpath," + cpu_dir])
+    build._run([gen], cwd=work)
+    build._run(["g++", "-shared", "-fopenmp", "-o", library("lstm_ref"), os.path.join(work, "lstm_ref.o")])
+
+
 def build_all(verbose=False):
     if not os.path.isdir(REFERENCE):
         if verbose:
@@ -115,6 +136,9 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", rel, flush=True)
         build_self_driven(rel, stem, obj)
+    if verbose:
+        print("[reference programs]", LSTM_NAIVE, "(CPU)", flush=True)
+    build_lstm_naive()
     return True
 
 

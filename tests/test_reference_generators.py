@@ -318,3 +318,23 @@ def test_reference_chain_mm_generator():
     runtime.Program(library("chain_mm"), "matmul")(A, B, C, O)
     expected = ((A.astype(np.float64) @ B.astype(np.float64)) @ C.astype(np.float64)).astype(np.float32)
     assert np.array_equal(O, expected)
+
+
+@pytest.mark.parametrize("L,B,H,S", [(2, 3, 8, 4), (1, 2, 5, 3), (3, 4, 6, 2)])
+def test_naive_lstm_program_pins_the_packing(L, B, H, S):
+    """benchmarks/DNN/blocks/LSTM/gpu/reference_generator.cpp, unchanged (a CPU program: four separate gate sums with
+    explicit loops, sizes at run time), compiled through the oracle's CPU emitter: its output must be
+    what the numpy oracle computes once the buffers are re-packed from the GPU generators' layout
+    (slot 0 = R, rows i, z, o, f).  Summation order differs (a j loop here, matrix products there)."""
+    if not os.path.exists(library("lstm_ref")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    rng = np.random.RandomState(10 * L + H)
+    weights = rng.uniform(-0.5, 0.5, (L, 2, 4 * H, H)).astype(np.float32)
+    biases = rng.uniform(-0.5, 0.5, (L, 4 * H)).astype(np.float32)
+    x = rng.uniform(-1, 1, (S, B, H)).astype(np.float32)
+    y = np.zeros((S, B, H), np.float32)
+    runtime.Program(library("lstm_ref"), "lstm_ref", needs_gpu_runtime=False)(np.array([H, B, L, S], np.int32), weights, biases, x, y)
+    expected = ref.lstm_gpu_packing(weights, biases, x)
+    assert np.max(np.abs(y - expected)) <= 2e-6
+    # and the packing matters: without the re-packing the result is a different one
+    assert np.max(np.abs(y - ref.lstm(weights, biases, x))) > 1e-3
