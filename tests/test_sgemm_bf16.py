@@ -102,3 +102,20 @@ def test_gpu_4096_sampled_rows():
     out = run_gpu(M, N, K, scal, A, B, np.zeros((M, N), np.float32))
     exact = from_bf16(A[rows]).astype(np.float64) @ from_bf16(B).astype(np.float64)
     assert np.array_equal(out[rows], exact.astype(np.float32))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K", [(4096, 3072, 64), (3072, 4096, 192)])
+def test_gpu_large_tiles_short_k(M, N, K):
+    """256x256 tiles (slices loaded straight into the LDS ring) with one and three K-slices: the
+    ring's start-up and drain paths, every element checked, with the alpha / beta epilogue."""
+    rng = np.random.RandomState(M + K)
+    scal = np.array([1.5, 0.5], np.float32)
+    A, B = to_bf16(rng.randint(-4, 5, (M, K)).astype(np.float32)), to_bf16(rng.randint(-4, 5, (K, N)).astype(np.float32))
+    C = rng.randint(-8, 9, (M, N)).astype(np.float32)
+    exact = 1.5 * (from_bf16(A).astype(np.float64) @ from_bf16(B).astype(np.float64)) + 0.5 * C
+    assert np.array_equal(run_gpu(M, N, K, scal, A, B, C.copy()), exact.astype(np.float32))     # integer data: exact
+    A, B = to_bf16(rng.uniform(-1, 1, (M, K))), to_bf16(rng.uniform(-1, 1, (K, N)))
+    exact = 1.5 * (from_bf16(A).astype(np.float64) @ from_bf16(B).astype(np.float64)) + 0.5 * C
+    out = run_gpu(M, N, K, scal, A, B, C.copy())
+    assert np.max(np.abs(out - exact)) <= 1e-5 * np.max(np.abs(exact))

@@ -195,5 +195,182 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
     if (kt < KT) slice(kt, std::false_type(), std::false_type());
 }
 
+// ---------------------------------------------------------------------------------------------
+// Variant whose operand slices go from global memory straight into LDS (global_load_lds, 16 bytes
+// per lane: lane l of a wave-wide load writes LDS bytes [base + 16 l, base + 16 l + 16), the global
+// address is the lane's own), through a ring of STAGES slices: no staging registers, no LDS store
+// instructions, and STAGES-1 slices in flight.
+//   * A slice [BM][BK] is kept row-major in 16-byte granules (8 k), granule kq of row m at position
+//     kq ^ swzA(m); one 16-byte LDS read is a lane's MFMA operand.
+//   * B slice [BK][BN] is kept row-major as it is in memory ([k][n], granule = 8 columns), granule g
+//     of row k at position g ^ swzB(k).  The MFMA operand (8 consecutive k of one column) comes
+//     from two transposing LDS reads (ds_read_b64_tr_b16): within 16 lanes, lane L receives element
+//     L % 4 of the 8 bytes addressed by lanes L / 4, L / 4 + 4, L / 4 + 8, L / 4 + 12; so lane r of
+//     the 16 addresses row k0 + r / 4, columns n0 + 4 (r % 4) .. + 3, and lane L ends up with
+//     (k0 .. k0 + 3, column n0 + L).
+//   * The swizzles keep the reads free of bank conflicts whether the LDS serves 128 bytes (8 lanes of
+//     a 16-byte read, 16 of a transposing one) or 256 bytes per cycle: swzA spreads 8 and 16
+//     consecutive rows, swzB (0, 4, 10, 14 for k % 4) the four rows of a transposing read, over
+//     distinct 16-byte bank groups in both cases (measured: SQ_LDS_BANK_CONFLICT = 0).
+// A call ends with a barrier (every wave is past its last read), so it may be repeated for a second
+// pair of operands.  Rows of A and of B must be 16-byte aligned.
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, int STAGES_>
+struct config_bf16_direct {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_, STAGES = STAGES_;
+    static constexpr bool EDGE = false;
+    static constexpr int NW = WGM * WGN, NT = 64 * NW;
+    static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    static constexpr int GA = BK / 8, GB = BN / 8;          // 16-byte granules per row of the A / B slice
+    static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BK * BN * 2, STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int LA = BM * GA / 64 / NW, LB = BK * GB / 64 / NW;   // wave-wide loads per wave and slice
+    static_assert(BK == 32 || BK == 64, "slices of 32 or 64 k");
+    static_assert(BM * GA % (64 * NW) == 0 && BK * GB % (64 * NW) == 0, "slices must split evenly over the waves");
+    static_assert(GB >= 16 && (GB & (GB - 1)) == 0, "row of B: a power of two of 128 columns or more (the swizzle spans 16 granules)");
+    static_assert(STAGES >= 2, "the ring needs two stages or more");
+};
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+template <class CFG>
+__device__ __forceinline__ void tile_accumulate_bf16_direct(accumulators<CFG> &acc, const uint16_t *__restrict__ A, long lda,
+                                                            const uint16_t *__restrict__ B, long ldb, int K, int m0, int n0,
+                                                            uint32_t *lds) {
+    constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK, GA = CFG::GA, GB = CFG::GB, LA = CFG::LA, LB = CFG::LB, ST = CFG::STAGES;
+    constexpr int Q = BK / 16;
+    typedef __attribute__((address_space(3))) char lds_char;
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
+    const int l32 = lane & 31, h = lane >> 5;
+    lds_char *const base = (lds_char *)lds;
+    auto swzA = [](int m) -> int { return GA == 8 ? (m & 7) : (((m >> 2) & 1) | ((((m >> 1) ^ (m >> 3)) & 1) << 1)); };
+    auto swzB = [](int k) -> int { return ((k & 1) << 2) | ((k & 2) ? 10 : 0); };   // 0, 4, 10, 14
+
+    // per-lane global sources of this wave's loads (advanced by one slice after each issue)
+    const uint16_t *pa[LA], *pb[LB];
+#pragma unroll
+    for (int v = 0; v < LA; v++) {
+        const int g = (wave * LA + v) * 64 + lane, m = g / GA, kq = (g % GA) ^ swzA(m);
+        pa[v] = A + (long)(m0 + m) * lda + 8 * kq;
+    }
+#pragma unroll
+    for (int v = 0; v < LB; v++) {
+        const int g = (wave * LB + v) * 64 + lane, k = g / GB, n8 = (g % GB) ^ swzB(k);
+        pb[v] = B + (long)k * ldb + n0 + 8 * n8;
+    }
+    auto issue = [&](int stage) {
+#pragma unroll
+        for (int v = 0; v < LA; v++) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)pa[v],
+                                             (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + (wave * LA + v) * 1024), 16, 0, 0);
+            pa[v] += BK;
+        }
+#pragma unroll
+        for (int v = 0; v < LB; v++) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)pb[v],
+                                             (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + CFG::A_BYTES + (wave * LB + v) * 1024), 16, 0, 0);
+            pb[v] += (long)BK * ldb;
+        }
+    };
+
+    // fragment addresses within a stage, per MFMA step s: A granule (row, 2 s + h); B: two reads of four k
+    int offA[TM], offB[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) offA[i] = wm * CFG::WM + i * 32 + l32;                    // row
+    const int r16 = lane & 15, grp = lane >> 4;                                             // lane of the 16, group
+#pragma unroll
+    for (int j = 0; j < TN; j++) offB[j] = wn * CFG::WN + j * 32 + 16 * (grp & 1) + 4 * (r16 & 3);   // first column addressed
+    const int kB = 8 * (grp >> 1) + (r16 >> 2);                                            // row addressed within the step (first read)
+
+    bf16x8 fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int stage, int s, int buf) {
+        lds_char *const sa = base + stage * CFG::STAGE_BYTES, *const sb = sa + CFG::A_BYTES;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int m = offA[i], kq = 2 * s + h;
+            const u32x4 w = *reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(sa + (m * GA + (kq ^ swzA(m))) * 16);
+            fa[buf][i] = __builtin_bit_cast(bf16x8, w);
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            s16x4 lo, hi;
+            {
+                const int k = 16 * s + kB, n = offB[j];
+                lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(sb + (k * GB + ((n >> 3) ^ swzB(k))) * 16 + (n & 7) * 2));
+            }
+            {
+                const int k = 16 * s + kB + 4, n = offB[j];
+                hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(sb + (k * GB + ((n >> 3) ^ swzB(k))) * 16 + (n & 7) * 2));
+            }
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            fb[buf][j] = __builtin_bit_cast(bf16x8, both);
+        }
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc.t[i][j], 0, 0, 0);
+    };
+
+    // Ring: slice kt lives in stage kt % STAGES; all stages are requested up front.  In the last MFMA
+    // step of slice kt -- all of the wave's reads of that slice have returned -- one barrier both
+    // publishes slice kt+1 (every wave waited for its own loads of it) and retires slice kt's stage,
+    // into which slice kt+STAGES is requested: STAGES-1 slices of matrix work cover a load.
+    const int KT = K / BK;
+    constexpr int PER = LA + LB;                    // loads per wave and slice
+    constexpr int MFMAS = TM * TN, READS = TM + 2 * TN;
+    static_assert((ST - 1) * PER <= 63, "the load counter holds 63");
+#pragma unroll
+    for (int p = 0; p < ST; p++)
+        if (p < KT) issue(p);
+    if (KT >= ST) wait_vmcnt<(ST - 1) * PER>(); else wait_vmcnt<0>();      // slice 0 has landed
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_frags(0, 0, 0);
+    // ISSUE: slice kt+STAGES exists (steady state: exactly STAGES-2 requests are behind slice kt+1);
+    // MORE: slice kt+1 exists
+    auto slice = [&](int stage, int next, auto issue_c, auto more_c) {
+        constexpr bool ISSUE = decltype(issue_c)::value, MORE = decltype(more_c)::value;
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+            const int buf = q & 1;
+            if (q + 1 < Q) {
+                read_frags(stage, q + 1, buf ^ 1);
+            } else if (MORE) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (ISSUE) wait_vmcnt<(ST - 2) * PER>(); else wait_vmcnt<0>();
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+                if (ISSUE) issue(stage);
+                read_frags(next, 0, buf ^ 1);
+            }
+            multiply(buf);
+            if (q + 1 < Q || MORE) {
+#pragma unroll
+                for (int i = 0; i < MFMAS; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (q + 1 == Q && ISSUE && i < PER) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+                    if (i < READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+            }
+        }
+    };
+    int kt = 0, stage = 0;
+    auto advance = [&]() { kt++; stage = stage + 1 == ST ? 0 : stage + 1; };
+    for (; kt + ST < KT; advance()) slice(stage, stage + 1 == ST ? 0 : stage + 1, std::true_type(), std::true_type());
+    for (; kt + 1 < KT; advance()) slice(stage, stage + 1 == ST ? 0 : stage + 1, std::false_type(), std::true_type());
+    if (kt < KT) slice(stage, 0, std::false_type(), std::false_type());
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 }  // namespace tgemm
 #endif

@@ -918,7 +918,9 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const int NT = 64 * WGM * WGN * WGK;
     if (bf16) {
         body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
-        body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
+        // large tiles: slices go straight from global memory into a two-stage LDS ring
+        if (BM == 256) body << "    typedef tgemm::config_bf16_direct<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << ", 2> CFG;\n";
+        else body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
     } else {
         body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
         body << "    typedef " << cfg << " CFG;\n";
@@ -933,7 +935,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         if (bf16) {
             used_buffers.insert(o.first.buf->get_name());
             used_buffers.insert(o.second.buf->get_name());
-            body << "        tgemm::tile_accumulate_bf16<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
+            body << "        tgemm::tile_accumulate_bf16" << (BM == 256 ? "_direct" : "") << "<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
                  << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << "), " << dev.print(o.second.ld)
                  << ", _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
             term++;
@@ -1024,7 +1026,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     k.name = kname;
     bool any_gather = false;
     for (auto &o : operands) any_gather = any_gather || !o.first.linear || !o.second.linear;
-    k.how = std::string("mfma-contraction: ") + (bf16 ? "v_mfma_f32_32x32x16_bf16, " : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
+    k.how = std::string("mfma-contraction: ") + (bf16 ? (BM == 256 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
             std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
             std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
             std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
