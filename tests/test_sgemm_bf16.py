@@ -15,7 +15,7 @@ from tiramisu_amd import runtime
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
-SMALL = [(128, 192, 128), (48, 40, 24)]
+SMALL = [(128, 192, 128), (48, 40, 24), (1024, 1280, 512)]
 RTOL = 2e-2
 
 
@@ -105,10 +105,11 @@ def test_gpu_4096_sampled_rows():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N,K", [(4096, 3072, 64), (3072, 4096, 192)])
+@pytest.mark.parametrize("M,N,K", [(4096, 3072, 32), (3072, 4096, 160)])
 def test_gpu_large_tiles_short_k(M, N, K):
-    """256x256 tiles (slices loaded straight into the LDS ring) with one and three K-slices: the
-    ring's start-up and drain paths, every element checked, with the alpha / beta epilogue."""
+    """256x256 tiles (slices loaded straight into the four-stage LDS ring) with one and five K-slices:
+    the ring's start-up, a single steady-state turn and the drain, every element checked, with the
+    alpha / beta epilogue."""
     rng = np.random.RandomState(M + K)
     scal = np.array([1.5, 0.5], np.float32)
     A, B = to_bf16(rng.randint(-4, 5, (M, K)).astype(np.float32)), to_bf16(rng.randint(-4, 5, (K, N)).astype(np.float32))

@@ -16,7 +16,8 @@
 //   * Row m of k-group kq of A sits at position m ^ swz(kq) for the same reason (the lanes that
 //     store the k-groups of one row are 4096 bytes apart).
 // Whole tiles only: M % BM == 0, N % BN == 0, K % BK == 0, rows of A 16-byte and rows of B 8-byte
-// aligned (the emitter checks).
+// aligned (the emitter checks).  Large tiles use the second variant further down
+// (tile_accumulate_bf16_direct: slices loaded straight into an LDS ring); this one serves 64x64 tiles.
 #ifndef TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
 #define TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
 #include "gemm_mfma.hip.h"
@@ -196,7 +197,7 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
 }
 
 // ---------------------------------------------------------------------------------------------
-// Variant whose operand slices go from global memory straight into LDS (global_load_lds, 16 bytes
+// Variant whose operand slices go from global memory straight into LDS (buffer_load ... lds, 16 bytes
 // per lane: lane l of a wave-wide load writes LDS bytes [base + 16 l, base + 16 l + 16), the global
 // address is the lane's own), through a ring of STAGES slices: no staging registers, no LDS store
 // instructions, and STAGES-1 slices in flight.
@@ -234,8 +235,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 
 template <class CFG>
 __device__ __forceinline__ void tile_accumulate_bf16_direct(accumulators<CFG> &acc, const uint16_t *__restrict__ A, long lda,
-                                                            const uint16_t *__restrict__ B, long ldb, int K, int m0, int n0,
-                                                            uint32_t *lds) {
+                                                            const uint16_t *__restrict__ B, long ldb, int M, int N, int K, int m0,
+                                                            int n0, uint32_t *lds) {
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK, GA = CFG::GA, GB = CFG::GB, LA = CFG::LA, LB = CFG::LB, ST = CFG::STAGES;
     constexpr int Q = BK / 16;
     typedef __attribute__((address_space(3))) char lds_char;
@@ -245,34 +246,44 @@ __device__ __forceinline__ void tile_accumulate_bf16_direct(accumulators<CFG> &a
     const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
     const int l32 = lane & 31, h = lane >> 5;
     lds_char *const base = (lds_char *)lds;
-    auto swzA = [](int m) -> int { return GA == 8 ? (m & 7) : (((m >> 2) & 1) | ((((m >> 1) ^ (m >> 3)) & 1) << 1)); };
+    auto swzA = [](int m) -> int { return GA == 8 ? ((m ^ (m >> 3)) & 7) : (((m >> 2) & 1) | ((((m >> 1) ^ (m >> 3)) & 1) << 1)); };
     auto swzB = [](int k) -> int { return ((k & 1) << 2) | ((k & 2) ? 10 : 0); };   // 0, 4, 10, 14
 
-    // per-lane global sources of this wave's loads (advanced by one slice after each issue)
-    const uint16_t *pa[LA], *pb[LB];
+    // The loads are buffer loads (base in a resource descriptor, 32-bit byte offset per lane, one
+    // scalar offset per operand that advances by a slice): no 64-bit address arithmetic in the loop,
+    // and an address past the operand reads as zero instead of faulting.
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void *)A, 0, (int)((((long)M - 1) * lda + K) * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void *)B, 0, (int)((((long)K - 1) * ldb + N) * 2), 0x00020000);
+    int va[LA], vb[LB];                              // per-lane byte offsets of this wave's loads within a slice
 #pragma unroll
     for (int v = 0; v < LA; v++) {
         const int g = (wave * LA + v) * 64 + lane, m = g / GA, kq = (g % GA) ^ swzA(m);
-        pa[v] = A + (long)(m0 + m) * lda + 8 * kq;
+        va[v] = (int)(((long)(m0 + m) * lda + 8 * kq) * 2);
     }
 #pragma unroll
     for (int v = 0; v < LB; v++) {
         const int g = (wave * LB + v) * 64 + lane, k = g / GB, n8 = (g % GB) ^ swzB(k);
-        pb[v] = B + (long)k * ldb + n0 + 8 * n8;
+        vb[v] = (int)(((long)k * ldb + n0 + 8 * n8) * 2);
     }
+    int sa_off = 0, sb_off = 0;                      // byte offsets of the next slice to request
+    const int sb_step = (int)((long)BK * ldb * 2);
+    auto issue_one = [&](int stage, int v) {
+        if (v < LA) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + (wave * LA + v) * 1024), 16,
+                                                     va[v], sa_off, 0, 0);
+        } else {
+            const int u = v - LA;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + CFG::A_BYTES + (wave * LB + u) * 1024),
+                                                     16, vb[u], sb_off, 0, 0);
+        }
+        if (v == LA + LB - 1) {
+            sa_off += BK * 2;
+            sb_off += sb_step;
+        }
+    };
     auto issue = [&](int stage) {
 #pragma unroll
-        for (int v = 0; v < LA; v++) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)pa[v],
-                                             (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + (wave * LA + v) * 1024), 16, 0, 0);
-            pa[v] += BK;
-        }
-#pragma unroll
-        for (int v = 0; v < LB; v++) {
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)pb[v],
-                                             (__attribute__((address_space(3))) void *)(base + stage * CFG::STAGE_BYTES + CFG::A_BYTES + (wave * LB + v) * 1024), 16, 0, 0);
-            pb[v] += (long)BK * ldb;
-        }
+        for (int v = 0; v < LA + LB; v++) issue_one(stage, v);
     };
 
     // fragment addresses within a stage, per MFMA step s: A granule (row, 2 s + h); B: two reads of four k
@@ -284,54 +295,56 @@ __device__ __forceinline__ void tile_accumulate_bf16_direct(accumulators<CFG> &a
     for (int j = 0; j < TN; j++) offB[j] = wn * CFG::WN + j * 32 + 16 * (grp & 1) + 4 * (r16 & 3);   // first column addressed
     const int kB = 8 * (grp >> 1) + (r16 >> 2);                                            // row addressed within the step (first read)
 
-    bf16x8 fa[2][TM], fb[2][TN];
-    auto read_frags = [&](int stage, int s, int buf) {
+    // fragments: one set in use, one in flight; B fragments arrive as two halves (four k each)
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    bf16x8 fa[2][TM];
+    s16x4 fbl[2][TN], fbh[2][TN];
+    constexpr int MFMAS = TM * TN, READS = TM + 2 * TN;
+    // read number r of a step, in the order the matrix instructions need them (row 0 of A, all of B,
+    // the other rows of A)
+    auto read_one = [&](int stage, int s, int buf, int r) {
         lds_char *const sa = base + stage * CFG::STAGE_BYTES, *const sb = sa + CFG::A_BYTES;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
+        if (r == 0 || r > 2 * TN) {
+            const int i = r == 0 ? 0 : r - 2 * TN;
             const int m = offA[i], kq = 2 * s + h;
             const u32x4 w = *reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>(sa + (m * GA + (kq ^ swzA(m))) * 16);
             fa[buf][i] = __builtin_bit_cast(bf16x8, w);
-        }
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            s16x4 lo, hi;
-            {
-                const int k = 16 * s + kB, n = offB[j];
-                lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(sb + (k * GB + ((n >> 3) ^ swzB(k))) * 16 + (n & 7) * 2));
-            }
-            {
-                const int k = 16 * s + kB + 4, n = offB[j];
-                hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(sb + (k * GB + ((n >> 3) ^ swzB(k))) * 16 + (n & 7) * 2));
-            }
-            typedef short s16x8 __attribute__((ext_vector_type(8)));
-            const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            fb[buf][j] = __builtin_bit_cast(bf16x8, both);
+        } else {
+            const int j = (r - 1) / 2, half = (r - 1) % 2;
+            const int k = 16 * s + kB + 4 * half, n = offB[j];
+            const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(sb + (k * GB + ((n >> 3) ^ swzB(k))) * 16 + (n & 7) * 2));
+            if (half) fbh[buf][j] = v; else fbl[buf][j] = v;
         }
     };
-    auto multiply = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc.t[i][j], 0, 0, 0);
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / TN, j = idx % TN;
+        const s16x8 both = __builtin_shufflevector(fbl[buf][j], fbh[buf][j], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc.t[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], __builtin_bit_cast(bf16x8, both), acc.t[i][j], 0, 0, 0);
     };
 
     // Ring: slice kt lives in stage kt % STAGES; all stages are requested up front.  In the last MFMA
-    // step of slice kt -- all of the wave's reads of that slice have returned -- one barrier both
-    // publishes slice kt+1 (every wave waited for its own loads of it) and retires slice kt's stage,
-    // into which slice kt+STAGES is requested: STAGES-1 slices of matrix work cover a load.
+    // step of slice kt, after its first PRE matrix instructions (the wave's last reads of the slice,
+    // issued a dozen matrix instructions earlier, have returned by then), one barrier both publishes
+    // slice kt+1 (every wave waited for its own loads of it) and retires slice kt's stage, into which
+    // slice kt+STAGES is requested: STAGES-1 slices of matrix work cover a load.  The instruction
+    // order is pinned (a scheduling barrier after every matrix instruction): the LDS reads of the next
+    // step's fragments -- and, after the barrier, the slice's loads -- are dealt out behind the matrix
+    // instructions, with large wave tiles one read each, so that a fragment is requested at least seven
+    // matrix instructions before its use and the compiler's waits count exactly (buffer loads, unlike
+    // global or flat ones, do not make it wait for every outstanding LDS access).
     const int KT = K / BK;
     constexpr int PER = LA + LB;                    // loads per wave and slice
-    constexpr int MFMAS = TM * TN, READS = TM + 2 * TN;
+    constexpr int PRE = MFMAS >= 16 ? 4 : 1;        // matrix instructions of the last step ahead of the barrier
     static_assert((ST - 1) * PER <= 63, "the load counter holds 63");
+    constexpr int SLOTS = READS < MFMAS ? (READS > MFMAS - 4 ? READS : MFMAS - 4) : MFMAS;   // matrix instructions of a step that are followed by reads
 #pragma unroll
     for (int p = 0; p < ST; p++)
         if (p < KT) issue(p);
     if (KT >= ST) wait_vmcnt<(ST - 1) * PER>(); else wait_vmcnt<0>();      // slice 0 has landed
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    read_frags(0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < READS; r++) read_one(0, 0, 0, r);
     // ISSUE: slice kt+STAGES exists (steady state: exactly STAGES-2 requests are behind slice kt+1);
     // MORE: slice kt+1 exists
     auto slice = [&](int stage, int next, auto issue_c, auto more_c) {
@@ -340,25 +353,38 @@ __device__ __forceinline__ void tile_accumulate_bf16_direct(accumulators<CFG> &a
         for (int q = 0; q < Q; q++) {
             const int buf = q & 1;
             if (q + 1 < Q) {
-                read_frags(stage, q + 1, buf ^ 1);
+#pragma unroll
+                for (int idx = 0; idx < MFMAS; idx++) {
+                    mfma_one(buf, idx);
+#pragma unroll
+                    for (int r = idx * READS / SLOTS; r < (idx + 1) * READS / SLOTS; r++) read_one(stage, q + 1, buf ^ 1, r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             } else if (MORE) {
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int idx = 0; idx < PRE; idx++) {
+                    mfma_one(buf, idx);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 if (ISSUE) wait_vmcnt<(ST - 2) * PER>(); else wait_vmcnt<0>();
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
                 __builtin_amdgcn_sched_barrier(0);
-                if (ISSUE) issue(stage);
-                read_frags(next, 0, buf ^ 1);
-            }
-            multiply(buf);
-            if (q + 1 < Q || MORE) {
 #pragma unroll
-                for (int i = 0; i < MFMAS; i++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    if (q + 1 == Q && ISSUE && i < PER) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-                    if (i < READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                for (int idx = PRE; idx < MFMAS; idx++) {
+                    mfma_one(buf, idx);
+#pragma unroll
+                    for (int r = (idx - PRE) * READS / (MFMAS - PRE); r < (idx - PRE + 1) * READS / (MFMAS - PRE); r++) read_one(next, 0, buf ^ 1, r);
+                    if (ISSUE) {
+#pragma unroll
+                        for (int v = (idx - PRE) * PER / (MFMAS - PRE); v < (idx - PRE + 1) * PER / (MFMAS - PRE); v++) issue_one(stage, v);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+            } else {
+#pragma unroll
+                for (int idx = 0; idx < MFMAS; idx++) mfma_one(buf, idx);
             }
         }
     };

@@ -856,7 +856,9 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     if (bf16) {
         // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
         if (!lit) return reject(24);
-        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 64 == 0) { BM = BN = 256; BK = 64; }
+        // 256x256 when that fills the chip, else 128x128 (both load their slices straight into LDS), else 64x64
+        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 32 == 0) { BM = BN = 256; BK = 32; }
+        else if (Ml % 128 == 0 && Nl % 128 == 0 && Kl % 32 == 0 && (Ml / 128) * (Nl / 128) >= 48) { BM = BN = 128; BK = 32; }
         else if (Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0) { BM = BN = 64; BK = 64; }
         else return reject(24);
         WGM = WGN = 2;
@@ -865,7 +867,13 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
             if (!o.first.linear || !o.second.linear || !o.first.kmajor || o.second.kmajor) return reject(25);
             for (const operand_info *g : {&o.first, &o.second})
                 if (!literal_value(g->ld, v) || v % 8 != 0 || !literal_value(g->base, v) || v % 8 != 0) return reject(25);
+            // the large tiles address their operands with 32-bit byte offsets (buffer loads)
+            long lda = 0, ldb = 0;
+            literal_value(o.first.ld, lda);
+            literal_value(o.second.ld, ldb);
+            if (BM >= 128 && ((double)Ml * lda * 2 >= 2147483648.0 || (double)Kl * ldb * 2 >= 2147483648.0)) { BM = BN = 64; BK = 64; }
         }
+        if (BM == 64 && Kl % 64 != 0) return reject(24);
     }
     bool edge = !(lit && Ml % BM == 0 && Nl % BN == 0 && Kl % BK == 0);
     for (auto &o : operands)
@@ -918,8 +926,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const int NT = 64 * WGM * WGN * WGK;
     if (bf16) {
         body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
-        // large tiles: slices go straight from global memory into a two-stage LDS ring
-        if (BM == 256) body << "    typedef tgemm::config_bf16_direct<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << ", 2> CFG;\n";
+        // large tiles: slices go straight from global memory into a four-stage LDS ring
+        if (BM >= 128) body << "    typedef tgemm::config_bf16_direct<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << ", 4> CFG;\n";
         else body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
     } else {
         body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
@@ -935,9 +943,9 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         if (bf16) {
             used_buffers.insert(o.first.buf->get_name());
             used_buffers.insert(o.second.buf->get_name());
-            body << "        tgemm::tile_accumulate_bf16" << (BM == 256 ? "_direct" : "") << "<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
+            body << "        tgemm::tile_accumulate_bf16" << (BM >= 128 ? "_direct" : "") << "<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
                  << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << "), " << dev.print(o.second.ld)
-                 << ", _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+                 << (BM >= 128 ? ", _M, _N" : "") << ", _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
             term++;
             continue;
         }
@@ -1026,7 +1034,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     k.name = kname;
     bool any_gather = false;
     for (auto &o : operands) any_gather = any_gather || !o.first.linear || !o.second.linear;
-    k.how = std::string("mfma-contraction: ") + (bf16 ? (BM == 256 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
+    k.how = std::string("mfma-contraction: ") + (bf16 ? (BM >= 128 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
             std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
             std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
             std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
@@ -1065,7 +1073,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         const int rowA = operands[0].first.kmajor ? (BK / 4) * (BM + PADX) * 4 : BK * BM;
         const int rowB = operands[0].second.kmajor ? (BK / 4) * (BN + PADX) * 4 : BK * BN;
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
-        if (bf16) k.lds_bytes = std::to_string(2 * (BK / 8) * (BM + BN) * 4 * 4);
+        if (bf16) k.lds_bytes = std::to_string((BM >= 128 ? 4 : 2) * (BK / 8) * (BM + BN) * 4 * 4);   // four-stage ring for the large tiles
         else if (ktab_words) k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4 + ktab_words * 4);
     }
     std::ostringstream src;

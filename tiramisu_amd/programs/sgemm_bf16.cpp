@@ -69,8 +69,9 @@ static void generate(int M, int N, int K)
 int main()
 {
     generate(4096, 4096, 4096);   // benchmark configuration 3, bf16-input variant
-    generate(4096, 3072, 64);     // 256x256 tiles, a single K-slice
-    generate(3072, 4096, 192);    // 256x256 tiles, three K-slices (ring start-up and drain only)
+    generate(4096, 3072, 32);     // 256x256 tiles, a single K-slice
+    generate(3072, 4096, 160);    // 256x256 tiles, five K-slices: one steady-state turn of the four-stage ring, then the drain
+    generate(1024, 1280, 512);    // 128x128 tiles
     generate(128, 192, 128);      // whole 64x64x64 tiles: MFMA path
     generate(48, 40, 24);         // no whole tiles: schedule-faithful kernel
     return 0;
