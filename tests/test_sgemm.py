@@ -94,7 +94,7 @@ def test_gpu_uniform_inputs_within_tolerance(M, N, K):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K,tile", [(2048, 2048, 48, "128x128x16"), (3072, 3072, 32, "192x192x16"),
-                                        (1024, 1024, 1024, "64x64x32"), (4096, 4096, 4096, "256x256x16")])
+                                        (1024, 1024, 1024, "64x64x64"), (4096, 4096, 4096, "256x256x16")])
 def test_gpu_tile_chosen_for_the_launch(M, N, K, tile):
     """The C tile is the one whose launch is modelled fastest on 256 compute units; the two
     sizes that no other test reaches are also checked for exact results on integer data."""

@@ -849,10 +849,17 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
         DEPTH = (int)std::min<long>(4, std::max<long>(1, Kl / BK - 1));   // latency-bound: ask for (up to) all slices at once
     }
+    // at most one 64x64 tile per compute unit and a long reduction: two groups of wavefronts share each
+    // (64-k) slice, so that every SIMD has two wavefronts to alternate between (1024^3: 20.6 us against 21.9)
+    if (lit && !bf16 && BM == 64 && BN == 64 && WGK == 1 && Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0 && Kl >= 512 &&
+        (Ml / 64) * (Nl / 64) <= 256) {
+        WGK = 2; BK = 64;
+    }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
     if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_WGK")) WGK = std::atoi(e);
     if (bf16) {
         // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
         if (!lit) return reject(24);
