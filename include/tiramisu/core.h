@@ -5,6 +5,8 @@
 // constant :5212); the implementation is new and lowers to HIP for gfx950.
 #ifndef TIRAMISU_AMD_CORE_H
 #define TIRAMISU_AMD_CORE_H
+#include <cassert>
+#include <cmath>
 #include <map>
 #include <memory>
 #include <set>
@@ -159,6 +161,12 @@ public:
     void dump(bool exhaustive = false) const;
     void dump_schedule() const;
     void dump_sched_graph();
+    /** Gives every computation that stores somewhere and has no buffer yet a buffer shaped after its
+      * iteration domain (largest index + 1 per dimension) and maps it one to one: computations that no
+      * other computation reads become outputs, unscheduled ones (read only) inputs, the rest temporaries
+      * (reference: tiramisu_function.cpp:1458-1511, tiramisu_core.cpp:2268-2335). */
+    void allocate_and_map_buffers_automatically();
+    void dump_dep_graph();
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
                  const hardware_architecture_t arch);
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
@@ -406,6 +414,20 @@ public:
     virtual void skew(var i, var j, int factor, var ni, var nj);
     virtual void skew(var i, var j, int factor);
     virtual void skew(int i, int j, int factor);
+    /** Generalised skewing of two consecutive loops (reference: tiramisu_core.cpp:4305-4531, :4533-4560):
+      * i' = a i + b j, and j' = gamma i + sigma j with a sigma - gamma b = 1 -- gamma and sigma given,
+      * or found as the reference finds them (a, b reduced by their gcd first). */
+    virtual void skew(var i, var j, int a, int b, var ni, var nj);
+    virtual void skew(int i, int j, int a, int b);
+    virtual void skew(var i, var j, int alpha, int beta, int gamma, int sigma, var ni, var nj);
+    virtual void skew(int i, int j, int alpha, int beta, int gamma, int sigma);
+    /** Skewing of three / four consecutive loops by one factor: j' = f i + j, k' = f i + k (, l' = f i + l)
+      * (reference: tiramisu_core.cpp:3813-3972, :3974-4160). */
+    virtual void skew(var i, var j, var k, int factor, var ni, var nj, var nk);
+    virtual void skew(var i, var j, var k, var l, int factor, var ni, var nj, var nk, var nl);
+    virtual void skew(var i, var j, var k, int factor);
+    virtual void skew(var i, var j, var k, var l, int factor);
+    virtual void skew(int i, int j, int k, int l, int factor);
     virtual void loop_reversal(var old_var, var new_var);
     virtual void loop_reversal(int i);
     virtual void parallelize(var L);
@@ -479,7 +501,7 @@ public:
     constant(std::string param_name, const expr &param_expr);
     constant(std::string param_name, const expr &param_expr, primitive_t t, function *func);
     constant(std::string param_name, const expr &param_expr, primitive_t t, bool function_wide,
-             computation *with_computation, int at_loop_level, function *func);
+             computation *with_computation, int at_loop_level, function *func = nullptr /* the implicit function */);
     operator expr();
 };
 

@@ -12,6 +12,7 @@
 #include <cstring>
 #include <initializer_list>
 #include <memory>
+#include <string>
 #include <vector>
 
 #ifndef HALIDE_BUFFER_T_DEFINED
@@ -76,6 +77,12 @@ public:
     Buffer(int e0, int e1, int e2) { build({e0, e1, e2}); }
     Buffer(int e0, int e1, int e2, int e3) { build({e0, e1, e2, e3}); }
     explicit Buffer(const std::vector<int> &extents) { build(extents); }
+    // the same with a trailing name, which is only a label
+    Buffer(int e0, const std::string &) { build({e0}); }
+    Buffer(int e0, int e1, const std::string &) { build({e0, e1}); }
+    Buffer(int e0, int e1, int e2, const std::string &) { build({e0, e1, e2}); }
+    Buffer(int e0, int e1, int e2, int e3, const std::string &) { build({e0, e1, e2, e3}); }
+    Buffer(const std::vector<int> &extents, const std::string &) { build(extents); }
 
     halide_buffer_t *raw_buffer() { return &s->raw; }
     const halide_buffer_t *raw_buffer() const { return &s->raw; }

@@ -371,14 +371,16 @@ def ref_warp_affine_gpu(img):
 
 def ref_edge_gpu(img):
     """benchmarks/halide/edgegpu_tiramisu.cpp:25-31, :47-49, in place on a planar uint8 image [3][M][N]:
-    R = (ring of the 8 neighbours of the 3x3 window at (i, j)) / 8 in int arithmetic for i < N-2,
-    j < M-2, then Img(i, j) = (R(i+1,j+1) - R(i+2,j)) + (R(i+2,j+1) - R(i+1,j)) stored as uint8.  R is
+    R = (ring of the 8 neighbours of the 3x3 window at (i, j)) / 8 for i < N-2, j < M-2 -- in uint8
+    arithmetic: the operands are uint8 expressions, so the sum wraps modulo 256 before the division,
+    as in the Halide program the reference checks this benchmark against (edgegpu_ref.cpp:10-18;
+    tests/test_56.cpp + wrapper_test_56.cpp pin the same rule for a uint8 blur) -- then Img(i, j) = (R(i+1,j+1) - R(i+2,j)) + (R(i+2,j+1) - R(i+1,j)) stored as uint8.  R is
     defined for indices below N-2 / M-2 only, so the result is fixed for i < N-4, j < M-4; returns
     that region, [3][M-4][N-4]."""
     x = img.astype(np.int32)
     C, M, N = img.shape
     s = lambda dj, di: x[:, dj:dj + M - 2, di:di + N - 2]          # Img(i+di, j+dj)
-    R = (s(0, 0) + s(1, 0) + s(2, 0) + s(0, 1) + s(2, 1) + s(0, 2) + s(1, 2) + s(2, 2)) // 8
+    R = ((s(0, 0) + s(1, 0) + s(2, 0) + s(0, 1) + s(2, 1) + s(0, 2) + s(1, 2) + s(2, 2)) % 256) // 8
     t = lambda dj, di: R[:, dj:dj + M - 4, di:di + N - 4]          # R(i+di, j+dj)
     out = (t(1, 1) - t(0, 2)) + (t(1, 2) - t(0, 1))
     return (out % 256).astype(np.uint8)

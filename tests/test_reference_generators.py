@@ -48,6 +48,16 @@ def test_restatements_on_closed_forms():
     assert np.all(u == 0) and np.all(v == 0)
     assert np.allclose(ref.ref_warp_affine_gpu(np.full((20, 24), 77, np.uint8)), 77.0, rtol=1e-6)
     assert np.all(ref.ref_edge_gpu(np.full((3, 12, 14), 200, np.uint8)) == 0)
+    # edge, element by element in uint8 scalars (sums wrap before the division, as in Halide)
+    small = np.random.RandomState(9).randint(0, 256, (1, 7, 8)).astype(np.uint8)
+    with np.errstate(over="ignore"):
+        u8 = lambda j, i: small[0, j, i]
+        ring = lambda j, i: (u8(j, i) + u8(j + 1, i) + u8(j + 2, i) + u8(j, i + 1) + u8(j + 2, i + 1) + u8(j, i + 2) + u8(j + 1, i + 2)
+                             + u8(j + 2, i + 2)) // np.uint8(8)
+        by_hand = np.array([[(ring(j + 1, i + 1) - ring(j, i + 2)) + (ring(j + 1, i + 2) - ring(j, i + 1)) for i in range(4)] for j in range(3)],
+                           np.uint8)
+    assert np.array_equal(ref.ref_edge_gpu(small)[0], by_hand)
+    assert int(ring(0, 0)) == (sum(int(small[0, j, i]) for j in range(3) for i in range(3)) - int(small[0, 1, 1])) % 256 // 8
 
 
 @pytest.mark.parametrize("name", sorted(PROGRAMS))

@@ -10,7 +10,7 @@ by the back-end at code-generation time) in a scratch directory, calls the named
 seeded inputs shaped after the back-end's description of its arguments, and prints one line per
 variant, fastest first.  Every variant's outputs are compared with the first variant's: a knob must
 not change results (integer-valued inputs, so contraction kernels compare exactly too).
-Knobs: TIRAMISU_STENCIL_STEPS / _ROWS / _WAVES / _MERGE / _XCD, TIRAMISU_MFMA_TILE / _BK / _PAD / _DEPTH,
+Knobs: TIRAMISU_STENCIL_STEPS / _ROWS / _WAVES / _MERGE / _XCD, TIRAMISU_MFMA_TILE / _BK / _PAD / _DEPTH / _WGK,
 TIRAMISU_NO_MFMA, TIRAMISU_NO_STENCIL, TIRAMISU_HIP_SERIAL_HOST_LOOPS."""
 import argparse
 import itertools

@@ -446,6 +446,18 @@ void function::gen_isl_ast() {
 
 namespace lir {
 
+expr extent_of_dimension(function *f, isl_set *domain, int d) {
+    isl_pw_aff *largest = isl_set_dim_max(isl_set_copy(domain), d);
+    isl_ast_build *build = isl_ast_build_from_context(isl_set_params(isl_set_copy(domain)));
+    isl_ast_expr *e = isl_ast_build_expr_from_pw_aff(build, largest);
+    lowering L;
+    L.f = f;
+    expr r = simplify(L.from_isl(e, {}) + value_cast(global::get_loop_iterator_data_type(), 1));
+    isl_ast_expr_free(e);
+    isl_ast_build_free(build);
+    return r;
+}
+
 node_ptr canonical_nest(function &f, computation &c, bool as_written) {
     isl_ctx *ctx = f.get_isl_ctx();
     int n = isl_set_dim(c.get_iteration_domain(), isl_dim_set);

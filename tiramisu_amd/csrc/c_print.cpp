@@ -97,6 +97,10 @@ std::string c_printer::print(const expr &e) const {
     op_t o = e.get_op_type();
     primitive_t t = e.get_data_type();
     auto P = [&](int i) { return print(e.get_operand(i)); };
+    // C promotes 8- and 16-bit integers to int; the reference's expressions keep their type and wrap
+    // (uint8 + uint8 is a uint8), so arithmetic on narrow types is cast back after every operation
+    const bool narrow = t == p_uint8 || t == p_int8 || t == p_uint16 || t == p_int16;
+    auto keep = [&](const std::string &v) { return narrow ? "((" + primitive_c_name(t) + ")" + v + ")" : v; };
     auto bin = [&](const char *sym) { return "(" + P(0) + " " + sym + " " + P(1) + ")"; };
     if (const char *m = math_name(o)) {
         std::string fn = m;
@@ -104,17 +108,17 @@ std::string c_printer::print(const expr &e) const {
         return fn + "(" + P(0) + ")";
     }
     switch (o) {
-    case o_minus: return "(-" + P(0) + ")";
+    case o_minus: return keep("(-" + P(0) + ")");
     case o_abs: return (is_float_type(t) ? (t == p_float64 ? "fabs(" : "fabsf(") : "t_abs(") + P(0) + ")";
     case o_logical_not: return "(!" + P(0) + ")";
     case o_cast:
         if (t == p_bfloat16) return "t_bf16_to_f32(t_f32_to_bf16(" + P(0) + "))";
         return "((" + primitive_c_name(t) + ")(" + P(0) + "))";
-    case o_add: return bin("+");
-    case o_sub: return bin("-");
-    case o_mul: return bin("*");
-    case o_div: return bin("/");
-    case o_mod: return is_float_type(t) ? "fmod(" + P(0) + ", " + P(1) + ")" : bin("%");
+    case o_add: return keep(bin("+"));
+    case o_sub: return keep(bin("-"));
+    case o_mul: return keep(bin("*"));
+    case o_div: return keep(bin("/"));
+    case o_mod: return is_float_type(t) ? "fmod(" + P(0) + ", " + P(1) + ")" : keep(bin("%"));
     case o_floordiv: return "t_floordiv(" + P(0) + ", " + P(1) + ")";
     case o_floormod: return "t_floormod(" + P(0) + ", " + P(1) + ")";
     case o_logical_and: return bin("&&");
@@ -127,8 +131,8 @@ std::string c_printer::print(const expr &e) const {
     case o_gt: return bin(">");
     case o_max: return "t_max(" + P(0) + ", " + P(1) + ")";
     case o_min: return "t_min(" + P(0) + ", " + P(1) + ")";
-    case o_right_shift: return bin(">>");
-    case o_left_shift: return bin("<<");
+    case o_right_shift: return keep(bin(">>"));
+    case o_left_shift: return keep(bin("<<"));
     case o_select: case o_cond: return "(" + P(0) + " ? " + P(1) + " : " + P(2) + ")";
     case o_lerp: return "t_lerp(" + P(0) + ", " + P(1) + ", " + P(2) + ")";
     case o_access: {
@@ -164,7 +168,11 @@ std::string c_prelude(bool device) {
     os << "template <typename T> " << q << " T t_max(T a, T b) { return a > b ? a : b; }\n";
     os << "template <typename T> " << q << " T t_min(T a, T b) { return a < b ? a : b; }\n";
     os << "template <typename T> " << q << " T t_abs(T a) { return a < 0 ? -a : a; }\n";
-    os << "template <typename T> " << q << " T t_lerp(T a, T b, T w) { return a + (b - a) * w; }\n";
+    // lerp as the reference's CPU back-end (Halide) defines it: a (1 - w) + b w, an unsigned integer
+    // weight standing for w / (largest value of its type), rounded to nearest
+    os << "template <typename T> " << q << " T t_lerp(T a, T b, T w) { return a * (1 - w) + b * w; }\n";
+    os << q << " uint8_t t_lerp(uint8_t a, uint8_t b, uint8_t w) { return (uint8_t)(((uint32_t)a * (255u - w) + (uint32_t)b * w + 127u) / 255u); }\n";
+    os << q << " uint16_t t_lerp(uint16_t a, uint16_t b, uint16_t w) { return (uint16_t)(((uint64_t)a * (65535u - w) + (uint64_t)b * w + 32767u) / 65535u); }\n";
     // floor division and the remainder with the sign of the divisor's magnitude (Euclidean for
     // positive divisors): what the CPU back-end of the reference computes for integer / and %
     os << "template <typename T> " << q << " T t_floordiv(T a, T b) { T q = a / b; T r = a % b; "

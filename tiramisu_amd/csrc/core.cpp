@@ -562,7 +562,11 @@ int computation::get_iteration_domain_dimensions_number() const {
 
 void computation::allocate_and_map_buffer_automatically(argument_t type) {
     std::vector<expr> sizes;
-    if (declared_vars.empty()) {
+    const int ndims = isl_set_dim(iteration_domain, isl_dim_set);
+    if (declared_vars.empty() && ndims > 0 && iterator_names_ != std::vector<std::string>{"_zero"}) {
+        // domain given as an isl string: one buffer dimension per iterator, largest value + 1
+        for (int d = 0; d < ndims; d++) sizes.push_back(lir::extent_of_dimension(fct, iteration_domain, d));
+    } else if (declared_vars.empty()) {
         sizes.push_back(expr((int32_t)1));
     } else {
         for (auto &v : declared_vars) {
@@ -574,6 +578,28 @@ void computation::allocate_and_map_buffer_automatically(argument_t type) {
     automatically_allocated_buffer = new buffer(bname, sizes, data_type, type, fct);
     store_in(automatically_allocated_buffer);
 }
+
+static void collect_reads(const expr &e, std::set<std::string> &names) {
+    if (!e.is_defined()) return;
+    if (e.get_expr_type() == e_op && e.get_op_type() == o_access) names.insert(e.get_name());
+    for (auto &o : e.get_operands()) collect_reads(o, names);
+    for (auto &a : e.get_arguments()) collect_reads(a, names);
+}
+
+void function::allocate_and_map_buffers_automatically() {
+    std::set<std::string> read;
+    for (computation *c : body) {
+        collect_reads(c->get_expr(), read);
+        collect_reads(c->get_predicate(), read);
+    }
+    for (computation *c : body) {
+        if (!c->has_accesses() || c->get_access_relation() || c->get_automatically_allocated_buffer()) continue;
+        const argument_t kind = !c->should_schedule_this_computation() ? a_input : (read.count(c->get_name()) ? a_temporary : a_output);
+        c->allocate_and_map_buffer_automatically(kind);
+    }
+}
+
+void function::dump_dep_graph() { dump_sched_graph(); }
 
 buffer *computation::get_buffer() const {
     if (!access) return nullptr;
@@ -857,6 +883,82 @@ void computation::skew(var i, var j, int factor, var ni, var nj) {
     skew(l[0], l[1], factor);
     level_names[l[0]] = ni.get_name();
     level_names[l[1]] = nj.get_name();
+}
+
+void computation::skew(int i, int j, int alpha, int beta, int gamma, int sigma) {
+    if (i + 1 != j) ERROR("skew: the two loop levels must be consecutive, outer first", true);
+    if (std::abs(alpha * sigma - beta * gamma) != 1) ERROR("skew: alpha * sigma - beta * gamma must be 1 or -1", true);
+    std::vector<std::string> in, out;
+    range_vars((int)level_names.size(), in);
+    out = in;
+    const std::string &vi = in[dynamic_pos(i)], &vj = in[dynamic_pos(j)];
+    out[dynamic_pos(i)] = std::to_string(alpha) + "*" + vi + " + " + std::to_string(beta) + "*" + vj;
+    out[dynamic_pos(j)] = std::to_string(gamma) + "*" + vi + " + " + std::to_string(sigma) + "*" + vj;
+    apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+}
+void computation::skew(int i, int j, int a, int b) {
+    // the second row of the unimodular matrix, chosen as the reference chooses it (tiramisu_core.cpp:4445-4497)
+    if (b == 0 || a < 0) ERROR("skew: needs a >= 0 and b != 0", true);
+    int n1 = std::abs(a), n2 = std::abs(b);
+    if (n1 == 0) n1 = n2;
+    while (n1 != n2) { if (n1 > n2) n1 -= n2; else n2 -= n1; }
+    a /= n1;
+    b /= n1;
+    int gamma = 0, sigma = 1;
+    if (b == 1 || a == 1) gamma = a - 1;
+    else if (b == -1 && a > 1) { gamma = 1; sigma = 0; }
+    else {
+        bool found = false;
+        for (int t = 0; t < 100 && !found; t++) {
+            if ((sigma * a) % std::abs(b) == 1) found = true;
+            else sigma++;
+        }
+        if (!found) ERROR("skew: no integer solution of a * sigma - b * gamma = 1", true);
+        gamma = (sigma * a - 1) / b;
+    }
+    skew(i, j, a, b, gamma, sigma);
+}
+void computation::skew(var i, var j, int a, int b, var ni, var nj) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name()});
+    skew(l[0], l[1], a, b);
+    level_names[l[0]] = ni.get_name();
+    level_names[l[1]] = nj.get_name();
+}
+void computation::skew(var i, var j, int alpha, int beta, int gamma, int sigma, var ni, var nj) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name()});
+    skew(l[0], l[1], alpha, beta, gamma, sigma);
+    level_names[l[0]] = ni.get_name();
+    level_names[l[1]] = nj.get_name();
+}
+void computation::skew(int i, int j, int k, int l, int factor) {
+    skew(i, j, factor);
+    skew(i, k, factor);
+    skew(i, l, factor);
+}
+void computation::skew(var i, var j, var k, int factor) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name(), k.get_name()});
+    skew(l[0], l[1], factor);
+    skew(l[0], l[2], factor);
+}
+void computation::skew(var i, var j, var k, var l4, int factor) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name(), k.get_name(), l4.get_name()});
+    skew(l[0], l[1], l[2], l[3], factor);
+}
+void computation::skew(var i, var j, var k, int factor, var ni, var nj, var nk) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name(), k.get_name()});
+    skew(l[0], l[1], factor);
+    skew(l[0], l[2], factor);
+    level_names[l[0]] = ni.get_name();
+    level_names[l[1]] = nj.get_name();
+    level_names[l[2]] = nk.get_name();
+}
+void computation::skew(var i, var j, var k, var l4, int factor, var ni, var nj, var nk, var nl) {
+    auto l = get_loop_level_numbers_from_dimension_names({i.get_name(), j.get_name(), k.get_name(), l4.get_name()});
+    skew(l[0], l[1], l[2], l[3], factor);
+    level_names[l[0]] = ni.get_name();
+    level_names[l[1]] = nj.get_name();
+    level_names[l[2]] = nk.get_name();
+    level_names[l[3]] = nl.get_name();
 }
 
 void computation::loop_reversal(int i) {
@@ -1298,6 +1400,7 @@ Input::Input(std::string nm, std::vector<expr> sizes, primitive_t t) : input(nm,
 
 constant::constant(std::string param_name, const expr &param_expr, primitive_t t, bool function_wide,
                    computation *with_computation, int at_loop_level, function *func) {
+    if (!func) func = global::get_implicit_function();
     if (!func) ERROR("call tiramisu::init() first", true);
     if (function_wide != (with_computation == nullptr))
         ERROR("constant " + param_name + ": give a computation exactly when the constant is not function-wide", true);

@@ -2,6 +2,7 @@
 // Type rules follow the reference's constructors (include/tiramisu/expr.h:300-520):
 // arithmetic keeps the operands' common type, comparisons and logical operators give
 // p_boolean, a cast carries its target type.
+#include <unordered_map>
 #include <tiramisu/core.h>
 #include <tiramisu/debug.h>
 #include <tiramisu/expr.h>
@@ -235,18 +236,34 @@ expr cast(primitive_t t, const expr &e) {
 
 var::var() : var("_v" + std::to_string(counter++)) {}
 
-var::var(std::string nm, bool) {
-    etype = e_var;
-    dtype = global::get_loop_iterator_data_type();
-    defined = true;
-    name = nm;
+// Types of the variables declared so far, by name: a later var of the same name takes the declared type
+// (reference: var::declared_vars, tiramisu_expr.cpp:88-143; int32 / int64 are interchangeable there too).
+static std::unordered_map<std::string, primitive_t> &declared_var_types() {
+    static std::unordered_map<std::string, primitive_t> m;
+    return m;
 }
 
-var::var(primitive_t t, std::string nm, bool) {
+var::var(std::string nm, bool save) {
     etype = e_var;
+    auto d = declared_var_types().find(nm);
+    dtype = d != declared_var_types().end() ? d->second : global::get_loop_iterator_data_type();
+    defined = true;
+    name = nm;
+    if (save && d == declared_var_types().end()) declared_var_types()[nm] = dtype;
+}
+
+var::var(primitive_t t, std::string nm, bool save) {
+    etype = e_var;
+    auto d = declared_var_types().find(nm);
+    if (d != declared_var_types().end()) {
+        const bool ints = (t == p_int32 && d->second == p_int64) || (t == p_int64 && d->second == p_int32);
+        if (!ints && d->second != t) ERROR("variable " + nm + " was declared with another type before", true);
+        t = d->second;
+    }
     dtype = t;
     defined = true;
     name = nm;
+    if (save && d == declared_var_types().end()) declared_var_types()[nm] = dtype;
 }
 
 var::var(std::string nm, expr lower_bound, expr upper_bound) : var(nm) {

@@ -105,6 +105,10 @@ node_ptr canonical_nest(function &f, computation &c, bool as_written = false);
 expr coefficient(const expr &e, const std::string &v, bool &ok);
 bool mentions(const expr &e, const std::string &v);
 
+/** Number of values dimension `d` of `domain` spans from 0: its largest value + 1, as an expression over
+  * the domain's parameters (the size of a buffer dimension indexed by that iterator). */
+expr extent_of_dimension(function *f, isl_set *domain, int d);
+
 }  // namespace lir
 }  // namespace tiramisu
 #endif
