@@ -167,6 +167,12 @@ public:
       * (reference: tiramisu_function.cpp:1458-1511, tiramisu_core.cpp:2268-2335). */
     void allocate_and_map_buffers_automatically();
     void dump_dep_graph();
+    /** Print the iteration domains / the time-space domains (domain mapped through the schedule) of all
+      * computations (reference: core.h:1071-1109). */
+    void dump_iteration_domain() const;
+    void dump_time_processor_domain() const;
+    void dump_trimmed_time_processor_domain() const { dump_time_processor_domain(); }
+    constant *get_invariant_by_name(std::string str) const;
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
                  const hardware_architecture_t arch);
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,

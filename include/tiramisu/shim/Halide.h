@@ -45,6 +45,7 @@ class Buffer {
         size_t count = 0;
         std::vector<halide_dimension_t> dims;
         halide_buffer_t raw;
+        std::string name;
     };
     std::shared_ptr<storage> s;   // copies share the array, as Halide's do
 
@@ -77,13 +78,14 @@ public:
     Buffer(int e0, int e1, int e2) { build({e0, e1, e2}); }
     Buffer(int e0, int e1, int e2, int e3) { build({e0, e1, e2, e3}); }
     explicit Buffer(const std::vector<int> &extents) { build(extents); }
-    // the same with a trailing name, which is only a label
-    Buffer(int e0, const std::string &) { build({e0}); }
-    Buffer(int e0, int e1, const std::string &) { build({e0, e1}); }
-    Buffer(int e0, int e1, int e2, const std::string &) { build({e0, e1, e2}); }
-    Buffer(int e0, int e1, int e2, int e3, const std::string &) { build({e0, e1, e2, e3}); }
-    Buffer(const std::vector<int> &extents, const std::string &) { build(extents); }
+    // the same with a trailing name (a label: print_buffer shows it)
+    Buffer(int e0, const std::string &nm) { build({e0}); s->name = nm; }
+    Buffer(int e0, int e1, const std::string &nm) { build({e0, e1}); s->name = nm; }
+    Buffer(int e0, int e1, int e2, const std::string &nm) { build({e0, e1, e2}); s->name = nm; }
+    Buffer(int e0, int e1, int e2, int e3, const std::string &nm) { build({e0, e1, e2, e3}); s->name = nm; }
+    Buffer(const std::vector<int> &extents, const std::string &nm) { build(extents); s->name = nm; }
 
+    const std::string &name() const { return s->name; }
     halide_buffer_t *raw_buffer() { return &s->raw; }
     const halide_buffer_t *raw_buffer() const { return &s->raw; }
     // Generated functions of this build leave their results in host memory (explicit or

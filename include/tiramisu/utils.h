@@ -5,6 +5,7 @@
 #ifndef TIRAMISU_AMD_UTILS_H
 #define TIRAMISU_AMD_UTILS_H
 #include "Halide.h"      // Halide's own, or tiramisu/shim/Halide.h when that directory is on the include path (reference: utils.h:4)
+#include <tiramisu/debug.h>
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
@@ -37,6 +38,29 @@ inline void copy_buffer(const Halide::Buffer<T> &from, Halide::Buffer<T> &to)
 }
 
 /** Report a test's outcome; a failure is reported, not fatal (reference: utils.h:227-233). */
+/** Prints the elements of a buffer of up to three dimensions, one row per line
+  * (reference: utils.h:37-66). */
+template <typename T>
+inline void print_buffer(const Halide::Buffer<T> &buf)
+{
+    std::cout << "Printing " << buf.name() << "[";
+    if (buf.channels() > 1) std::cout << buf.channels() << ",";
+    if (buf.height() > 1) std::cout << buf.height() << ",";
+    std::cout << buf.width() << "]: " << std::endl;
+    for (int z = 0; z < buf.channels(); z++) {
+        for (int y = 0; y < buf.height(); y++) {
+            for (int x = 0; x < buf.width(); x++) {
+                if (sizeof(T) == 1) std::cout << (int)buf(x, y, z);
+                else std::cout << buf(x, y, z);
+                if (x + 1 != buf.width()) std::cout << ", ";
+            }
+            std::cout << "\n";
+        }
+        std::cout << std::endl;
+    }
+    std::cout << std::endl;
+}
+
 inline void print_test_results(const std::string &test, bool success)
 {
     if (success) std::cout << "\033[1;32mTest " << test << " succeeded.\033[0m" << std::endl;

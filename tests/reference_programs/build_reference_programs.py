@@ -134,6 +134,21 @@ SUITE = """01 02 03 04 06 07 08 09 10 11 12 13 16 17 18 19 20 41 42 43 44 45 46 
 176 177 178 197""".split()
 
 
+# Developer tutorials of the reference that pass the same way (04gpu and 04gpu2 run on the GPU, above; 01's
+# wrapper hands an int32 buffer to a uint8 function, 11 and 12 are distributed, 13 accesses a 2-D computation
+# with one index -- an error in the reference too).
+SUITE_TUTORIALS = ["tutorial_02", "tutorial_03", "tutorial_04A", "tutorial_04B", "tutorial_05", "tutorial_06", "tutorial_07", "tutorial_08",
+                   "tutorial_10"]
+
+
+def suite_sources(n):
+    if n.startswith("tutorial_"):
+        d = os.path.join(REFERENCE, "tutorials", "developers", n)
+        return d, os.path.join(d, n + ".cpp"), os.path.join(d, "wrapper_" + n + ".cpp")
+    d = os.path.join(REFERENCE, "tests")
+    return d, os.path.join(d, "test_%s.cpp" % n), os.path.join(d, "wrapper_test_%s.cpp" % n)
+
+
 def suite_program(n):
     return os.path.join(HERE, "build", "suite", n, "wrapper")
 
@@ -143,11 +158,11 @@ def build_suite_test(n):
     from oracle import build as oracle_build
     work = os.path.join(HERE, "build", "suite", n)
     os.makedirs(os.path.join(work, "build"), exist_ok=True)
-    tests = os.path.join(REFERENCE, "tests")
+    tests, generator_source, wrapper_source = suite_sources(n)
     shim = os.path.join(build.INCLUDE, "tiramisu", "shim")
     cpu_dir = os.path.dirname(oracle_build.CPU_BACKEND)
     gen = os.path.join(work, "gen")
-    build._run(["g++", "-std=c++17", "-O0", "-w", "-I" + build.INCLUDE, "-I" + shim, "-I" + tests, "-o", gen, os.path.join(tests, "test_%s.cpp" % n),
+    build._run(["g++", "-std=c++17", "-O0", "-w", "-I" + build.INCLUDE, "-I" + shim, "-I" + tests, "-o", gen, generator_source,
                 "-L" + build.PKG, "-ltiramisu", "-Wl,--no-as-needed", "-L" + cpu_dir, "-ltiramisu_cpu_backend", "-Wl,--as-needed",
                 "-Wl,-rpath," + build.PKG, "-Wl,-rpath," + cpu_dir])
     for f in os.listdir(os.path.join(work, "build")):
@@ -159,8 +174,8 @@ def build_suite_test(n):
         raise RuntimeError("generator of reference test %s failed:\n%s" % (n, r.stdout[-2000:]))
     objects = [os.path.join(work, "build", f) for f in os.listdir(os.path.join(work, "build")) if f.endswith(".o")]
     build._run(["g++", "-std=c++17", "-O0", "-w", "-fopenmp", "-I" + build.INCLUDE, "-I" + shim, "-I" + tests, "-o", suite_program(n),
-                os.path.join(tests, "wrapper_test_%s.cpp" % n)] + objects +
-               ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, work)])
+                wrapper_source] + objects +
+               ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-ltiramisu", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, work)])
 
 
 def build_suite(verbose=False):
@@ -168,7 +183,7 @@ def build_suite(verbose=False):
     if verbose:
         print("[reference programs] tests/test_N.cpp + wrapper_test_N.cpp: %d tests through the CPU emitter" % len(SUITE), flush=True)
     with ThreadPoolExecutor(8) as pool:
-        list(pool.map(build_suite_test, SUITE))
+        list(pool.map(build_suite_test, SUITE + SUITE_TUTORIALS))
 
 
 def build_all(verbose=False):

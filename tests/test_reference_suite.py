@@ -16,7 +16,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests", "reference_programs"))
 import build_reference_programs as brp  # noqa: E402
 
 
-@pytest.mark.parametrize("n", brp.SUITE)
+@pytest.mark.parametrize("n", brp.SUITE + brp.SUITE_TUTORIALS)
 def test_reference_test_passes(n):
     program = brp.suite_program(n)
     assert os.path.exists(program), "not built: run tests/reference_programs/build_reference_programs.py where the reference tree is"

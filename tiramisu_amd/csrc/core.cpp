@@ -601,6 +601,26 @@ void function::allocate_and_map_buffers_automatically() {
 
 void function::dump_dep_graph() { dump_sched_graph(); }
 
+void function::dump_iteration_domain() const {
+    for (auto c : body) c->dump_iteration_domain();
+}
+
+void function::dump_time_processor_domain() const {
+    for (auto c : body) {
+        isl_set *ts = isl_set_apply(isl_set_copy(c->get_iteration_domain()), isl_map_copy(c->get_schedule()));
+        char *str = isl_set_to_str(ts);
+        std::cout << c->get_name() << ": " << str << std::endl;
+        free(str);
+        isl_set_free(ts);
+    }
+}
+
+constant *function::get_invariant_by_name(std::string str) const {
+    for (auto c : invariants)
+        if (c->get_name() == str) return static_cast<constant *>(c);
+    return nullptr;
+}
+
 buffer *computation::get_buffer() const {
     if (!access) return nullptr;
     const char *bn = isl_map_get_tuple_name(access, isl_dim_out);
