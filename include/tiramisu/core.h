@@ -271,6 +271,8 @@ protected:
     primitive_t data_type = p_none;
     bool schedule_this = true;
     bool is_let = false;
+    computation *first_definition = nullptr;     // set for an update
+    std::vector<computation *> updates;          // of a first definition
     bool inline_ = false;
     buffer *automatically_allocated_buffer = nullptr;
     std::vector<std::pair<std::string, expr>> associated_let_stmts;
@@ -355,6 +357,19 @@ public:
     bool has_accesses() const;
     buffer *get_buffer() const;
     buffer *get_automatically_allocated_buffer() const { return automatically_allocated_buffer; }
+
+    /** Further definitions of this computation over other parts of its domain ("updates": C[0] = ...,
+      * then C[i] = f(C[i-1]) for i >= 1).  Each is a computation of its own for scheduling and data
+      * mapping, reached with get_update(k) (0 is this computation); accesses C(...) in expressions read
+      * through the first definition's mapping, so all definitions are expected to store in one buffer
+      * (reference: core.h:3236-3262, tiramisu_core.cpp:254-273; internally a definition is named
+      * _<name>_update_<k>). */
+    void add_definitions(std::string iteration_domain, expr e, bool schedule_this_computation, primitive_t t, function *fct);
+    computation &get_update(int index);
+    computation *get_first_definition() { return first_definition ? first_definition : this; }
+    computation &get_last_update() { return updates.empty() ? *this : *updates.back(); }
+    bool is_first_definition() const { return first_definition == nullptr; }
+    const std::vector<computation *> &get_updates() const { return updates; }
     buffer *auto_buffer() const { return automatically_allocated_buffer; }
     const std::vector<std::pair<std::string, expr>> &get_associated_let_stmts() const { return associated_let_stmts; }
     int get_loop_level_number_from_dimension_name(std::string dim_name) const {

@@ -248,6 +248,10 @@ void function::gen_ordering_schedules() {
 }
 
 void function::gen_time_space_domain() {
+    // an update without a mapping of its own stores where its first definition stores
+    for (auto c : body)
+        if (!c->is_first_definition() && !c->get_access_relation() && c->get_first_definition()->get_access_relation())
+            c->set_access(isl_map_copy(c->get_first_definition()->get_access_relation()));
     gen_ordering_schedules();
     align_schedules();
     for (auto c : body) c->gen_time_space_domain();
@@ -594,9 +598,13 @@ void function::allocate_and_map_buffers_automatically() {
     }
     for (computation *c : body) {
         if (!c->has_accesses() || c->get_access_relation() || c->get_automatically_allocated_buffer()) continue;
+        if (!c->is_first_definition()) continue;      // updates share the first definition's buffer, below
         const argument_t kind = !c->should_schedule_this_computation() ? a_input : (read.count(c->get_name()) ? a_temporary : a_output);
         c->allocate_and_map_buffer_automatically(kind);
     }
+    for (computation *c : body)
+        if (!c->is_first_definition() && c->has_accesses() && !c->get_access_relation() && c->get_first_definition()->get_buffer())
+            c->store_in(c->get_first_definition()->get_buffer());
 }
 
 void function::dump_dep_graph() { dump_sched_graph(); }
@@ -642,7 +650,30 @@ void computation::set_access(std::string access_str) {
 
 void computation::set_access(isl_map *acc) {
     if (access) isl_map_free(access);
+    // an update is addressed by the name of its first definition in the relations the user writes
+    if (first_definition && acc) acc = isl_map_set_tuple_name(acc, isl_dim_in, name.c_str());
     access = acc;
+}
+
+void computation::add_definitions(std::string iteration_domain_str, expr e, bool schedule_this_computation, primitive_t t, function *f) {
+    if (first_definition) ERROR("add_definitions: call it on the first definition of " + first_definition->get_name(), true);
+    isl_set *dom = isl_set_read_from_str(ctx, iteration_domain_str.c_str());
+    if (!dom) ERROR("cannot parse iteration domain " + iteration_domain_str, true);
+    const std::string update_name = "_" + name + "_update_" + std::to_string(updates.size() + 1);
+    dom = isl_set_set_tuple_name(dom, update_name.c_str());
+    char *text = isl_set_to_str(dom);
+    computation *c = new computation(std::string(text), e, schedule_this_computation, t, f);
+    free(text);
+    isl_set_free(dom);
+    c->first_definition = this;
+    c->is_let = is_let;
+    updates.push_back(c);
+}
+
+computation &computation::get_update(int index) {
+    if (index == 0) return *this;
+    if (index < 0 || index > (int)updates.size()) ERROR("get_update: " + name + " has no definition number " + std::to_string(index), true);
+    return *updates[index - 1];
 }
 
 void computation::store_in(buffer *buff) {
