@@ -128,8 +128,8 @@ def build_lstm_naive():
 # 10-element buffer handed to a 100-iteration loop); 133-140 (a recurrence whose dependent loop the test
 # tags parallel: the result depends on thread timing).
 SUITE = """01 02 03 04 06 07 08 09 10 11 12 13 16 17 18 19 20 26 41 42 43 44 45 46 47 48 51 52 53 54 55 56 57 58 59 60 61 62 63 64
-65 66 67 68 69 70 71 72 74 75 76 77 78 80 81 84 89 91 97 103 104 105 107 108 109 110 111 112 113 114 115 116 117 118 119 120 121 122 123
-125 126 127 128 129 131 141 142 143 144 145 146 147 148 149 150 151 152 153 154 155 156 157 158 159 161 163 167 168 169 170 171 175
+65 66 67 68 69 70 71 72 73 74 75 76 77 78 80 81 84 87 88 89 91 97 103 104 105 106 107 108 109 110 111 112 113 114 115 116 117 118 119 120 121 122 123
+124 125 126 127 128 129 131 141 142 143 144 145 146 147 148 149 150 151 152 153 154 155 156 157 158 159 161 163 167 168 169 170 171 175
 176 177 178 197""".split()
 
 

@@ -137,7 +137,14 @@ std::string c_printer::print(const expr &e) const {
     case o_lerp: return "t_lerp(" + P(0) + ", " + P(1) + ", " + P(2) + ")";
     case o_access: {
         auto it = fct->get_buffers().find(e.get_name());
-        if (it == fct->get_buffers().end()) ERROR("access to unknown buffer " + e.get_name(), true);
+        if (it == fct->get_buffers().end()) {
+            // an access to a computation outside a loop nest (the size of a buffer read from an input, as in
+            // S0_b({N_input(0), N_input(0)})): the element of the computation's buffer, for one-to-one mappings
+            for (computation *c : fct->get_computations())
+                if (c->get_name() == e.get_name() && c->get_buffer() && (int)e.get_access().size() == c->get_buffer()->get_n_dims())
+                    return element(c->get_buffer(), e.get_access());
+            ERROR("access to unknown buffer " + e.get_name(), true);
+        }
         std::string s = element(it->second, e.get_access());
         if (it->second->get_elements_type() == p_bfloat16) s = "t_bf16_to_f32(" + s + ")";
         return s;

@@ -682,19 +682,20 @@ void computation::store_in(buffer *buff) {
     // A buffer with fewer dimensions than the domain takes the innermost iterators.
     int nb = buff->get_n_dims();
     for (int i = std::max(0, n - nb); i < n; i++) idx.push_back(var(iterator_names_[i]));
-    if (declared_vars.empty() && n == 1) idx = {expr((int32_t)0)};
+    if (iterator_names_ == std::vector<std::string>{"_zero"}) idx = {expr((int32_t)0)};   // a computation without iterators
     store_in(buff, idx);
 }
 
 void computation::store_in(buffer *buff, std::vector<expr> iterators) {
+    // no index at all: every iteration stores into element 0 (a scalar kept in a one-element buffer)
+    if (iterators.empty()) iterators.assign(std::max(1, buff->get_n_dims()), expr((int32_t)0));
     std::vector<std::string> out;
     for (auto &e : iterators) {
         bool ok = true;
         out.push_back(expr_to_isl_str(e, ok));
         if (!ok) ERROR("store_in of " + name + ": index " + e.to_str() + " is not affine", true);
     }
-    std::vector<std::string> in = iterator_names_;
-    if (declared_vars.empty() && in.size() == 1) in = {"_zero"};
+    const std::vector<std::string> &in = iterator_names_;
     std::string s = params_prefix(fct->get_invariant_names()) + "{ " + name + "[" + join(in, ", ") + "] -> " +
                     buff->get_name() + "[" + join(out, ", ") + "] }";
     set_access(s);
