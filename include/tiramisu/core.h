@@ -364,6 +364,10 @@ public:
       * through the first definition's mapping, so all definitions are expected to store in one buffer
       * (reference: core.h:3236-3262, tiramisu_core.cpp:254-273; internally a definition is named
       * _<name>_update_<k>). */
+    /** Gives this computation a temporary buffer of its whole size, allocated inside the loop nest of
+      * \p comp at loop level \p L0, right before \p comp there (reference: tiramisu_core.cpp:1138-1171);
+      * returns the allocation. */
+    computation *store_at(computation &comp, var L0);
     void add_definitions(std::string iteration_domain, expr e, bool schedule_this_computation, primitive_t t, function *fct);
     computation &get_update(int index);
     computation *get_first_definition() { return first_definition ? first_definition : this; }

@@ -670,6 +670,16 @@ void computation::add_definitions(std::string iteration_domain_str, expr e, bool
     updates.push_back(c);
 }
 
+computation *computation::store_at(computation &comp, var L0) {
+    const int level = comp.get_loop_level_number_from_dimension_name(L0.get_name());
+    allocate_and_map_buffer_automatically(a_temporary);
+    if (!automatically_allocated_buffer) ERROR("store_at: the size of " + name + " is not known", true);
+    computation *allocation = automatically_allocated_buffer->allocate_at(comp, level);
+    if (comp.get_predecessor()) allocation->between(*comp.get_predecessor(), L0, comp, L0);
+    else allocation->before(comp, level);
+    return allocation;
+}
+
 computation &computation::get_update(int index) {
     if (index == 0) return *this;
     if (index < 0 || index > (int)updates.size()) ERROR("get_update: " + name + " has no definition number " + std::to_string(index), true);
