@@ -4,15 +4,24 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|heat2d|sgemm1024|sgemm4096|...]
 
 Prints ONE JSON line.  The headline is benchmark configuration 2 (heat2d 8192x8192, 32 time steps,
-the configuration the HBM-roofline target is quoted on): `value` is algorithmic HBM GB/s of the
-whole compiled Tiramisu function with its buffers already resident in HBM.  A "step" is one
-call of the compiled function (32 stencil time steps).  The other configurations that exist
-as compiled programs are measured the same way and reported under "workloads".
+the configuration the HBM-roofline target is quoted on).  A "step" is one call of the compiled
+Tiramisu function (32 stencil time steps) with its buffers already resident in HBM.  The compiled
+function fuses up to 11 time steps per launch, so it moves far fewer bytes than the un-fused
+program's 8 bytes per cell and time step: `value` is the HBM traffic the function really causes
+(hardware counters, per kernel, from profiles/hbm_traffic_by_kernel.md) per second, and
+`algorithmic_gbs` -- the un-fused program's bytes per second of this run, the figure that time
+tiling raises above the HBM peak -- is kept beside it.  The other configurations that exist as
+compiled programs are measured the same way and reported under "workloads".
 
-`roofline` is measured per kernel with HIP events around every launch (the runtime ABI's
-tiramisu_hip_profile_*), on the stream the generated code launches on.  `cpu_baseline` times
-the CPU-generated code of the same Tiramisu program (the oracle's CPU back-end restatement:
-parallelize + vectorize schedule, OpenMP) on the host cores of this machine.
+`roofline` is for the kernel with the largest share of the time, its duration measured here with
+HIP events around every launch (the runtime ABI's tiramisu_hip_profile_*) on the stream the
+generated code launches on: flops per launch over duration against the MFMA peak for the
+contractions; counter-measured HBM bytes per launch over duration against the HBM peak for the
+stencil (`frac` <= 1 by construction; `algorithmic_gbs` and `vector_alu_busy` say why a fused
+launch sits below the HBM peak).  `traffic` is looked up by the emitter's own description of the
+kernel, so a kernel the table does not know reports null instead of a stale figure.
+`cpu_baseline` times the CPU-generated code of the same Tiramisu program (the oracle's CPU
+back-end restatement: parallelize + vectorize schedule, OpenMP) on the host cores of this machine.
 """
 import argparse
 import json
@@ -31,13 +40,34 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
-# HBM bytes per launch of the dominant heat2d kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size); see profiles/.
-HEAT2D_TRAFFIC_BYTES_PER_LAUNCH = {   # by time steps per launch; KiB counters x calibration factor
-    11: (176981.2 * 2.000 + 262402.5 * 1.000) * 1024,
-    9: (172771.4 * 2.000 + 262401.0 * 1.000) * 1024,
-    1: (144475.0 * 2.000 + 266309.6 * 1.000) * 1024,
-}
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_by_kernel.md")
+
+
+def traffic_table():
+    """{(function, kernel description): {"bytes": HBM bytes per launch, "vector_alu_busy": share or None}} from the
+    table of counter measurements in profiles/ (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
+    scaled by what the same counters read for a plain copy of known size)."""
+    out = {}
+    if not os.path.exists(TRAFFIC_TABLE):
+        return out
+    for line in open(TRAFFIC_TABLE):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) < 6 or not cells[4].replace(".", "", 1).isdigit():
+            continue
+        busy = cells[5].rstrip("%").strip()
+        out[(cells[0].strip("`"), cells[1].strip("`"))] = {
+            "bytes": float(cells[4]), "vector_alu_busy": float(busy) / 100.0 if busy.replace(".", "", 1).isdigit() else None}
+    return out
+
+
+def kernel_descriptions(name):
+    """{kernel name: the emitter's description of it} from the manifest written beside the object."""
+    with open(os.path.join(PROGRAMS, "build", name + ".o.json")) as f:
+        return {k["name"]: k["how"] for k in json.load(f)["kernels"]}
+
+
+def kernel_traffic(name, kernel):
+    return traffic_table().get((name, kernel_descriptions(name).get(kernel, "")))
 
 
 def device_array(host):
@@ -83,8 +113,9 @@ def kernel_profile(call, steps):
     return {k: (float(np.mean(v)), len(v) // steps) for k, v in by.items()}
 
 
-def cpu_time(call, min_seconds=3.0, max_runs=5):
-    call()  # warm-up
+def cpu_time(call, min_seconds=3.0, max_runs=5, warm=True):
+    if warm:
+        call()  # warm-up
     ts = []
     t_all = time.perf_counter()
     while len(ts) < max_runs and (len(ts) < 1 or time.perf_counter() - t_all < min_seconds):
@@ -138,15 +169,31 @@ def bench_heat2d(steps, warmup, with_cpu):
     dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
     # algorithmic bytes of one launch: every cell the kernel advances is read once and written once per step
     fused_steps, cells = stencil_kernels(os.path.join(PROGRAMS, "build", name + ".o.hip"), (n - 2) * (n - 2))[dom[0]]
-    per_launch_bytes = fused_steps * 2.0 * cells * 4
-    achieved = per_launch_bytes / (dom[1][0] * 1e-3) / 1e9
+    per_launch_alg = fused_steps * 2.0 * cells * 4
+    fused_min = 2.0 * n * n * 4              # a fused launch cannot do with less than one read and one write of the plane
+    measured = {k: kernel_traffic(name, k) for k in prof}
+    t_dom = measured[dom[0]]
+    # whole function: counter bytes of every launch; the fused minimum stands in for a kernel the table does not know
+    call_bytes = sum((measured[k]["bytes"] if measured[k] else fused_min) * v[1] for k, v in prof.items())
+    dom_bytes = t_dom["bytes"] if t_dom else None
+    achieved = (dom_bytes if dom_bytes else fused_min) / (dom[1][0] * 1e-3) / 1e9
     out = {
-        "value": alg_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
+        "value": call_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
+        "value_basis": "HBM bytes moved per call (hardware counters per kernel x launches%s) / time per call"
+                       % ("" if all(measured.values()) else "; read-once-write-once minimum for kernels without a counter record"),
+        "algorithmic_gbs": alg_bytes / (ms * 1e-3) / 1e9,
+        "algorithmic_basis": "8 bytes per cell and time step of the un-fused program (32 x 2 x 8192^2 x 4 B = 17.18 GB per call)",
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": HEAT2D_TRAFFIC_BYTES_PER_LAUNCH.get(fused_steps),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": dom_bytes,
                      "kernel": dom[0], "kernel_ms": dom[1][0], "launches_per_step": dom[1][1],
-                     "time_steps_per_launch": fused_steps, "cells_per_launch": cells},
-        "kernels": {k: {"ms": v[0], "launches_per_step": v[1]} for k, v in prof.items()},
+                     "time_steps_per_launch": fused_steps, "cells_per_launch": cells,
+                     "algorithmic_gbs": per_launch_alg / (dom[1][0] * 1e-3) / 1e9,
+                     "fused_minimum_bytes": fused_min,
+                     "traffic_over_fused_minimum": dom_bytes / fused_min if dom_bytes else None,
+                     "vector_alu_busy": t_dom["vector_alu_busy"] if t_dom else None,
+                     "limiter": "vector ALUs (time-fused launch: the stencil arithmetic of all fused steps, not HBM, sets its duration)"
+                                if fused_steps > 1 else "hbm"},
+        "kernels": {k: {"ms": v[0], "launches_per_step": v[1], "traffic": measured[k]["bytes"] if measured[k] else None} for k, v in prof.items()},
     }
     if with_cpu:
         cpu = runtime.Program(oracle_build.cpu_program_library(PROGRAMS, name), name, needs_gpu_runtime=False)
@@ -180,7 +227,8 @@ def bench_sgemm(M, steps, warmup, with_cpu):
     out = {
         "value": flop / (ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None, "kernel": dom[0], "kernel_ms": dom[1][0]},
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": (kernel_traffic(name, dom[0]) or {}).get("bytes"),
+                     "kernel": dom[0], "kernel_ms": dom[1][0]},
     }
     if with_cpu:
         cpu = runtime.Program(oracle_build.cpu_program_library(PROGRAMS, name), name, needs_gpu_runtime=False)
@@ -228,12 +276,12 @@ def _generic_bench(name, host_arrays, flop, peak_tflops, steps, warmup, with_cpu
     ms = time_steps(lambda: prog(*args), steps, warmup)
     prof = kernel_profile(lambda: prog(*args), max(1, min(steps, 5)))
     dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
-    dom_flop = flop * dominant_flop_share / dom[1][1]   # flops of one launch of the dominant kernel
+    dom_flop = flop * dominant_flop_share / dom[1][1]   # flops of an average launch of the dominant kernel
     achieved = dom_flop / (dom[1][0] * 1e-3) / 1e12
     out = {"value": flop / (ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
            "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
-                        "frac": achieved / peak_tflops, "traffic": None, "kernel": dom[0], "kernel_ms": dom[1][0],
-                        "launches_per_step": dom[1][1]},
+                        "frac": achieved / peak_tflops, "traffic": (kernel_traffic(name, dom[0]) or {}).get("bytes"),
+                        "kernel": dom[0], "kernel_ms": dom[1][0], "launches_per_step": dom[1][1]},
            "kernels": {k: {"ms": v[0], "launches_per_step": v[1]} for k, v in prof.items()}}
     if with_cpu:
         cpu = runtime.Program(oracle_build.cpu_program_library(PROGRAMS, name), name, needs_gpu_runtime=False)
@@ -256,7 +304,8 @@ def bench_sgemm_bf16(steps, warmup, with_cpu):
     A, B = bf16(rng.uniform(-1, 1, (M, K))), bf16(rng.uniform(-1, 1, (K, N)))
     C = np.zeros((M, N), np.float32)
     return _generic_bench("sgemm_bf16_4096x4096x4096", [("host", np.array([1.0, 0.0], np.float32)), A, B, C],
-                          2.0 * M * N * K, BF16_MFMA_PEAK_TFLOPS, steps, warmup, False, "")
+                          2.0 * M * N * K, BF16_MFMA_PEAK_TFLOPS, steps, warmup, with_cpu,
+                          "parallelize i, vectorize j by 8; bf16 operands widened to fp32 on load -- the reference has no bf16 type")
 
 
 def bench_conv2d(steps, warmup, with_cpu):
@@ -312,7 +361,7 @@ def main():
     names = [n for n in WORKLOADS if n != "copy"] if a.workload == "all" else [a.workload]
     results = {}
     for n in names:
-        with_cpu = (not a.no_cpu) and (a.workload != "all" or n in ("heat2d", "sgemm1024"))
+        with_cpu = not a.no_cpu
         results[n] = WORKLOADS[n](a.steps, a.warmup, with_cpu)
     head_name = "heat2d" if "heat2d" in results else names[0]
     head = results[head_name]

@@ -91,7 +91,10 @@ void tiramisu_hip_parallel_for(int32_t first, int32_t last, void (*body)(int32_t
  *      benchmarks bracket device work with get_time() calls,
  *      benchmarks/linear_algebra/blas/level3/sgemm/gpu/generator3.cpp:66-69) ---- */
 /* Make `stream` (a hipStream_t) the calling thread's current stream; NULL restores the
- * per-thread default stream. */
+ * per-thread default stream.  Pooled memory follows the stream rule of tiramisu_hip_free: a block
+ * must be freed by a thread whose current stream is the one its last use was issued on (or after
+ * that stream has been synchronised); freeing it from a thread on another stream may hand the
+ * block out again while that work still runs. */
 int tiramisu_hip_set_stream(void *stream);
 void *tiramisu_hip_get_stream(void);
 void *tiramisu_hip_event_create(void);

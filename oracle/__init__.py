@@ -6,7 +6,6 @@ in this package.  It holds CPU restatements of what the reference computes on th
 * reference_loops.py  numpy restatements of the nested-loop references that the reference's own
                       wrapper programs compare against (tests/wrapper_test_*.cpp) and of the
                       five benchmark computations;
-* kernels.c           the same computations in plain C for sizes numpy loops cannot reach;
 * cpu_backend/        a restatement of the reference's CPU back-end (loop tags -> C + OpenMP
                       from the same isl AST), used to compile the CPU-scheduled variant of each
                       Tiramisu program: the "reference's own CPU-generated code" of the parity

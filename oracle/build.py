@@ -5,7 +5,6 @@
 * <program dir>/build/lib<name>_cpu.so -- every Tiramisu program compiled for the host: programs
   with their own CPU schedule are built with -DTIRAMISU_TARGET_CPU, the others are forced onto
   the CPU back-end with TIRAMISU_FORCE_ARCH=cpu (GPU-mapped loops then run serially).
-* oracle/liboracle_kernels.so -- plain C restatements (kernels.c).
 """
 import os
 import subprocess
@@ -17,7 +16,6 @@ from tiramisu_amd import build as product_build  # noqa: E402  (compiler library
 
 ORACLE = os.path.join(ROOT, "oracle")
 CPU_BACKEND = os.path.join(ORACLE, "cpu_backend", "libtiramisu_cpu_backend.so")
-KERNELS = os.path.join(ORACLE, "liboracle_kernels.so")
 
 
 def _run(cmd, cwd=None, env=None):
@@ -32,12 +30,6 @@ def build_cpu_backend():
     _run(["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-I" + product_build.INCLUDE, "-o", CPU_BACKEND,
           os.path.join(ORACLE, "cpu_backend", "cpu_emit.cpp"), "-L" + product_build.PKG, "-ltiramisu",
           "-Wl,-rpath," + product_build.PKG])
-
-
-def build_kernels():
-    src = os.path.join(ORACLE, "kernels.c")
-    if os.path.exists(src):
-        _run(["gcc", "-O2", "-fPIC", "-shared", "-fopenmp", "-ffp-contract=off", "-o", KERNELS, src, "-lm"])
 
 
 def cpu_program_library(directory, name):
@@ -76,7 +68,6 @@ def build_cpu_program(source):
 
 def build_all(force=True, verbose=False):
     build_cpu_backend()
-    build_kernels()
     for src in product_build.program_sources():
         if verbose:
             print("[oracle build] cpu variant of", os.path.relpath(src, ROOT), flush=True)

@@ -34,3 +34,22 @@ class DeviceArray:
             self.free()
         except Exception:
             pass
+
+
+def assert_fp32_parity(out, ref, what, rtol=1e-4, atol=None):
+    """The fp32 bar of the parity statement ("max relative error <= 1e-4"; 2e-2 for bf16 inputs), read two
+    ways, both asserted and both printed:
+      * normalised maximum norm:  max|out - ref| <= rtol * max|ref|;
+      * element by element:       |out - ref| <= rtol * |ref| + atol  with  atol = rtol * rms(ref)
+        (results are sums of many products, so an element near zero carries the rounding error of terms
+        of the typical magnitude: the absolute allowance is rtol times that magnitude)."""
+    r = np.asarray(ref, np.float64)
+    d = np.abs(np.asarray(out, np.float64) - r)
+    if atol is None:
+        atol = rtol * float(np.sqrt(np.mean(r * r)))
+    norm_err = float(d.max() / max(np.max(np.abs(r)), 1e-300))
+    worst = float(np.max(d / (rtol * np.abs(r) + atol))) if atol > 0 else (0.0 if d.max() == 0 else np.inf)
+    print("%s: max|d|/max|ref| = %.3g (bar %g); worst element |d|/(rtol*|ref|+atol) = %.3g (rtol %g, atol %.3g)"
+          % (what, norm_err, rtol, worst, rtol, atol), flush=True)
+    assert norm_err <= rtol, what
+    assert worst <= 1.0, what

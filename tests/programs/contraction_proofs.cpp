@@ -10,8 +10,11 @@
 //                            (the redirected load indexes modulo the shape) -> kept as scheduled
 //  * proofs_shared_register: two rows of a thread's register tile share
 //                            one accumulator element                       -> kept as scheduled
-// The last four compute something else than the GEMM when run as scheduled (and the shifted tile
-// reads past its operand), so they are generated and inspected, never run.
+//  * proofs_epilogue_other_element: a plain nest (global accumulator, one
+//                            thread per row) whose fused epilogue reads the
+//                            accumulator of column 0, not its own element   -> kept as scheduled
+// The four flawed tilings compute something else than the GEMM when run as scheduled (and the
+// shifted tile reads past its operand), so they are generated and inspected, never run.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -62,8 +65,32 @@ static void generate(const std::string &name, flaw what)
     tiramisu::codegen({A.get_buffer(), B.get_buffer(), C.get_buffer()}, "build/" + name + ".o", true);
 }
 
+// D(i, j) = 2 * acc(i, 0): race-free as scheduled (a thread owns row i), but the value is not the
+// one the epilogue of an MFMA tile has at hand for element (i, j).
+static void generate_epilogue_other_element(const std::string &name)
+{
+    const int M = 128, N = 64, K = 32;
+    tiramisu::init(name);
+    var i("i", 0, M), j("j", 0, N), k("k", 0, K), i0("i0"), i1("i1");
+    input A({i, k}, p_float32);
+    input B({k, j}, p_float32);
+    computation acc_init({i, j}, (float)0);
+    computation acc({i, j, k}, p_float32);
+    acc.store_in(acc_init.get_buffer(), {i, j});
+    acc.set_expression(acc(i, j, 0) + A(i, k) * B(k, j));
+    computation D({i, j}, acc(i, 0, 0) * expr((float)2));
+    for (buffer *b : {A.get_buffer(), B.get_buffer(), acc_init.get_buffer(), D.get_buffer()}) b->tag_gpu_global();
+    for (computation *c : {&acc_init, &acc, &D}) {
+        c->split(i, 64, i0, i1);
+        c->tag_gpu_level(i0, i1);
+    }
+    acc_init.then(acc, i1).then(D, i1);
+    tiramisu::codegen({A.get_buffer(), B.get_buffer(), acc_init.get_buffer(), D.get_buffer()}, "build/" + name + ".o", true);
+}
+
 int main()
 {
+    generate_epilogue_other_element("proofs_epilogue_other_element");
     generate("proofs_sound", none);
     generate("proofs_short_tile", short_tile);
     generate("proofs_shifted_tile", shifted_tile);

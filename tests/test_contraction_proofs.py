@@ -1,7 +1,8 @@
 """What the HIP back-end proves before a scheduled GEMM nest becomes its MFMA kernel
 (tests/programs/contraction_proofs.cpp): LDS tiles installed with cache_shared must hold exactly
 what the nest reads through them, and no two results of a thread may share an element of its
-register tile.  The flawed schedules stay as scheduled; they are generated, not run."""
+register tile; a fused epilogue may read the accumulator only at its own element.  The flawed
+schedules stay as scheduled; they are generated, not run."""
 import os
 import re
 
@@ -23,6 +24,7 @@ def kernel_kind(programs_dir, name):
     ("proofs_shifted_tile", "generic"),
     ("proofs_unaligned_tile", "generic"),
     ("proofs_shared_register", "generic"),
+    ("proofs_epilogue_other_element", "generic"),
 ])
 def test_kernel_chosen(programs_dir, name, kind):
     assert kernel_kind(programs_dir, name) == kind

@@ -107,7 +107,8 @@ def test_gpu_uniform_inputs_within_tolerance(s):
     out_cpu = np.zeros((s[0], s[2], s[3], s[3]), np.float32)
     cpu_program(s)(xp, w, b, out_cpu)
     out = run_gpu(s, xp, w, b)
-    assert np.max(np.abs(out - out_cpu)) <= RTOL * np.max(np.abs(out_cpu))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(out, out_cpu, "conv2d vs CPU-generated code", RTOL)
 
 
 @pytest.mark.gpu
@@ -119,6 +120,7 @@ def test_gpu_full_size():
     # the benchmark's distributions: within tolerance of the float64 restatement
     xp, w, b = make_inputs(s, 113, integer=False)
     out, exact = run_gpu(s, xp, w, b), ref.conv2d_bias_relu(xp, w, b)
-    assert np.max(np.abs(out - exact)) <= RTOL * np.max(np.abs(exact))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(out, exact, "conv2d vs float64 restatement", RTOL)
     # linearity in the input away from the clamp: conv(2x) - 2 conv(x) + bias term
     assert np.count_nonzero(out) > 0.3 * out.size

@@ -98,8 +98,9 @@ def test_gpu_matches_cpu_generated_code(s):
     y_cpu = np.zeros((s[3], s[1], s[2]), np.float32)
     cpu_program(s)(w, b, x, y_cpu)
     y = run_gpu(s, w, b, x)
-    assert np.max(np.abs(y - y_cpu)) <= RTOL * np.max(np.abs(y_cpu))
-    assert np.max(np.abs(y - ref.lstm(w, b, x))) <= RTOL * np.max(np.abs(y_cpu))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(y, y_cpu, "lstm %s vs CPU-generated code" % (s,), RTOL)
+    assert_fp32_parity(y, ref.lstm(w, b, x), "lstm %s vs numpy oracle" % (s,), RTOL)
 
 
 @pytest.mark.gpu
@@ -108,7 +109,8 @@ def test_gpu_full_size_matches_oracle():
     w, b, x = make_inputs(s, 512)
     y = run_gpu(s, w, b, x)
     expected = ref.lstm(w, b, x)
-    assert np.max(np.abs(y - expected)) <= RTOL * np.max(np.abs(expected))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(y, expected, "lstm full size vs numpy oracle", RTOL)
     # zero weights: every time step of every sample equals the closed-form recurrence
     w0 = np.zeros_like(w)
     y0 = run_gpu(s, w0, b, x)

@@ -37,6 +37,36 @@ def test_gemm_restatement_closed_forms():
     assert np.array_equal(ref.sgemm(A, B, C, 1.0, 0.0), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
 
 
+def test_strided_gemm_restatement_against_numpy_slicing():
+    """sgemm_strided (leading dimensions, element offsets, transposition as tiramisu_cublas_sgemm defines
+    them, tiramisu_cuda_wrappers.cpp:74-115) against plain numpy: the operands are cut out of larger flat
+    buffers by slicing and .T, so a swapped ld / offset / transposition rule fails.  Integer data: exact."""
+    rng = np.random.RandomState(74)
+    M, N, K = 5, 7, 6
+    for tA in (False, True):
+        for tB in (False, True):
+            ldA, ldB, ldC = (M + 3 if tA else K + 2), (K + 1 if tB else N + 4), N + 5
+            offA, offB, offC = 3, 11, 2
+            rowsA, rowsB = (K if tA else M), (N if tB else K)
+            Abuf, Bbuf = ints(rng, (offA + rowsA * ldA,)), ints(rng, (offB + rowsB * ldB,))
+            Cbuf = ints(rng, (offC + M * ldC,))
+            A2 = Abuf[offA:offA + rowsA * ldA].reshape(rowsA, ldA)[:, :(M if tA else K)]
+            B2 = Bbuf[offB:offB + rowsB * ldB].reshape(rowsB, ldB)[:, :(K if tB else N)]
+            opA, opB = (A2.T if tA else A2), (B2.T if tB else B2)
+            expected = Cbuf.copy()
+            Cview = expected[offC:offC + M * ldC].reshape(M, ldC)[:, :N]
+            Cview[...] = (3.0 * (opA.astype(np.float64) @ opB.astype(np.float64)) + 2.0 * Cview).astype(np.float32)
+            out = ref.sgemm_strided(Abuf, Bbuf, Cbuf, M, N, K, 3.0, 2.0, ldA, ldB, ldC, offA, offB, offC, tA, tB)
+            assert np.array_equal(out, expected), (tA, tB)
+    # ld == 0 means tightly packed; beta == 0 ignores what C held (NaN included)
+    A, B = ints(rng, (M, K)), ints(rng, (K, N))
+    C = np.full((M, N), np.nan, np.float32)
+    out = ref.sgemm_strided(A, B, C, M, N, K, 1.0, 0.0, 0, 0, 0, 0, 0, 0, False, False)
+    assert np.array_equal(out, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+    out = ref.sgemm_strided(A.T.copy(), B.T.copy(), C, M, N, K, 1.0, 0.0, 0, 0, 0, 0, 0, 0, True, True)
+    assert np.array_equal(out, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+
+
 # ---------------------------------------------------------------- CPU back-end vs restatements
 
 def test_cpu_gemm_gpu_tile():

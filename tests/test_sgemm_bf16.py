@@ -84,7 +84,8 @@ def test_gpu_matches_cpu_generated_code(M, N, K):
     A, B = to_bf16(rng.uniform(-1, 1, (M, K))), to_bf16(rng.uniform(-1, 1, (K, N)))
     cpu_program(M, N, K)(scal, A, B, C_cpu)
     out = run_gpu(M, N, K, scal, A, B, C)
-    assert np.max(np.abs(out - C_cpu)) <= RTOL * np.max(np.abs(C_cpu))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(out, C_cpu, "sgemm bf16 vs CPU-generated code", RTOL)
 
 
 @pytest.mark.gpu
@@ -96,7 +97,8 @@ def test_gpu_4096_sampled_rows():
     out = run_gpu(M, N, K, scal, A, B, np.zeros((M, N), np.float32))
     rows = rng.choice(M, 32, replace=False)
     exact = from_bf16(A[rows]).astype(np.float64) @ from_bf16(B).astype(np.float64)
-    assert np.max(np.abs(out[rows] - exact)) <= RTOL * np.max(np.abs(exact))
+    from gpu_util import assert_fp32_parity
+    assert_fp32_parity(out[rows], exact, "sgemm bf16 4096^3 sampled rows vs float64", RTOL)
     # integer-valued data: exact
     A, B = to_bf16(rng.randint(-3, 4, (M, K)).astype(np.float32)), to_bf16(rng.randint(-3, 4, (K, N)).astype(np.float32))
     out = run_gpu(M, N, K, scal, A, B, np.zeros((M, N), np.float32))

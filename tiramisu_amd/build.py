@@ -188,6 +188,32 @@ def build_python_programs(verbose=False):
             _run([sys.executable, os.path.join(PYTHON_PROGRAMS, f)])
 
 
+CMAKE_BUILD = os.path.join(ROOT, "build", "cmake")
+CMAKE_HIP_TESTS = ("17", "18", "19", "162", "164", "165", "166", "167", "168", "169", "170", "171", "197")
+
+
+def build_cmake(reference_tree=None, verbose=False):
+    """The same two libraries through the CMake build (CMakeLists.txt + configure.cmake at the root), into
+    build/cmake; with a Tiramisu source tree at hand also the reference's GPU tests that the build
+    registers under the `hip` label (generator and wrapper unchanged, executables build/cmake/test_<n>).
+    Returns (build directory, whether the tests were built)."""
+    import shutil
+    if shutil.which("cmake") is None:
+        raise RuntimeError("cmake is not installed")
+    with_tests = bool(reference_tree) and os.path.isdir(os.path.join(reference_tree, "tests"))
+    os.makedirs(CMAKE_BUILD, exist_ok=True)
+    cfg = ["cmake", "-S", ROOT, "-B", CMAKE_BUILD, "-DUSE_HIP=ON", "-DWITH_TESTS=" + ("ON" if with_tests else "OFF")]
+    if with_tests:
+        cfg.append("-DTIRAMISU_REFERENCE_DIR=" + reference_tree)
+    _run(cfg)
+    if verbose:
+        print("[build] cmake --build", os.path.relpath(CMAKE_BUILD, ROOT), flush=True)
+    _run(["cmake", "--build", CMAKE_BUILD, "-j8"])
+    if with_tests:
+        _run(["cmake", "--build", CMAKE_BUILD, "-j8", "--target"] + ["test_" + n for n in CMAKE_HIP_TESTS])
+    return CMAKE_BUILD, with_tests
+
+
 def build_all(force=True, verbose=False):
     build_compiler(force)
     build_wrappers(force)

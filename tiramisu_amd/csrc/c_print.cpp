@@ -66,6 +66,13 @@ static const char *math_name(op_t o) {
 std::string c_printer::element(const buffer *b, const std::vector<expr> &index) const {
     if (used_buffers) used_buffers->insert(b->get_name());
     if (is_scalar_buffer(b)) return b->get_name();
+    // indices are linearised in the 32-bit loop iterator type (the reference's, expr.h:130-143)
+    if (b->has_constant_extents()) {
+        double cnt = 1;
+        for (auto &d : b->get_dim_sizes()) cnt *= (double)lir::simplify(d).get_int_val();
+        if (cnt > 2147483647.0)
+            ERROR("buffer " + b->get_name() + " holds more than 2^31-1 elements: its 32-bit linear index would wrap", true);
+    }
     return b->get_name() + "[" + print(lir::linearize(b, index)) + "]";
 }
 

@@ -12,8 +12,11 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <fcntl.h>
 #include <fstream>
 #include <sstream>
+#include <sys/wait.h>
+#include <unistd.h>
 
 #include "util.h"
 
@@ -549,10 +552,53 @@ void collect_used_buffers(const node_ptr &root, std::set<std::string> &used) {
     });
 }
 
-int run(const std::string &cmd) {
-    if (debug_level() >= 1) std::cout << "[tiramisu-hip] " << cmd << std::endl;
-    return std::system(cmd.c_str());
+// Runs a compiler with an argument vector (no shell: paths may hold spaces, quotes or `;`).
+// The child's stderr goes to `stderr_file` when one is given.  Returns the exit status.
+int run(const std::vector<std::string> &argv, const std::string &stderr_file = "") {
+    if (debug_level() >= 1) {
+        std::cout << "[tiramisu-hip]";
+        for (auto &a : argv) std::cout << " " << a;
+        std::cout << std::endl;
+    }
+    std::vector<char *> args;
+    for (auto &a : argv) args.push_back(const_cast<char *>(a.c_str()));
+    args.push_back(nullptr);
+    const pid_t pid = fork();
+    if (pid < 0) return -1;
+    if (pid == 0) {
+        if (!stderr_file.empty()) {
+            const int fd = open(stderr_file.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
+            if (fd >= 0) { dup2(fd, 2); close(fd); }
+        }
+        execvp(args[0], args.data());
+        _exit(127);
+    }
+    int status = 0;
+    if (waitpid(pid, &status, 0) < 0) return -1;
+    return WIFEXITED(status) ? WEXITSTATUS(status) : -1;
 }
+
+// Whitespace-separated words of an option string taken from the environment.
+std::vector<std::string> words(const std::string &s) {
+    std::vector<std::string> r;
+    std::istringstream is(s);
+    for (std::string w; is >> w;) r.push_back(w);
+    return r;
+}
+
+// A path inside a double-quoted string of assembler or C source.
+std::string escaped(const std::string &s) {
+    std::string r;
+    for (char c : s) { if (c == '"' || c == '\\') r += '\\'; r += c; }
+    return r;
+}
+
+#ifndef TIRAMISU_DEFAULT_HIPCC
+#define TIRAMISU_DEFAULT_HIPCC "/opt/rocm/bin/hipcc"
+#endif
+#ifndef TIRAMISU_DEFAULT_HIP_ARCH
+#define TIRAMISU_DEFAULT_HIP_ARCH "gfx950"
+#endif
 
 std::string sanitize(const std::string &s) {
     std::string r;
@@ -651,10 +697,13 @@ public:
             const char *hipcc = std::getenv("HIPCC_PATH");
             const char *arch = std::getenv("TIRAMISU_HIP_ARCH");
             const char *flags = std::getenv("TIRAMISU_HIP_FLAGS");
-            std::string cmd = std::string(hipcc ? hipcc : "/opt/rocm/bin/hipcc") + " --genco --offload-arch=" +
-                              (arch ? arch : "gfx950") + " -std=c++17 " + (flags ? flags : "-O3") +
-                              " -Xclang -target-feature -Xclang -packed-fp32-ops -o " + hsaco + " " + hip_file + " 2>" + obj + ".hipcc.log";
-            if (run(cmd) != 0) {
+            std::vector<std::string> cmd = {hipcc ? hipcc : TIRAMISU_DEFAULT_HIPCC, "--genco",
+                                            std::string("--offload-arch=") + (arch ? arch : TIRAMISU_DEFAULT_HIP_ARCH), "-std=c++17"};
+            for (auto &w : words(flags ? flags : "-O3")) cmd.push_back(w);
+            for (const char *w : {"-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o"}) cmd.push_back(w);
+            cmd.push_back(hsaco);
+            cmd.push_back(hip_file);
+            if (run(cmd, obj + ".hipcc.log") != 0) {
                 std::ifstream log(obj + ".hipcc.log");
                 std::cerr << log.rdbuf();
                 ERROR("hipcc failed on " + hip_file, true);
@@ -674,7 +723,7 @@ public:
                 char *abs_path = realpath(hsaco.c_str(), nullptr);
                 const std::string hsaco_abs = abs_path ? abs_path : hsaco;
                 free(abs_path);
-                h << "__asm__(\".section .rodata\\n.balign 4096\\n.global " << sym << "\\n" << sym << ":\\n.incbin \\\"" << hsaco_abs
+                h << "__asm__(\".section .rodata\\n.balign 4096\\n.global " << sym << "\\n" << sym << ":\\n.incbin \\\"" << escaped(escaped(hsaco_abs))
                   << "\\\"\\n.global " << sym << "_end\\n" << sym << "_end:\\n.byte 0\\n.previous\\n\");\n";
                 h << "extern \"C\" const unsigned char " << sym << "[], " << sym << "_end[];\n";
                 h << "static void *_tiramisu_module() {\n    static void *m = tiramisu_hip_module_load((const void *)" << sym
@@ -688,7 +737,7 @@ public:
             const char *cxx = std::getenv("TIRAMISU_HOST_CXX");
             std::string inc = TIRAMISU_AMD_INCLUDE_DIR;
             if (const char *e = std::getenv("TIRAMISU_AMD_INCLUDE")) inc = e;
-            std::string cmd = std::string(cxx ? cxx : "g++") + " -std=c++17 -O2 -fPIC -I" + inc + " -c " + host_file + " -o " + obj;
+            const std::vector<std::string> cmd = {cxx ? cxx : "g++", "-std=c++17", "-O2", "-fPIC", "-I" + inc, "-c", host_file, "-o", obj};
             if (run(cmd) != 0) ERROR("host compiler failed on " + host_file, true);
         }
         // ---- manifest: what a harness needs to call the function and to know what was emitted

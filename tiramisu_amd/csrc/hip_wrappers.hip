@@ -243,7 +243,20 @@ void *tiramisu_hip_malloc(uint64_t size) {
         }
     }
     void *p = nullptr;
-    check(hipMalloc(&p, size), __FUNCTION__);
+    hipError_t e = hipMalloc(&p, size);
+    if (e == hipErrorOutOfMemory) {
+        // give the idle blocks back to HIP and try once more
+        (void)hipGetLastError();
+        {
+            std::lock_guard<std::mutex> g(pool_mutex);
+            for (auto &kv : pool_free)
+                for (void *q : kv.second) check(hipFree(q), __FUNCTION__);
+            pool_free.clear();
+            pool_idle_bytes = 0;
+        }
+        e = hipMalloc(&p, size);
+    }
+    check(e, __FUNCTION__);
     std::lock_guard<std::mutex> g(pool_mutex);
     pool_live[p] = size;
     return p;
@@ -353,6 +366,10 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
     if (ldC == 0) ldC = N;
     if (M == 0 || N == 0) return 0;
     scoped_record rec("tiramisu_hip_dgemm");
+    if (M > 0x7fffffffull || N > 0x7fffffffull || K > 0x7fffffffull) {
+        fprintf(stderr, "Error at %s: dimension exceeds 2^31-1\n", __FUNCTION__);
+        exit(1);
+    }
     dim3 blk(16, 16), grd((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
     hipLaunchKernelGGL(gemm_generic_kernel<double>, grd, blk, 0, current_stream, (const double *)(A + offsetA),
                        (const double *)(B + offsetB), C + offsetC, (int)M, (int)N, (int)K,

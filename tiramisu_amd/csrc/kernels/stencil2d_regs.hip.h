@@ -74,9 +74,10 @@ __device__ __forceinline__ float st_from_right(float v) {
 
 // Four cells of row gy starting at column gx (a multiple of 4) of a plane of NY x NX cells;
 // cells outside the plane read as 0.  With CHECK false the quad is known to be inside.
-// Element loads always use a clamped (valid) address and select afterwards.
+// Element loads always use a clamped (valid) address and select afterwards.  `plane` carries no
+// restrict qualifier: the boundary path reads the plane that the same kernel later writes.
 template <bool CHECK, int NY, int NX>
-__device__ __forceinline__ st_f4 st_load_quad(const float *__restrict__ plane, int gy, int gx) {
+__device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx) {
     st_f4 v = {0.f, 0.f, 0.f, 0.f};
     if (NX % 4 == 0) {
         if (!CHECK) return *reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx);

@@ -723,6 +723,23 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
                      (paired.empty() && !same_element(expr(o_access, acc_buf->get_name(), leaves[ii]->lhs_index, p_float32), acc_buf, ureal->lhs_index))))
         return reject(13);
     if (has_init && reads_buffer(cs[ii].leaf->rhs, acc_buf->get_name())) return reject(14);
+    // The kernel's epilogue has one value at hand per element: the finished sum of that element.  A fused
+    // statement may therefore read the accumulator and the output only at the element it belongs to (index
+    // compared in kernel variables; for a private accumulator the pairing above already ties the elements).
+    auto reads_only = [&](canon &c, const buffer *b, const std::vector<expr> &own, const std::map<std::string, expr> &own_subs) {
+        bool only = true;
+        c.leaf->rhs.visit([&](const expr &x) {
+            if (!is_load(x) || x.get_name() != b->get_name()) return;
+            if (x.get_access().size() != own.size()) { only = false; return; }
+            for (size_t d = 0; d < own.size(); d++)
+                if (!lir::simplify(x.get_access()[d].substitute(c.subs)).is_equal(lir::simplify(own[d].substitute(own_subs)))) only = false;
+        });
+        return only;
+    };
+    if (has_epi && paired.empty() && !reads_only(cs[ei], acc_buf, U.leaf->lhs_index, U.subs)) return reject(27);
+    if (has_epi && out_buf != acc_buf)
+        for (int other : {ii, ei})
+            if (other >= 0 && other < (int)leaves.size() && other != ui && !reads_only(cs[other], out_buf, cs[ei].leaf->lhs_index, cs[ei].subs)) return reject(27);
 
     // ---- extents of the three groups
     struct group_info { std::vector<int> dims; std::vector<expr> extent; bool literal = true; std::vector<long> ext; expr total; };

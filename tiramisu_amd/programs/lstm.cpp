@@ -8,20 +8,15 @@
 // structure (merged 4H gate rows, h/c buffers indexed [m+1][l+1]) is that of
 // benchmarks/DNN/blocks/LSTM/cpu/generator.cpp:31-60, and sigmoid is 1 / (1 + exp(-x)) (:43).
 //
-// The input half of the gates does not depend on the recurrence, so it is computed for a block of
-// MB time steps of a layer at once (gin = bias + W * h_below, one contraction with M = MB*B rows),
-// as the reference's library variant does (gpu_lib/generator.cpp:63-73, GEMM_BATCH = 10); the
-// recurrent half then starts from it: gates(m) = gin(m) + R * h(m-1).
-//
-// GPU schedule, after the reference's library variant (gpu_lib/generator.cpp:120-135): layers and
-// blocks of time steps are host loops, skewed and interchanged so that the outer loop walks the
-// diagonals l + m0 and the inner one, tagged parallel, the independent (layer, block) pairs of a
-// diagonal -- the runtime runs them on pool threads with a stream each, so up to L cells are in
-// flight at once.  Per pair one MFMA kernel for gin (the bias initialisation fused in, the
-// block's time steps mapped to workgroups); per cell the copy of gin and the recurrent reduction
-// are fused in one nest (a contraction with K = H), and the nine element-wise computations in a
-// second nest (one kernel).  Cell temporaries are per layer.  All tensors are GPU-resident; h is
-// laid out [layer][time][batch][hidden] so that the rows of the block-wide contraction are contiguous.
+// GPU schedule: one cell (layer l, time step m) is two loop nests -- the gates of the cell as one
+// contraction with two product terms (input weights against the layer below, recurrent weights
+// against the previous step; the bias initialisation fused in), then the nine element-wise
+// computations over (sample, hidden unit) -- and the back-end fuses the two into one MFMA kernel
+// whose workgroups hold the four gate columns of their hidden units.  Layers and time steps are host
+// loops, skewed and interchanged so that the outer loop walks the diagonals l + m and the inner one,
+// tagged parallel, the independent cells of a diagonal (the traversal of the reference's library
+// variant, gpu_lib/generator.cpp:120-135, at the granularity of single time steps): the back-end
+// runs the cells of a diagonal as one launch.  All tensors are GPU-resident.
 // CPU schedule (-DTIRAMISU_TARGET_CPU): the same computations in the reference's unscheduled order
 // (cpu/generator.cpp:59-75) with the batch loop parallelized.
 // One generated function per shape: lstm_<L>x<B>x<H>x<S>.
@@ -36,16 +31,12 @@ static void generate(int L, int B, int H, int S)
     const std::string name = "lstm_" + std::to_string(L) + "x" + std::to_string(B) + "x" + std::to_string(H) + "x" + std::to_string(S);
     tiramisu::init(name);
 
-    int MB = 1;                                   // time steps per input contraction: largest divisor of S up to 10
-    for (int d = 1; d <= 10; d++) if (S % d == 0) MB = d;
     var l("l", 0, L), m("m", 0, S), k("k", 0, B), i("i", 0, H), j("j", 0, H), g("g", 0, 4 * H);
-    var m0("m0", 0, S / MB), m1("m1", 0, MB);
 
     buffer buf_weights("buf_weights", {L, 2, 4 * H, H}, p_float32, a_input);
     buffer buf_biases("buf_biases", {L, 4 * H}, p_float32, a_input);
     buffer buf_x("buf_x", {S, B, H}, p_float32, a_input);
     buffer buf_y("buf_y", {S, B, H}, p_float32, a_output);
-    buffer buf_gin("buf_gin", {S, B, 4 * H}, p_float32, a_temporary);
     buffer buf_gates("buf_gates", {L, B, 4 * H}, p_float32, a_temporary);
     buffer buf_i("buf_i", {L, B, H}, p_float32, a_temporary);
     buffer buf_f("buf_f", {L, B, H}, p_float32, a_temporary);
@@ -64,13 +55,9 @@ static void generate(int L, int B, int H, int S)
     computation h_init("h_init", {l, k, i}, expr((float)0));
     computation c_init("c_init", {l, k, i}, expr((float)0));
     computation h_copy_x("h_copy_x", {m, k, i}, x(m, k, i));
-    computation gin_init("gin_init", {l, m0, m1, k, g}, bias(l, g));
-    computation gin("gin", {l, m0, m1, k, g, j}, p_float32);
-    gin.set_expression(gin(l, m0, m1, k, g, 0) + W(l, g, j) * h(l - 1, m0 * MB + m1, k, j));
-    input gin_at("gin_at", {m, k, g}, p_float32);   // gin of the current layer at time step m
-    computation gates_init("gates_init", {l, m, k, g}, gin_at(m, k, g));
+    computation gates_init("gates_init", {l, m, k, g}, bias(l, g));
     computation gates("gates", {l, m, k, g, j}, p_float32);
-    gates.set_expression(gates(l, m, k, g, 0) + R(l, g, j) * h(l, m - 1, k, j));
+    gates.set_expression(gates(l, m, k, g, 0) + W(l, g, j) * h(l - 1, m, k, j) + R(l, g, j) * h(l, m - 1, k, j));
     computation sig_i("sig_i", {l, m, k, i}, sigmoid(gates(l, m, k, i, 0)));
     computation sig_f("sig_f", {l, m, k, i}, sigmoid(gates(l, m, k, i + H, 0)));
     computation tnh_z("tnh_z", {l, m, k, i}, expr(o_tanh, gates(l, m, k, i + 2 * H, 0)));
@@ -87,9 +74,6 @@ static void generate(int L, int B, int H, int S)
     bias.store_in(&buf_biases, {l, g});
     x.store_in(&buf_x);
     y.store_in(&buf_y);
-    gin_init.store_in(&buf_gin, {m0 * MB + m1, k, g});
-    gin.store_in(&buf_gin, {m0 * MB + m1, k, g});
-    gin_at.store_in(&buf_gin, {m, k, g});
     gates_init.store_in(&buf_gates, {l, k, g});
     gates.store_in(&buf_gates, {l, k, g});
     sig_i.store_in(&buf_i, {l, k, i});
@@ -106,13 +90,11 @@ static void generate(int L, int B, int H, int S)
     h_copy_x.store_in(&buf_h, {0, m + 1, k, i});
 
 #ifdef TIRAMISU_TARGET_CPU
-    for (computation *q : {&gin_init, &gin, &gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
+    for (computation *q : {&gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
         q->parallelize(k);
     h_init.then(c_init, computation::root)
           .then(h_copy_x, computation::root)
-          .then(gin_init, computation::root)
-          .then(gin, l)
-          .then(gates_init, l)
+          .then(gates_init, computation::root)
           .then(gates, m)
           .then(sig_i, m)
           .then(sig_f, m)
@@ -126,37 +108,26 @@ static void generate(int L, int B, int H, int S)
           .then(y, computation::root);
     tiramisu::codegen({&buf_weights, &buf_biases, &buf_x, &buf_y}, "build/" + name + "_cpu.o", false);
 #else
-    for (buffer *q : {&buf_weights, &buf_biases, &buf_x, &buf_y, &buf_gin, &buf_gates, &buf_i, &buf_f, &buf_z, &buf_o, &buf_h, &buf_c})
+    for (buffer *q : {&buf_weights, &buf_biases, &buf_x, &buf_y, &buf_gates, &buf_i, &buf_f, &buf_z, &buf_o, &buf_h, &buf_c})
         q->tag_gpu_global();
     var kb("kb"), kt("kt"), ib("ib"), it("it"), gb("gb"), gt("gt"), ls("ls"), ms("ms");
     // fuse the initialisations, the copy of x and the output into one kernel each: layer / time innermost
     for (computation *q : {&h_init, &c_init}) { q->interchange(l, k); q->interchange(l, i); }
     for (computation *q : {&h_copy_x, &y}) { q->interchange(m, k); q->interchange(m, i); }
-    // cells in blocks of MB time steps (before the loops are mapped to the GPU: tags name loop levels)
+    // diagonal traversal of (layer, time step); the cells of a diagonal are independent
     block cells({&gates_init, &gates, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h});
-    cells.split(m, MB, m0, m1);
+    cells.skew(l, m, 1, ls, ms);
+    cells.interchange(ls, ms);
+    gates_init.parallelize(ls);
     for (computation *q : {&h_init, &c_init, &h_copy_x, &y, &sig_i, &sig_f, &tnh_z, &sig_o, &mul_iz, &mul_fc, &c, &tnh_c, &h})
         q->gpu_tile(k, i, 16, 16, kb, ib, kt, it);
-    // the block-wide contraction: loops l m0 | m1 kb gb | kt gt | j, the block's time steps and the tile loops on workgroups
-    for (computation *q : {&gin_init, &gin}) {
-        q->tile(k, g, 16, 16, kb, gb, kt, gt);
-        q->tag_gpu_block_level(2, 3, 4);
-        q->tag_gpu_thread_level(5, 6);
-    }
     gates_init.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
     gates.gpu_tile(k, g, 16, 16, kb, gb, kt, gt);
-    // diagonal traversal of (layer, block of time steps); the pairs of a diagonal run side by side
-    block wave({&gin_init, &gin, &cells});
-    wave.skew(l, m0, 1, ls, ms);
-    wave.interchange(ls, ms);
-    gin_init.parallelize(ls);
     h_init.then(c_init, computation::root)
           .then(h_copy_x, computation::root)
-          .then(gin_init, computation::root)
-          .then(gin, gt)
-          .then(gates_init, ls)
+          .then(gates_init, computation::root)
           .then(gates, gt)
-          .then(sig_i, m1)
+          .then(sig_i, ls)
           .then(sig_f, it)
           .then(tnh_z, it)
           .then(sig_o, it)
