@@ -1,5 +1,6 @@
 """Stacked LSTM (benchmark configuration 5): oracle pins, CPU-generated code vs the oracle, and the GPU
-program (MFMA gate GEMMs + fused element-wise kernel per cell) vs both.
+program (per cell one MFMA kernel: both gate products, bias and the element-wise cell update on the
+finished tile; the independent cells of a diagonal of (layer, time step) in one launch) vs both.
 
 Tolerance: max |gpu - ref| <= 1e-4 * max |ref| on the output sequence y (fp32; the MFMA kernel
 sums in a different order and the device's expf/tanhf differ from libm in the last ulps)."""
@@ -89,6 +90,20 @@ def run_gpu(s, w, b, x):
     for q in d:
         q.free()
     return out
+
+
+@pytest.mark.parametrize("s", SMALL + [(4, 64, 512, 100)])
+def test_cell_is_one_fused_kernel(s):
+    """The gate contraction takes the element-wise nest that follows it into its kernel (the four gate
+    columns of a hidden unit in one workgroup), the gate buffer and the four activation temporaries stay
+    in registers, and -- with more than one layer -- the cells of a diagonal share a launch."""
+    import json
+    kernels = json.load(open(os.path.join(PROGRAMS, "build", name_of(s) + ".o.json")))["kernels"]
+    fused = [k["how"] for k in kernels if k["how"].startswith("mfma-contraction")]
+    assert len(fused) == 1 and len(kernels) == 5          # h_init, c_init, copy of x, the cell, y
+    assert "2 product term(s), fused initialisation, 9 point-wise statement(s) of the following nest fused" in fused[0]
+    assert "4 column group(s) per unit, 5 temporaries kept in registers" in fused[0]
+    assert ("gridDim.z" in fused[0]) == (s[0] > 1)
 
 
 @pytest.mark.gpu

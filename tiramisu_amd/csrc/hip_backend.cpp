@@ -28,10 +28,10 @@ using lir::node;
 using lir::node_kind;
 using lir::node_ptr;
 
-int context::next_kernel_id() {
-    static int counter = 0;  // process-wide, like the reference's kernel_count (tiramisu_codegen_cuda.cpp:1320)
-    return counter++;
-}
+static int kernel_counter = 0;  // process-wide, like the reference's kernel_count (tiramisu_codegen_cuda.cpp:1320)
+int context::next_kernel_id() { return kernel_counter++; }
+int context::peek_next_kernel_id() { return kernel_counter; }
+void context::set_next_kernel_id(int id) { kernel_counter = id; }
 
 namespace {
 
@@ -408,7 +408,7 @@ struct host_gen {
         if (!n) return;
         switch (n->kind) {
         case node_kind::block:
-            for (auto &c : n->children) emit(c, ind);
+            emit_sequence(n->children, ind);
             break;
         case node_kind::cond:
             out << pad(ind) << "if (" << hp.print(n->condition) << ") {\n";
@@ -430,6 +430,7 @@ struct host_gen {
                     out << plan.host_code;
                     break;
                 }
+                if (runs_in_parallel(n) && emit_batched(n, ind)) break;
                 if (runs_in_parallel(n)) {
                     // iterations on pool threads, each with a stream of its own (what the reference's
                     // Halide parallel loop around kernel calls does: tiramisu_codegen_halide.cpp:2104-2145)
@@ -437,7 +438,9 @@ struct host_gen {
                     out << pad(ind) << "{\n";
                     out << pad(ind + 1) << "auto " << body << " = [&](int32_t " << n->iterator << ") {\n";
                     in_parallel_loop = true;
+                    ctx.host_iterators.push_back(n->iterator);
                     emit(n->body, ind + 2);
+                    ctx.host_iterators.pop_back();
                     in_parallel_loop = false;
                     out << pad(ind + 1) << "};\n";
                     out << pad(ind + 1) << "tiramisu_hip_parallel_for(" << hp.print(n->init) << ", " << hp.print(n->upper)
@@ -447,7 +450,9 @@ struct host_gen {
                 }
                 out << pad(ind) << "for (int32_t " << n->iterator << " = " << hp.print(n->init) << "; " << n->iterator
                     << " <= " << hp.print(n->upper) << "; " << n->iterator << " += " << hp.print(n->increment) << ") {\n";
+                ctx.host_iterators.push_back(n->iterator);
                 emit(n->body, ind + 1);
+                ctx.host_iterators.pop_back();
                 out << pad(ind) << "}\n";
             }
             break;
@@ -455,12 +460,77 @@ struct host_gen {
         }
     }
 
+    void take(launch_plan &plan, int ind) {
+        for (auto &k : plan.kernels) ctx.kernels.push_back(k);
+        if (!plan.host_code.empty()) out << plan.host_code;
+        else for (auto &k : plan.kernels) out << launch_text(k, pad(ind));
+    }
+
+    // Statements in order.  A contraction nest directly followed by another GPU-mapped nest is offered
+    // to the contraction emitter as a pair: a point-wise consumer of the result runs in the same kernel.
+    void emit_sequence(const std::vector<node_ptr> &nodes, int ind) {
+        for (size_t i = 0; i < nodes.size(); i++) {
+            if (i + 1 < nodes.size() && is_gpu_loop(nodes[i]) && is_gpu_loop(nodes[i + 1])) {
+                fusion_request req;
+                req.consumer = nodes[i + 1];
+                launch_plan plan;
+                const int first_id = context::peek_next_kernel_id();
+                if (emit_contraction(ctx, nodes[i], plan, &req)) {
+                    take(plan, ind);
+                    i++;
+                    continue;
+                }
+                context::set_next_kernel_id(first_id);
+            }
+            emit(nodes[i], ind);
+        }
+    }
+
+    // A host loop tagged parallel whose body is nothing but GPU-mapped nests that the contraction
+    // emitter takes: its iterations become gridDim.z of one launch per kernel instead of launches of
+    // their own on pool threads.  (Independence of the iterations is what the tag asserts; kernels of
+    // the body still run one after the other, each over all iterations, which keeps every dependence
+    // that the serial loop body had within an iteration.)
+    bool emit_batched(const node_ptr &n, int ind) {
+        if (std::getenv("TIRAMISU_HIP_NO_BATCHED_LAUNCH")) return false;
+        std::vector<node_ptr> nests;
+        if (n->body && n->body->kind == node_kind::block) nests = n->body->children;
+        else if (n->body) nests.push_back(n->body);
+        if (nests.empty()) return false;
+        for (auto &x : nests)
+            if (!is_gpu_loop(x)) return false;
+        const int first_id = context::peek_next_kernel_id();
+        std::vector<launch_plan> plans;
+        ctx.host_iterators.push_back(n->iterator);
+        bool ok = true;
+        for (size_t i = 0; i < nests.size() && ok; i++) {
+            fusion_request req;
+            req.batch_iterator = n->iterator;
+            req.batch_first = n->init;
+            req.batch_last = n->upper;
+            launch_plan plan;
+            if (i + 1 < nests.size()) {
+                req.consumer = nests[i + 1];
+                if (emit_contraction(ctx, nests[i], plan, &req)) { plans.push_back(plan); i++; continue; }
+                req.consumer = nullptr;
+                plan = launch_plan();
+            }
+            if (emit_contraction(ctx, nests[i], plan, &req)) plans.push_back(plan);
+            else ok = false;
+        }
+        ctx.host_iterators.pop_back();
+        if (!ok) {
+            context::set_next_kernel_id(first_id);
+            return false;
+        }
+        for (auto &p : plans) take(p, ind);
+        return true;
+    }
+
     void emit_kernel_nest(const node_ptr &n, int ind) {
         launch_plan plan;
         if (emit_contraction(ctx, n, plan) || emit_stencil(ctx, n, nullptr, plan)) {
-            for (auto &k : plan.kernels) ctx.kernels.push_back(k);
-            if (!plan.host_code.empty()) out << plan.host_code;
-            else for (auto &k : plan.kernels) out << launch_text(k, pad(ind));
+            take(plan, ind);
             return;
         }
         kernel k = emit_generic_kernel(ctx, n);

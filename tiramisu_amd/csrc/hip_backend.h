@@ -52,7 +52,26 @@ struct context {
     std::string includes;               // extra text at the top of the kernel file
     std::set<std::string> include_once;
     std::set<std::string> constant_buffers;   // buffers living in the code object's constant memory
+    std::vector<std::string> host_iterators;  // iterators of the host loops around the nest being emitted
     int next_kernel_id();
+    /** The number the next kernel gets; set_next_kernel_id() takes numbers back when an attempt
+      * that already named kernels is abandoned. */
+    static int peek_next_kernel_id();
+    static void set_next_kernel_id(int id);
+};
+
+/** What the contraction emitter may fold into its kernel beyond the nest itself.
+  *  * consumer: the GPU-mapped nest that follows the contraction in the same host loop body.  When
+  *    its statements are point-wise over (row, unit) and read the contraction's result only at the
+  *    row's own columns `unit + q * units` (q = 0, 1, ...: column groups, e.g. the four gates of a
+  *    recurrent cell), they run in the contraction kernel, on the tile that the workgroup has just
+  *    finished: columns are dealt to workgroups so that a tile holds all groups of its units.
+  *  * batch_iterator: a host loop tagged parallel around the nest; its iterations become
+  *    gridDim.z of one launch instead of launches of their own. */
+struct fusion_request {
+    lir::node_ptr consumer;
+    std::string batch_iterator;
+    expr batch_first, batch_last;
 };
 
 /** Schedule-faithful kernel: one thread per (block-iterator, thread-iterator) point, untagged
@@ -61,7 +80,7 @@ kernel emit_generic_kernel(context &ctx, const lir::node_ptr &root);
 
 /** Pattern-directed emitters.  Each returns false when the nest is not provably of its kind, in
   * which case the generic emitter is used. */
-bool emit_contraction(context &ctx, const lir::node_ptr &root, launch_plan &plan);
+bool emit_contraction(context &ctx, const lir::node_ptr &root, launch_plan &plan, const fusion_request *fuse = nullptr);
 bool emit_stencil(context &ctx, const lir::node_ptr &root, const lir::node_ptr &time_loop, launch_plan &plan);
 
 /** Text of the launch of \p k with the argument list taken from host variables of the same names. */

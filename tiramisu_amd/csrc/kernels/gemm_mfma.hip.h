@@ -59,6 +59,23 @@ struct linear_source {
     }
 };
 
+// Columns of C (rows x of the B operand) dealt to tiles in groups: the operand's XE-long x range is
+// made of column groups that lie UE apart (x = q * UE + u), and a tile of BN columns takes UB = BN / G
+// consecutive units u out of every one of the G groups -- tile position x' stands for
+//     x = (x' % BN / UB) * UE + (x' / BN) * UB + x' % UB.
+// A workgroup then owns all G columns of its units, which is what an epilogue that combines them
+// (the gates of a recurrent cell) needs.  UB must be a multiple of 4 for operands whose x is contiguous.
+template <int BN, int UB>
+__device__ __forceinline__ int regrouped_index(int x, int UE) {
+    return ((x % BN) / UB) * UE + (x / BN) * UB + (x % UB);
+}
+template <class SRC, int BN, int UB>
+struct regrouped_rows {
+    SRC src;
+    int UE;
+    __device__ __forceinline__ auto load4(int x, int k) const { return src.load4(regrouped_index<BN, UB>(x, UE), k); }
+};
+
 // One operand tile of X x BK elements (X = BM for A, BN for B).
 template <int X, int BK, int NT, bool KMAJOR, bool EDGE, int PAD>
 struct operand_tile {

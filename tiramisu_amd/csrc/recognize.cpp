@@ -529,6 +529,46 @@ bool multiple_of(const expr &e_in, long m) {
     }
 }
 
+// e as constant + sum of coefficient * variable (integers); false when e is not of that form.
+bool affine_form(const expr &e_in, std::map<std::string, long> &coef, long &constant, long scale = 1) {
+    const expr e = lir::simplify(e_in);
+    if (e.is_integer_literal()) { constant += scale * e.get_int_val(); return true; }
+    if (e.get_expr_type() == e_var) { coef[e.get_name()] += scale; return true; }
+    if (e.get_expr_type() != e_op) return false;
+    switch (e.get_op_type()) {
+    case o_add: return affine_form(e.get_operand(0), coef, constant, scale) && affine_form(e.get_operand(1), coef, constant, scale);
+    case o_sub: return affine_form(e.get_operand(0), coef, constant, scale) && affine_form(e.get_operand(1), coef, constant, -scale);
+    case o_minus: return affine_form(e.get_operand(0), coef, constant, -scale);
+    case o_cast: return affine_form(e.get_operand(0), coef, constant, scale);
+    case o_mul: {
+        long v;
+        if (literal_value(e.get_operand(0), v)) return affine_form(e.get_operand(1), coef, constant, scale * v);
+        if (literal_value(e.get_operand(1), v)) return affine_form(e.get_operand(0), coef, constant, scale * v);
+        return false;
+    }
+    default: return false;
+    }
+}
+
+// a - b is the same non-zero integer whatever the variables are
+bool differ_by_nonzero_constant(const expr &a, const expr &b) {
+    std::map<std::string, long> coef;
+    long c = 0;
+    if (!affine_form(a, coef, c, 1) || !affine_form(b, coef, c, -1)) return false;
+    for (auto &kv : coef)
+        if (kv.second != 0) return false;
+    return c != 0;
+}
+
+bool same_affine_value(const expr &a, const expr &b) {
+    std::map<std::string, long> coef;
+    long c = 0;
+    if (!affine_form(a, coef, c, 1) || !affine_form(b, coef, c, -1)) return lir::simplify(a).is_equal(lir::simplify(b));
+    for (auto &kv : coef)
+        if (kv.second != 0) return false;
+    return c == 0;
+}
+
 bool reject(int where) {
     if (std::getenv("TIRAMISU_HIP_REPORT")) std::cout << "[tiramisu-hip] contraction check " << where << " failed" << std::endl;
     return false;
@@ -536,8 +576,11 @@ bool reject(int where) {
 
 }  // namespace
 
-bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
+bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, const fusion_request *fuse) {
     if (std::getenv("TIRAMISU_NO_MFMA")) return false;
+    const bool with_consumer = fuse && fuse->consumer && !std::getenv("TIRAMISU_MFMA_NO_CONSUMER");
+    const bool batched = fuse && !fuse->batch_iterator.empty();
+    if (fuse && fuse->consumer && !with_consumer) return false;
     function *f = ctx.f;
     std::set<std::string> inner;
     std::vector<node_ptr> leaves;
@@ -837,6 +880,153 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     const expr Me = GM.total, Ne = GN.total, Ke = GK.total;
     long Ml = -1, Nl = -1, Kl = -1;
     const bool lit = literal_value(Me, Ml) && literal_value(Ne, Nl) && literal_value(Ke, Kl);
+
+    // ---- a point-wise consumer nest folded into the kernel (see fusion_request).  Its statements are
+    // written per point (row, unit) of a two-dimensional domain; the row is the contraction's M index,
+    // and the result is read only at columns unit + q * units of that row.
+    std::vector<canon> xs;               // consumer statements, in program order
+    std::vector<node_ptr> xleaves;
+    int G = 1;                           // column groups of the result
+    long UE = 0, u_lo = 0;               // units per group, first unit
+    std::vector<std::map<std::string, int>> acc_group;   // per statement: printed canonical load of the result -> group q
+    std::vector<int> row_of, unit_of;    // per statement: which of its dimensions is the row / the unit
+    if (with_consumer) {
+        if (has_epi || acc_private || Mg.size() != 1 || Ng.size() != 1 || !lit || bf16) return reject(30);
+        std::set<std::string> xinner;
+        bool xbad = false;
+        lir::walk(fuse->consumer, [&](const node_ptr &x) {
+            if (x->kind == node_kind::cond) xbad = true;
+            if (x->kind == node_kind::loop) {
+                xinner.insert(x->iterator);
+                if (x->gpu_block < 0 && x->gpu_thread < 0) xbad = true;   // one point per thread: a point's statements are the leaves in order
+            }
+            if (x->kind != node_kind::leaf) return;
+            if (x->lkind != leaf_kind::assign || x->predicate.is_defined() || !x->lets.empty() || !x->lhs) xbad = true;
+            xleaves.push_back(x);
+        });
+        if (xbad || xleaves.empty()) return reject(30);
+        xs.resize(xleaves.size());
+        for (size_t n = 0; n < xleaves.size(); n++)
+            if (!canonicalize(f, xleaves[n], xinner, xs[n])) return reject(30);
+        const canon_dim &UM = U.dims[Mg[0]], &UN = U.dims[Ng[0]];
+        long m_lo, m_hi, n_lo, n_hi;
+        if (!literal_value(UM.lo, m_lo) || !literal_value(UM.hi, m_hi) || !literal_value(UN.lo, n_lo) || !literal_value(UN.hi, n_hi)) return reject(30);
+        // host value of an index expression of statement c: dimensions outside the kernel by their value in
+        // terms of the host loops, dimensions inside renamed per side so that they never cancel
+        auto host_view = [&](const canon &c, const expr &e, const std::string &side) {
+            std::map<std::string, expr> m;
+            for (auto &d : c.dims) {
+                if (!d.lo.is_defined()) continue;
+                if (d.in_kernel) m[d.cvar] = var(side + d.cvar);
+                else m[d.cvar] = c.real->iterators.at(d.name);
+            }
+            return lir::simplify(e.substitute(m));
+        };
+        // a dimension in which the two elements always differ by a non-zero constant
+        auto always_apart = [&](const canon &a, const std::vector<expr> &ia, const canon &b, const std::vector<expr> &ib) {
+            if (ia.size() != ib.size()) return false;
+            for (size_t d = 0; d < ia.size(); d++) {
+                if (differ_by_nonzero_constant(host_view(a, ia[d], "_a_"), host_view(b, ib[d], "_b_"))) return true;
+            }
+            return false;
+        };
+        // roles of the two dimensions, from the first statement that reads the result
+        expr Er, Eu;   // row / unit as expressions of the consumer nest's loop iterators
+        row_of.assign(xs.size(), -1);
+        unit_of.assign(xs.size(), -1);
+        auto in_kernel_dims = [&](const canon &c) {
+            std::vector<int> r;
+            for (size_t p = 0; p < c.dims.size(); p++)
+                if (c.dims[p].in_kernel && c.dims[p].lo.is_defined()) r.push_back((int)p);
+            return r;
+        };
+        // matches a load of the result in statement c: row dimension, unit dimension and column offset
+        auto match_result_load = [&](const canon &c, const expr &ld, int &pr, int &pu, long &off) {
+            if (ld.get_access().size() != U.leaf->lhs_index.size()) return false;
+            pr = pu = -1;
+            off = 0;
+            for (size_t d = 0; d < U.leaf->lhs_index.size(); d++) {
+                const expr ui = lir::simplify(U.leaf->lhs_index[d]), xi = lir::simplify(ld.get_access()[d]);
+                const bool in_m = lir::mentions(ui, UM.cvar), in_n = lir::mentions(ui, UN.cvar);
+                if (in_m || in_n) {
+                    if (ui.get_expr_type() != e_var) return false;           // the result's index is the bare dimension
+                    bool found = false;
+                    for (int p : in_kernel_dims(c)) {
+                        long o;
+                        if (!var_plus_const(xi, c.dims[p].cvar, o)) continue;
+                        if (in_m) { if (o != 0) return false; pr = p; } else { pu = p; off = o; }
+                        found = true;
+                    }
+                    if (!found) return false;
+                } else {
+                    for (int p : in_kernel_dims(c)) if (lir::mentions(xi, c.dims[p].cvar)) return false;
+                    if (!same_affine_value(host_view(U, ui, "_a_"), host_view(c, xi, "_b_"))) return false;
+                }
+            }
+            return pr >= 0 && pu >= 0 && pr != pu;
+        };
+        for (size_t n = 0; n < xs.size() && !Er.is_defined(); n++) {
+            expr first;
+            xs[n].leaf->rhs.visit([&](const expr &x) { if (!first.is_defined() && is_load(x) && x.get_name() == acc_buf->get_name()) first = x; });
+            if (!first.is_defined()) continue;
+            int pr, pu;
+            long off;
+            if (!match_result_load(xs[n], first, pr, pu, off)) return reject(31);
+            Er = lir::simplify(xleaves[n]->iterators.at(xs[n].dims[pr].name));
+            Eu = lir::simplify(xleaves[n]->iterators.at(xs[n].dims[pu].name));
+            long lo, hi;
+            if (!literal_value(xs[n].dims[pu].lo, lo) || !literal_value(xs[n].dims[pu].hi, hi)) return reject(31);
+            u_lo = lo;
+            UE = hi - lo + 1;
+        }
+        if (!Er.is_defined() || UE <= 0 || (n_hi - n_lo + 1) % UE != 0) return reject(31);
+        G = (int)((n_hi - n_lo + 1) / UE);
+        acc_group.resize(xs.size());
+        for (size_t n = 0; n < xs.size(); n++) {
+            canon &X = xs[n];
+            const std::vector<int> ik = in_kernel_dims(X);
+            if (ik.size() != 2) return reject(32);
+            for (int p : ik) {
+                const expr e = lir::simplify(xleaves[n]->iterators.at(X.dims[p].name));
+                long lo, hi;
+                if (!literal_value(X.dims[p].lo, lo) || !literal_value(X.dims[p].hi, hi)) return reject(32);
+                if (e.is_equal(Er) && lo == m_lo && hi == m_hi) row_of[n] = p;
+                else if (e.is_equal(Eu) && lo == u_lo && hi - lo + 1 == UE) unit_of[n] = p;
+                else return reject(32);
+            }
+            if (row_of[n] < 0 || unit_of[n] < 0) return reject(32);
+            // the result is read only at (own row, own unit + q * units)
+            bool okx = true;
+            X.leaf->rhs.visit([&](const expr &x) {
+                if (!is_load(x) || x.get_name() != acc_buf->get_name()) return;
+                int pr, pu;
+                long off;
+                if (!match_result_load(X, x, pr, pu, off) || pr != row_of[n] || pu != unit_of[n]) { okx = false; return; }
+                const long shifted = off + u_lo - n_lo;
+                if (shifted < 0 || shifted % UE != 0 || shifted / UE >= G) { okx = false; return; }
+                acc_group[n][x.to_str()] = (int)(shifted / UE);
+            });
+            if (!okx) return reject(33);
+            // it may not write what the contraction reads or writes in the same launch ...
+            if (X.leaf->lhs == acc_buf || X.leaf->lhs == out_buf) return reject(34);
+            auto clashes = [&](const canon &reader, const expr &e) {
+                bool clash = false;
+                e.visit([&](const expr &x) {
+                    if (is_load(x) && x.get_name() == X.leaf->lhs->get_name() && !always_apart(X, X.leaf->lhs_index, reader, x.get_access())) clash = true;
+                });
+                return clash;
+            };
+            for (auto &pr : products)
+                if (clashes(U, pr.first) || clashes(U, pr.second)) return reject(34);
+            if (has_init && clashes(cs[ii], cs[ii].leaf->rhs)) return reject(34);
+            // ... and what it reads of the consumer's own buffers is either the element this point wrote
+            // (same index text as the point's latest store, checked when the statements are printed) or an
+            // element that no point of the launch writes
+            X.subs[X.dims[row_of[n]].cvar] = var(UM.kvar);
+            X.subs[X.dims[unit_of[n]].cvar] = var("_u");
+            name_outer_dims(X);
+        }
+    }
     int BM = 64, BN = 64, BK = 16, PADX = 1, WGM = 2, WGN = 2, WGK = 1, DEPTH = 1;
     if (lit) {
         if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
@@ -907,6 +1097,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
             if (g->linear && !multiple_of(g->base, 4)) edge = true;
         }
 
+    // a consumer needs tiles that hold all column groups of their units
+    int UB = 0;
+    if (with_consumer) {
+        UB = BN / G;
+        if (BN % G != 0 || UB == 0 || UE % UB != 0 || Nl % BN != 0) return reject(35);
+        for (auto &o : operands)
+            if (!o.second.linear || (!o.second.kmajor && UB % 4 != 0)) return reject(35);
+    }
+
     // ---- kernel text
     c_printer dev;
     dev.fct = f;
@@ -914,9 +1113,122 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     std::set<std::string> used_buffers, used_scalars;
     dev.used_buffers = &used_buffers;
     dev.used_scalars = &used_scalars;
-    std::set<std::string> locals = {"_accv", "_sum", "_r", "_c", "_x", "_k"};
+    std::set<std::string> locals = {"_accv", "_sum", "_r", "_c", "_x", "_k", "_u", "_cq"};
     for (int p : spatial) locals.insert(U.dims[p].kvar);
     for (int p : reduction) locals.insert(U.dims[p].kvar);
+    if (batched) locals.insert(fuse->batch_iterator);
+
+    // ---- the consumer's statements, once per point of the tile.  A value that the point itself stored
+    // earlier is taken from its register instead of memory; a temporary of the function that nothing else
+    // in the program reads is then not stored at all.
+    std::ostringstream consumer_text;
+    std::set<std::string> dead;                 // buffers whose stores are dropped
+    if (with_consumer) {
+        struct stmt { const buffer *lhs; std::vector<expr> idx; std::string value, decl; primitive_t type; };
+        std::vector<stmt> stmts;
+        std::set<std::string> loaded;           // buffers that some statement still loads from memory
+        std::map<std::string, std::pair<std::string, std::string>> latest;   // buffer -> (index text, value) of the point's latest store
+        c_printer plain;
+        plain.fct = f;
+        plain.device = true;
+        std::set<int> groups_used;
+        // an element as a text that is the same for every statement of a point: row and unit by their role,
+        // outer dimensions by their value in terms of the host loops
+        auto element_key = [&](size_t n, const buffer *b, const std::vector<expr> &index) {
+            std::map<std::string, expr> m;
+            for (size_t p = 0; p < xs[n].dims.size(); p++) {
+                const canon_dim &d = xs[n].dims[p];
+                if (!d.lo.is_defined()) continue;
+                m[d.cvar] = (int)p == row_of[n] ? expr(var("_row")) : (int)p == unit_of[n] ? expr(var("_unit")) : xs[n].real->iterators.at(d.name);
+            }
+            std::vector<expr> v;
+            for (auto &e : index) v.push_back(lir::simplify(e.substitute(m)));
+            return b->get_name() + "[" + plain.print(lir::simplify(lir::linearize(b, v))) + "]";
+        };
+        // the element that statement w stores and the one statement n loads always differ by a non-zero
+        // constant in some dimension (row and unit of the two points taken as unrelated)
+        auto never_the_same = [&](size_t w, size_t n, const std::vector<expr> &loaded_index) {
+            const std::vector<expr> &ia = xs[w].leaf->lhs_index;
+            std::map<std::string, expr> ma, mb;
+            for (auto &dd : xs[w].dims) if (dd.lo.is_defined()) ma[dd.cvar] = dd.in_kernel ? expr(var("_a_" + dd.cvar)) : xs[w].real->iterators.at(dd.name);
+            for (auto &dd : xs[n].dims) if (dd.lo.is_defined()) mb[dd.cvar] = dd.in_kernel ? expr(var("_b_" + dd.cvar)) : xs[n].real->iterators.at(dd.name);
+            for (size_t d = 0; d < ia.size() && d < loaded_index.size(); d++)
+                if (differ_by_nonzero_constant(ia[d].substitute(ma), loaded_index[d].substitute(mb))) return true;
+            return false;
+        };
+        for (size_t n = 0; n < xs.size(); n++) {
+            canon &X = xs[n];
+            bool okx = true;
+            // on the canonical form: the result comes from the tile, a value the point stored earlier from its
+            // register; any other load of a buffer that the consumer writes must be of an element that no
+            // point of the launch stores
+            expr val = X.leaf->rhs.transform([&](const expr &x) -> expr {
+                if (!is_load(x)) return x;
+                if (x.get_name() == acc_buf->get_name()) {
+                    const int q = acc_group[n].at(x.to_str());
+                    groups_used.insert(q);
+                    return var(p_float32, "_g" + std::to_string(q));
+                }
+                const buffer *b = f->get_buffers().at(x.get_name());
+                auto it = latest.find(x.get_name());
+                const std::string key = element_key(n, b, x.get_access());
+                if (it != latest.end() && it->second.first == key) return var(x.get_data_type(), it->second.second);
+                for (size_t w = 0; w < xs.size(); w++) {
+                    if (xs[w].leaf->lhs != b) continue;
+                    if (element_key(w, b, xs[w].leaf->lhs_index) == key) continue;   // the point's own element, read from memory
+                    if (!never_the_same(w, n, x.get_access())) okx = false;
+                }
+                loaded.insert(x.get_name());
+                return x;
+            }).substitute(X.subs);
+            if (!okx) return reject(36);
+            stmt st;
+            st.lhs = X.leaf->lhs;
+            for (auto &e : X.leaf->lhs_index) st.idx.push_back(e.substitute(X.subs));
+            st.value = "_v" + std::to_string(n);
+            st.type = val.get_data_type();
+            st.decl = "const " + primitive_c_name(st.type) + " " + st.value + " = " + dev.print(val) + ";";
+            locals.insert(st.value);
+            latest[st.lhs->get_name()] = {element_key(n, st.lhs, X.leaf->lhs_index), st.value};
+            stmts.push_back(st);
+        }
+        // a temporary that only this kernel touches and never loads back from memory is not stored
+        auto only_used_here = [&](const buffer *b) {
+            if (b->get_argument_type() != a_temporary || !b->get_auto_allocate()) return false;
+            for (auto *a : f->get_arguments()) if (a == b) return false;
+            bool elsewhere = false;
+            lir::walk(ctx.prog->root, [&](const node_ptr &x) {
+                if (x->kind != node_kind::leaf) return;
+                for (auto &l : leaves) if (l == x) return;
+                for (auto &l : xleaves) if (l == x) return;
+                if (x->lhs == b || x->copy_from == b || x->copy_to == b || x->target == b) { elsewhere = true; return; }
+                for (const expr *e : {&x->rhs, &x->predicate})
+                    if (e->is_defined() && reads_buffer(*e, b->get_name())) elsewhere = true;
+                for (auto &l : x->lets) if (reads_buffer(l.second, b->get_name())) elsewhere = true;
+                for (auto &ix : x->lhs_index) if (reads_buffer(ix, b->get_name())) elsewhere = true;
+            });
+            for (auto &inv : ctx.prog->invariants) if (reads_buffer(inv.value, b->get_name())) elsewhere = true;
+            return !elsewhere;
+        };
+        for (auto &st : stmts)
+            if (!loaded.count(st.lhs->get_name()) && only_used_here(st.lhs)) dead.insert(st.lhs->get_name());
+        if (only_used_here(acc_buf)) dead.insert(acc_buf->get_name());
+        const std::string m_var = U.dims[Mg[0]].kvar;
+        consumer_text << "    __syncthreads();\n";
+        consumer_text << "    for (int _p = threadIdx.x; _p < CFG::BM * " << UB << "; _p += CFG::NT) {\n";
+        consumer_text << "        const int _lr = _p / " << UB << ", _lu = _p % " << UB << ";\n";
+        if (edge) consumer_text << "        if (_tm * CFG::BM + _lr >= _M) continue;\n";
+        consumer_text << "        const int32_t " << m_var << " = _tm * CFG::BM + _lr + (" << dev.print(U.dims[Mg[0]].lo.substitute(U.subs)) << ");\n";
+        consumer_text << "        const int32_t _u = _tn * " << UB << " + _lu + (" << u_lo << ");\n";
+        for (int q : groups_used)
+            consumer_text << "        const float _g" << q << " = _gt[_lr * (CFG::BN + 1) + " << q * UB << " + _lu];\n";
+        for (auto &st : stmts) {
+            consumer_text << "        " << st.decl << "\n";
+            if (!dead.count(st.lhs->get_name())) consumer_text << "        " << dev.store(st.lhs, st.idx, st.value, st.type) << "\n";
+        }
+        consumer_text << "    }\n";
+        for (int q = 0; q < G; q++) locals.insert("_g" + std::to_string(q));
+    }
     auto replace_acc = [&](const expr &e) {
         return e.transform([&](const expr &x) -> expr {
             if (is_load(x) && x.get_name() == acc_buf->get_name()) return var(p_float32, "_accv");
@@ -1027,12 +1339,25 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
             }
             which++;
         }
-        body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _B, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+        if (with_consumer) {
+            body << "        const tgemm::regrouped_rows<decltype(_B), CFG::BN, " << UB << "> _Bq{_B, " << UE << "};\n";
+            body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _Bq, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+        } else {
+            body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _B, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+        }
         term++;
     }
+    if (with_consumer)   // the finished tile, handed to the consumer's statements through LDS (behind the operand stages)
+        body << "    float *_gt = _lds + CFG::LDS_BYTES / 4 + " << ktab_words << ";\n";
     if (WGK > 1) body << "    if (tgemm::tile_reduce_k<CFG>(_acc, _lds))\n";
     body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, [&](int _r, int _c, float _sum) {\n";
-    body << digits(GM, "_r", "        ", true) << digits(GN, "_c", "        ", true);
+    if (with_consumer) {
+        body << digits(GM, "_r", "        ", true);
+        body << "        const int _cq = tgemm::regrouped_index<CFG::BN, " << UB << ">(_c, " << UE << ");\n";
+        body << digits(GN, "_cq", "        ", true);
+    } else {
+        body << digits(GM, "_r", "        ", true) << digits(GN, "_c", "        ", true);
+    }
     std::vector<expr> acc_index;
     for (auto &e : U.leaf->lhs_index) acc_index.push_back(e.substitute(U.subs));
     if (has_init) {
@@ -1043,8 +1368,10 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     } else {
         body << "        float _accv = " << dev.element(acc_buf, acc_index) << " + _sum;\n";
     }
-    if (!acc_private && !(has_epi && cs[ei].leaf->lhs == acc_buf && same_element(expr(o_access, acc_buf->get_name(), leaves[ei]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
+    if (!acc_private && !dead.count(acc_buf->get_name()) &&
+        !(has_epi && cs[ei].leaf->lhs == acc_buf && same_element(expr(o_access, acc_buf->get_name(), leaves[ei]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
         body << "        " << dev.store(acc_buf, acc_index, "_accv", p_float32) << "\n";
+    if (with_consumer) body << "        _gt[(_r - _tm * CFG::BM) * (CFG::BN + 1) + (_c - _tn * CFG::BN)] = _accv;\n";
     if (has_epi) {
         canon &E = cs[ei];
         std::vector<expr> ix;
@@ -1053,6 +1380,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         body << "        " << dev.store(E.leaf->lhs, ix, dev.print(val), val.get_data_type()) << "\n";
     }
     body << "    });\n";
+    body << consumer_text.str();
 
     kernel k;
     k.name = kname;
@@ -1061,17 +1389,35 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
     k.how = std::string("mfma-contraction: ") + (bf16 ? (BM >= 128 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
             std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
             std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
-            std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "");
+            std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "") +
+            (with_consumer ? ", " + std::to_string(xs.size()) + " point-wise statement(s) of the following nest fused (" + std::to_string(G) + " column group(s) per unit, " +
+                                 std::to_string(dead.size()) + " temporaries kept in registers)" : "") +
+            (batched ? ", iterations of the parallel host loop as gridDim.z" : "");
     std::ostringstream host;
     host << "    {\n";
+    // With a batched launch the values of the outer dimensions depend on blockIdx.z: they are computed
+    // in the kernel from the iterators of the enclosing host loops, which become its parameters.
+    std::ostringstream batch_prologue;
+    if (batched) {
+        batch_prologue << "    const int32_t " << fuse->batch_iterator << " = (int32_t)blockIdx.z + _batch_first;\n";
+        std::set<std::string> declared;
+        for (auto &o : outers)
+            if (used_scalars.count(o.name) && declared.insert(o.name).second) {
+                batch_prologue << "    const int32_t " << o.name << " = " << dev.print(o.host_value) << ";\n";
+                locals.insert(o.name);
+            }
+        used_scalars.insert("_batch_first");
+    }
     for (auto &nm : used_scalars) {
         if (locals.count(nm)) continue;
         primitive_t t = p_int32;
-        bool known = false;
+        bool known = nm == "_batch_first";
         for (auto &o : outers)
             if (o.name == nm) known = true;
         for (auto c : f->get_invariants())
             if (c->get_name() == nm) { t = c->get_data_type(); known = true; }
+        for (auto &it : ctx.host_iterators)
+            if (batched && it == nm) known = true;
         if (!known) return reject(21);
         k.params.push_back({false, nm, t});
     }
@@ -1079,8 +1425,12 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         c_printer hp;
         hp.fct = f;
         std::set<std::string> declared;
+        if (batched) {
+            host << "        const int32_t _batch_first = " << hp.print(fuse->batch_first) << ";\n";
+            k.grid[2] = "((" + hp.print(fuse->batch_last) + ") >= _batch_first ? (" + hp.print(fuse->batch_last) + ") - _batch_first + 1 : 0)";
+        }
         for (auto &o : outers)
-            if (used_scalars.count(o.name) && declared.insert(o.name).second)
+            if (!batched && used_scalars.count(o.name) && declared.insert(o.name).second)
                 host << "        const int32_t " << o.name << " = " << hp.print(o.host_value) << ";\n";
         // grid: number of tiles (outer parameters are in scope here)
         k.grid[0] = "((" + hp.print(Me) + " + " + std::to_string(BM - 1) + ") / " + std::to_string(BM) + ") * ((" + hp.print(Ne) + " + " +
@@ -1099,6 +1449,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4);
         if (bf16) k.lds_bytes = std::to_string((BM >= 128 ? 4 : 2) * (BK / 8) * (BM + BN) * 4 * 4);   // four-stage ring for the large tiles
         else if (ktab_words) k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4 + ktab_words * 4);
+        if (with_consumer) k.lds_bytes = std::to_string(std::stol(k.lds_bytes) + BM * (BN + 1) * 4);
     }
     std::ostringstream src;
     src << pre.str();
@@ -1109,7 +1460,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan) {
         if (p.is_buffer) src << primitive_c_name(p.type) << " *__restrict__ " << p.name;
         else src << "const " << primitive_c_name(p.type) << " " << p.name;
     }
-    src << ")\n{\n" << body.str() << "}\n";
+    src << ")\n{\n" << batch_prologue.str() << body.str() << "}\n";
     k.source = src.str();
     add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma.hip.h\"");
     if (bf16) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_bf16.hip.h\"");
