@@ -201,7 +201,8 @@ def bench_heat2d(steps, warmup, with_cpu):
         sec, runs = cpu_time(lambda: cpu(host))
         out["cpu_baseline"] = {"value": alg_bytes / sec / 1e9, "unit": "GB/s", "cores": cpu_threads(), "kind": "port",
                                "sample": "whole workload (8192x8192, 32 steps), median of %d runs of the CPU-generated "
-                                         "code (parallelize y, vectorize x by 8; g++ -O2 -mavx, OpenMP)" % runs}
+                                         "code (parallelize y, vectorize x by 8; g++ -O2 -mavx, OpenMP); bytes = 8 per cell and "
+                                         "time step, which is what the un-fused CPU code moves" % runs}
     dev.free()
     return out
 
@@ -378,6 +379,7 @@ def main():
                                 "lstm": "4-layer LSTM B64 H512 S100 (benchmark configs[4])"}.get(head_name, head_name)},
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
+        **{k: head[k] for k in ("value_basis", "algorithmic_gbs", "algorithmic_basis") if k in head},
         "workloads": {k: v for k, v in results.items() if k != head_name},
     }
     print(json.dumps(line))

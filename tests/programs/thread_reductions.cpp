@@ -1,0 +1,79 @@
+// Sums whose reduction loop is mapped to GPU threads.  In the reference such a schedule is a data
+// race: every thread of the loop does a read-modify-write of the same element (its CUDA printer
+// emits the statement as it stands, src/tiramisu_codegen_cuda.cpp:549-707).  The HIP back-end lowers
+// it to what the schedule means on a wave64 machine: a private partial sum per thread, a sum across
+// the lanes with DPP row shifts and row broadcasts (across wavefronts through LDS when the loop is
+// wider than one wavefront) and a single update of the element.
+//  * gemv_wavefront        y(i) = sum_j A(i,j) x(j), 300 x 1000: four rows per workgroup, the 64 lanes
+//                          of a wavefront share a row (ragged: 1000 = 15 x 64 + 40);
+//  * row_sums_quarter_wave s(i) = 1 + sum_j A(i,j), 128 x 50: 16 lanes per row, four rows per wavefront;
+//  * row_sums_block        s(i) = sum_j A(i,j), 40 x 5000: 256 threads (four wavefronts) per row.
+#include <tiramisu/tiramisu.h>
+
+using namespace tiramisu;
+
+static void gemv_wavefront()
+{
+    const int M = 300, N = 1000;
+    tiramisu::init("gemv_wavefront");
+    var i("i", 0, M), j("j", 0, N), i0("i0"), i1("i1"), j0("j0"), j1("j1");
+    input A("A", {i, j}, p_float32);
+    input x("x", {j}, p_float32);
+    computation y_init("y_init", {i}, expr((float)0));
+    computation y("y", {i, j}, p_float32);
+    y.store_in(y_init.get_buffer(), {i});
+    y.set_expression(y(i, 0) + A(i, j) * x(j));
+    y.split(j, 64, j0, j1);
+    y.interchange(j0, j1);
+    y.split(i, 4, i0, i1);
+    y_init.split(i, 4, i0, i1);
+#ifndef TIRAMISU_TARGET_CPU
+    for (buffer *b : {A.get_buffer(), x.get_buffer(), y_init.get_buffer()}) b->tag_gpu_global();
+    y.tag_gpu_block_level(0);
+    y.tag_gpu_thread_level(1, 2);            // loops: i0 | i1 j1 | j0
+    y_init.tag_gpu_block_level(0);
+    y_init.tag_gpu_thread_level(1);
+#endif
+    y_init.then(y, i1);
+#ifdef TIRAMISU_TARGET_CPU
+    tiramisu::codegen({A.get_buffer(), x.get_buffer(), y_init.get_buffer()}, "build/gemv_wavefront_cpu.o", false);
+#else
+    tiramisu::codegen({A.get_buffer(), x.get_buffer(), y_init.get_buffer()}, "build/gemv_wavefront.o", true);
+#endif
+}
+
+static void row_sums(const std::string &name, int M, int N, int rows_per_block, int lanes)
+{
+    tiramisu::init(name);
+    var i("i", 0, M), j("j", 0, N), i0("i0"), i1("i1"), j0("j0"), j1("j1");
+    input A("A", {i, j}, p_float32);
+    computation s_init("s_init", {i}, expr((float)(rows_per_block > 1 ? 1 : 0)));
+    computation s("s", {i, j}, p_float32);
+    s.store_in(s_init.get_buffer(), {i});
+    s.set_expression(A(i, j) + s(i, 0));     // the element on the right of the sum
+    s.split(j, lanes, j0, j1);
+    s.interchange(j0, j1);
+    s.split(i, rows_per_block, i0, i1);
+    s_init.split(i, rows_per_block, i0, i1);
+#ifndef TIRAMISU_TARGET_CPU
+    for (buffer *b : {A.get_buffer(), s_init.get_buffer()}) b->tag_gpu_global();
+    s.tag_gpu_block_level(0);
+    s.tag_gpu_thread_level(1, 2);
+    s_init.tag_gpu_block_level(0);
+    s_init.tag_gpu_thread_level(1);
+#endif
+    s_init.then(s, i1);
+#ifdef TIRAMISU_TARGET_CPU
+    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/" + name + "_cpu.o", false);
+#else
+    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/" + name + ".o", true);
+#endif
+}
+
+int main()
+{
+    gemv_wavefront();
+    row_sums("row_sums_quarter_wave", 128, 50, 16, 16);
+    row_sums("row_sums_block", 40, 5000, 1, 256);
+    return 0;
+}

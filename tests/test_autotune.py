@@ -1,6 +1,7 @@
-"""Host-side pieces of tiramisu_amd.autotune (knob combinations, argument construction from the
-back-end's description of a function) and of the argument check in runtime.Program.  Timing runs
-need a GPU and a code-generation pass per variant, so they are not part of the test suite."""
+"""tiramisu_amd.autotune: knob combinations, argument construction from the back-end's description of
+a function, the argument check in runtime.Program, and evaluation by execution -- two candidates of one
+program are generated ahead of time (no GPU needed: the generator calls hipcc), then timed on the GPU
+through evaluate_by_execution, which must give equal results and a positive time for each."""
 import json
 import os
 
@@ -53,3 +54,44 @@ def test_arguments_are_checked_before_the_call(product_programs_dir):
         p.check([scal, dev((1024, 1024), np.float64), dev((1024, 1024)), dev((1024, 1024))])
     with pytest.raises(ValueError, match="device memory"):
         p.check([scal, runtime.Buffer.from_numpy(np.zeros((1024, 1024), np.float32)), dev((1024, 1024)), dev((1024, 1024))])
+
+
+# ---------------------------------------------------------------- evaluation by execution
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+EVAL_DIR = os.path.join(ROOT, "tests", "programs", "build", "evaluate_by_execution")
+CANDIDATES = [{"TIRAMISU_MFMA_BK": "16"}, {"TIRAMISU_MFMA_BK": "32"}]
+
+
+def evaluator():
+    return autotune.evaluate_by_execution(os.path.join(ROOT, "tests", "programs", "gemm_gpu_tile.cpp"), "gemm_gpu_tile", EVAL_DIR, repeat=10)
+
+
+def test_candidates_are_prepared_without_a_gpu():
+    ev = evaluator()
+    for c in CANDIDATES:
+        lib = ev.prepare(c)
+        assert os.path.exists(lib)
+        slices = "x%s," % c["TIRAMISU_MFMA_BK"]
+        assert any(slices in k["how"] for k in runtime.manifest_of(lib, "gemm_gpu_tile")["kernels"])   # the knob reached the emitter
+
+
+@pytest.mark.gpu
+def test_evaluate_by_execution_times_candidates_on_the_gpu():
+    ev = evaluator()
+    outputs, times = [], []
+    for c in CANDIDATES:
+        if not os.path.exists(ev.library(c)):
+            pytest.skip("candidates were not prepared (run the CPU test suite or __graft_entry__.build() first)")
+        print("evaluating", c, flush=True)
+        samples = ev.get_measurements(c, repeat=10)
+        assert len(samples) == 10 and all(t > 0 for t in samples)
+        times.append(ev.evaluate(c))
+        outputs.append(ev.last_outputs)
+        assert ev.last_kernels[0].startswith("mfma-contraction")
+    assert all(t > 0 for t in times)
+    assert all(np.array_equal(a, b) for a, b in zip(outputs[0], outputs[1]))
+    # the result is the program's: C += A x B on the harness's seeded integer inputs
+    m = runtime.manifest_of(ev.library(CANDIDATES[0]), "gemm_gpu_tile")
+    A, B, C = autotune.make_arguments(m, ev.seed)
+    assert np.array_equal(outputs[0][0], C + A @ B)

@@ -15,7 +15,7 @@ from tiramisu_amd import runtime
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
-SMALL = [(2, 8, 32, 5), (1, 4, 16, 3), (3, 20, 64, 4)]
+SMALL = [(2, 8, 32, 5), (1, 4, 16, 3), (3, 20, 64, 4), (2, 64, 256, 6)]
 RTOL = 1e-4
 
 

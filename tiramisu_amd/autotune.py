@@ -82,30 +82,79 @@ def make_arguments(manifest, seed):
     return args
 
 
-def run_variant(lib, function, manifest, repeat, seed):
-    program = runtime.Program(lib, function)
-    args = make_arguments(manifest, seed)
+class evaluate_by_execution:
+    """Evaluation of a candidate by running it on the GPU: the counterpart of the reference's
+    tiramisu::auto_scheduler::evaluate_by_execution (include/tiramisu/auto_scheduler/evaluator.h,
+    src/auto_scheduler/tiramisu_evaluator.cpp:14-72 -- apply the candidate's optimisations, compile the
+    program to an object, turn it into a shared library, run it, return the time).  A candidate here is
+    a setting of the back-end's code-generation knobs ({name: value}, environment variables that the
+    emitters read) instead of a syntax tree of schedule transformations; `evaluate` returns the median
+    time of one call in milliseconds (HIP events on the calling stream), `get_measurements` every
+    sample, as the reference's method of the same name does (:74-125).
 
-    def call():
-        program(*[runtime.Buffer.from_device(a.ptr, a.host.shape, a.host.dtype) if isinstance(a, DeviceBuffer) else a for a in args])
-    call()
-    outputs = [(a.download() if isinstance(a, DeviceBuffer) else a.copy())
-               for a, m in zip(args, manifest["arguments"]) if m["kind"] == "output"]
-    for _ in range(max(3, repeat // 2)):
+    `prepare` does the part that needs no GPU (run the generator under the candidate's knobs, which
+    calls hipcc, and link the library) and keeps its result in `directory`/<candidate>/ so that it can
+    run ahead of time on a machine without a GPU; `evaluate` prepares what is not there yet.  The
+    outputs of the last evaluated candidate stay in `last_outputs` (inputs are seeded, integer-valued:
+    candidates can be compared bit for bit)."""
+
+    def __init__(self, source, function, directory, repeat=20, seed=1):
+        self.source, self.function, self.directory = os.path.abspath(source), function, os.path.abspath(directory)
+        self.repeat, self.seed = repeat, seed
+        self.last_outputs, self.last_kernels = None, None
+
+    @staticmethod
+    def candidate_name(candidate):
+        return "_".join("%s-%s" % (k, candidate[k]) for k in sorted(candidate)) or "default"
+
+    def library(self, candidate):
+        return os.path.join(self.directory, self.candidate_name(candidate), "build", "lib%s.so" % self.function)
+
+    def prepare(self, candidate, force=False):
+        lib = self.library(candidate)
+        newest_input = max(os.path.getmtime(self.source), os.path.getmtime(build.compiler_library()))
+        if os.path.exists(lib) and os.path.getmtime(lib) >= newest_input and not force:
+            return lib
+        os.makedirs(self.directory, exist_ok=True)
+        gen = os.path.join(self.directory, "generator")
+        if force or not os.path.exists(gen) or os.path.getmtime(gen) < newest_input:
+            subprocess.run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.dirname(self.source), "-o", gen,
+                            self.source, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG], check=True)
+        directory = os.path.join(self.directory, self.candidate_name(candidate))
+        generate(gen, directory, {k: str(v) for k, v in candidate.items()})
+        return link(directory, self.function)
+
+    def get_measurements(self, candidate, repeat=None):
+        lib = self.prepare(candidate)
+        manifest = runtime.manifest_of(lib, self.function)
+        program = runtime.Program(lib, self.function)
+        args = make_arguments(manifest, self.seed)
+
+        def call():
+            program(*[runtime.Buffer.from_device(a.ptr, a.host.shape, a.host.dtype) if isinstance(a, DeviceBuffer) else a for a in args])
         call()
-    times = []
-    for _ in range(repeat):
-        with runtime.DeviceTimer() as t:
+        self.last_outputs = [(a.download() if isinstance(a, DeviceBuffer) else a.copy())
+                             for a, m in zip(args, manifest["arguments"]) if m["kind"] == "output"]
+        self.last_kernels = [k["how"] for k in manifest["kernels"]]
+        repeat = repeat or self.repeat
+        for _ in range(max(3, repeat // 2)):
             call()
-        times.append(t.ms)
-    for a in args:
-        if isinstance(a, DeviceBuffer):
-            a.free()
-    return float(np.median(times)), outputs
+        times = []
+        for _ in range(repeat):
+            with runtime.DeviceTimer() as t:
+                call()
+            times.append(t.ms)
+        for a in args:
+            if isinstance(a, DeviceBuffer):
+                a.free()
+        return times
+
+    def evaluate(self, candidate):
+        return float(np.median(self.get_measurements(candidate)))
 
 
 def main(argv=None):
-    ap = argparse.ArgumentParser(description=__doc__.split("\\n\\n")[0])
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("source")
     ap.add_argument("function")
     ap.add_argument("--knob", action="append", default=[], help="NAME=v1,v2,...")
@@ -115,23 +164,16 @@ def main(argv=None):
     if runtime.wrappers().tiramisu_hip_device_count() < 1:
         raise SystemExit("no HIP device visible")
     scratch = a.keep or tempfile.mkdtemp(prefix="tiramisu_autotune_")
-    os.makedirs(scratch, exist_ok=True)
-    gen = os.path.join(scratch, "generator")
-    subprocess.run(["g++", "-std=c++17", "-O1", "-I" + build.INCLUDE, "-I" + os.path.dirname(os.path.abspath(a.source)), "-o", gen,
-                    a.source, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG], check=True)
+    evaluator = evaluate_by_execution(a.source, a.function, scratch, repeat=a.repeat)
     results, first = [], None
-    for n, env in enumerate(variants(a.knob)):
-        directory = os.path.join(scratch, "v%d" % n)
-        generate(gen, directory, env)
-        lib = link(directory, a.function)
-        manifest = runtime.manifest_of(lib, a.function)
-        ms, outputs = run_variant(lib, a.function, manifest, a.repeat, seed=1)
+    for candidate in variants(a.knob):
+        ms = evaluator.evaluate(candidate)
         same = True
         if first is None:
-            first = outputs
+            first = evaluator.last_outputs
         else:
-            same = all(np.array_equal(x, y) for x, y in zip(first, outputs))
-        results.append({"knobs": env, "ms": ms, "same_as_first": same, "kernels": [k["how"].split(",")[0] for k in manifest["kernels"]]})
+            same = all(np.array_equal(x, y) for x, y in zip(first, evaluator.last_outputs))
+        results.append({"knobs": candidate, "ms": ms, "same_as_first": same, "kernels": [k.split(",")[0] for k in evaluator.last_kernels]})
     results.sort(key=lambda r: r["ms"])
     for r in results:
         print(json.dumps(r))

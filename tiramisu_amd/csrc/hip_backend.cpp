@@ -77,7 +77,134 @@ struct generic_kernel_gen {
                 if (n->lkind == leaf_kind::let) inner.insert(n->comp->get_name());
             }
         });
+        if (!std::getenv("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
+            std::vector<node_ptr> stack;
+            find_reductions(root, stack);
+        }
     }
+
+    // ---- sums across threads.  A statement  X[e] = X[e] + term  under a loop mapped to threadIdx.x whose
+    // iterator the element e does not involve asks every thread of that loop to add into one element:
+    // as written that is a race (the reference emits it as such).  Floating-point addition being what
+    // the program asks to be reassociated here, the loop is lowered to a private partial sum per thread,
+    // a sum across the lanes of the wavefront with DPP row shifts and broadcasts (across wavefronts
+    // through LDS when the loop is wider than a wavefront), and one read-modify-write of X[e] by the last
+    // thread of the loop.
+    struct thread_reduction { node_ptr leaf; expr term; int width; };
+    std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
+    int reduction_count = 0;
+    int guard_depth = 0;          // mapped loops with a guard around the code being emitted
+
+    static bool is_same_element(const expr &e, const buffer *b, const std::vector<expr> &idx) {
+        if (e.get_expr_type() != e_op || e.get_op_type() != o_access || e.get_name() != b->get_name() || e.get_access().size() != idx.size())
+            return false;
+        for (size_t i = 0; i < idx.size(); i++)
+            if (!lir::simplify(e.get_access()[i]).is_equal(lir::simplify(idx[i]))) return false;
+        return true;
+    }
+
+    void find_reductions(const node_ptr &n, std::vector<node_ptr> &stack) {
+        if (!n) return;
+        if (n->kind == node_kind::loop) stack.push_back(n);
+        if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && !n->predicate.is_defined() && n->lets.empty() &&
+            n->rhs.is_defined() && n->rhs.get_data_type() == p_float32 && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
+            consider_reduction(n, stack);
+        for (auto &c : n->children) find_reductions(c, stack);
+        find_reductions(n->body, stack);
+        find_reductions(n->then_body, stack);
+        find_reductions(n->else_body, stack);
+        if (n->kind == node_kind::loop) stack.pop_back();
+    }
+
+    void consider_reduction(const node_ptr &leaf, const std::vector<node_ptr> &stack) {
+        expr term;
+        if (is_same_element(leaf->rhs.get_operand(0), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(1);
+        else if (is_same_element(leaf->rhs.get_operand(1), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(0);
+        else return;
+        bool reads_self = false;
+        term.visit([&](const expr &x) {
+            if (x.get_expr_type() == e_op && x.get_op_type() == o_access && x.get_name() == leaf->lhs->get_name()) reads_self = true;
+        });
+        if (reads_self) return;
+        auto element_involves = [&](const std::string &it) {
+            for (auto &e : leaf->lhs_index) if (lir::mentions(e, it)) return true;
+            return false;
+        };
+        // the thread-mapped loops around the statement that its element does not involve
+        node_ptr R;
+        size_t at = 0;
+        for (size_t d = 0; d < stack.size(); d++)
+            if (stack[d]->gpu_thread >= 0 && !element_involves(stack[d]->iterator)) {
+                if (R || stack[d]->gpu_thread != 0) return;     // one loop, on threadIdx.x (consecutive lanes)
+                R = stack[d];
+                at = d;
+            }
+        if (!R || loops_per_dim[1][0] != 1) return;
+        // inside it: this statement only, under serial loops whose iterators the element does not involve either
+        for (size_t d = at + 1; d < stack.size(); d++)
+            if (stack[d]->gpu_thread >= 0 || stack[d]->gpu_block >= 0 || element_involves(stack[d]->iterator)) return;
+        int leaves_inside = 0;
+        lir::walk(R, [&](const node_ptr &x) { if (x->kind == node_kind::leaf) leaves_inside++; });
+        if (leaves_inside != 1) return;
+        // width of the loop = blockDim.x: a power of two up to a wavefront, or whole wavefronts
+        bool guard;
+        expr first;
+        const expr ext = lir::simplify(host_extent(R, first, guard));
+        if (!ext.is_integer_literal()) return;
+        const long w = ext.get_int_val();
+        const bool in_wave = w >= 2 && w <= 64 && (w & (w - 1)) == 0, waves = w >= 128 && w <= 1024 && w % 64 == 0;
+        if (!in_wave && !waves) return;
+        if (waves) {
+            // the barrier of the LDS stage must be reached by every thread: no guarded mapped loop around it,
+            // no serial loop or condition between the kernel entry and the loop
+            for (size_t d = 0; d < at; d++) {
+                bool g;
+                expr f0;
+                if (stack[d]->gpu_thread < 0 && stack[d]->gpu_block < 0) return;
+                host_extent(stack[d], f0, g);
+                const int dim = stack[d]->gpu_block >= 0 ? stack[d]->gpu_block : stack[d]->gpu_thread;
+                if (g || loops_per_dim[stack[d]->gpu_block >= 0 ? 0 : 1][dim] > 1) return;
+            }
+        }
+        reductions[R.get()] = {leaf, term, (int)w};
+    }
+
+    void emit_thread_reduction(const node_ptr &n, const thread_reduction &r, int ind) {
+        bool guard;
+        expr first;
+        block_ext[0].push_back(host_extent(n, first, guard));
+        const std::string acc = "_partial" + std::to_string(reduction_count++);
+        body << pad(ind) << "{\n";
+        body << pad(ind + 1) << "float " << acc << " = 0.0f;   // this thread's share of the sum\n";
+        body << pad(ind + 1) << "{\n";
+        body << pad(ind + 2) << "const int32_t " << n->iterator << " = (int32_t)threadIdx.x + " << dev.print(first) << ";\n";
+        if (guard)
+            body << pad(ind + 2) << "if (" << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+        pending_partial = acc;
+        pending_leaf = r.leaf.get();
+        pending_term = r.term;
+        emit(n->body, ind + (guard ? 3 : 2));
+        pending_leaf = nullptr;
+        if (guard) body << pad(ind + 2) << "}\n";
+        body << pad(ind + 1) << "}\n";
+        if (r.width <= 64) {
+            body << pad(ind + 1) << acc << " = twave::wave_group_sum<" << r.width << ">(" << acc << ");\n";
+        } else {
+            needs_reduction_scratch = true;
+            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", _reduction_scratch, "
+                 << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
+        }
+        body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << ") "
+             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, p_float32) << "\n";
+        body << pad(ind) << "}\n";
+        add_include_once(ctx, "#include \"" + kernel_dir() + "/wave_reduce.hip.h\"");
+        wave_reductions++;
+    }
+    std::string pending_partial;
+    const node *pending_leaf = nullptr;
+    expr pending_term;
+    bool needs_reduction_scratch = false;
+    int wave_reductions = 0;
 
     // Kernel-invariant part of a bound that is a min() (upper bounds) or max() (lower bounds) of
     // several expressions: the arguments that do not involve in-kernel iterators.
@@ -139,6 +266,11 @@ struct generic_kernel_gen {
 
     void emit_loop(const node_ptr &n, int ind) {
         const bool is_block = n->gpu_block >= 0, is_thread = n->gpu_thread >= 0;
+        auto red = reductions.find(n.get());
+        if (red != reductions.end()) {
+            emit_thread_reduction(n, red->second, ind);
+            return;
+        }
         if (is_block || is_thread) {
             const int dim = is_block ? n->gpu_block : n->gpu_thread;
             bool guard;
@@ -187,6 +319,10 @@ struct generic_kernel_gen {
     }
 
     void emit_leaf(const node_ptr &n, int ind) {
+        if (n.get() == pending_leaf) {
+            body << pad(ind) << pending_partial << " = " << pending_partial << " + " << dev.print(pending_term) << ";\n";
+            return;
+        }
         switch (n->lkind) {
         case leaf_kind::sync: body << pad(ind) << "__syncthreads();\n"; return;
         case leaf_kind::allocate:
@@ -239,6 +375,9 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
 
     kernel k;
     k.how = "generic";
+    if (g.wave_reductions)
+        k.how += ", " + std::to_string(g.wave_reductions) + " sum(s) across the threads of a loop lowered to DPP wavefront reductions" +
+                 (g.needs_reduction_scratch ? " (wavefront totals combined through LDS)" : "");
     k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
     function *f = ctx.f;
 
@@ -309,6 +448,7 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
     }
     os << ")\n{\n";
     for (auto &d : top_decls) os << "    " << d << "\n";
+    if (g.needs_reduction_scratch) os << "    __shared__ float _reduction_scratch[16];\n";
     os << g.body.str() << "}\n";
     k.source = os.str();
     return k;

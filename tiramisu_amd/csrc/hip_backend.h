@@ -83,6 +83,11 @@ kernel emit_generic_kernel(context &ctx, const lir::node_ptr &root);
 bool emit_contraction(context &ctx, const lir::node_ptr &root, launch_plan &plan, const fusion_request *fuse = nullptr);
 bool emit_stencil(context &ctx, const lir::node_ptr &root, const lir::node_ptr &time_loop, launch_plan &plan);
 
+/** Directory of the kernel headers that emitted code includes (TIRAMISU_AMD_KERNEL_DIR overrides the
+  * one compiled in), and the helper that adds an #include line to the kernel file once. */
+std::string kernel_dir();
+void add_include_once(context &ctx, const std::string &line);
+
 /** Text of the launch of \p k with the argument list taken from host variables of the same names. */
 std::string launch_text(const kernel &k, const std::string &indent);
 

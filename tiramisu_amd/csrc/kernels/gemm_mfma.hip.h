@@ -76,6 +76,17 @@ struct regrouped_rows {
     __device__ __forceinline__ auto load4(int x, int k) const { return src.load4(regrouped_index<BN, UB>(x, UE), k); }
 };
 
+// Two operands behind one another along k: k < K1 reads the first, the rest the second (from its own
+// k = 0).  Lets several product terms that feed the same accumulators run as one pipelined loop;
+// K1 must be a multiple of 4 (a 16-byte load along k never straddles the seam).
+template <class S1, class S2>
+struct concat_k {
+    S1 first;
+    S2 second;
+    int K1;
+    __device__ __forceinline__ f32x4 load4(int x, int k) const { return k < K1 ? first.load4(x, k) : second.load4(x, k - K1); }
+};
+
 // One operand tile of X x BK elements (X = BM for A, BN for B).
 template <int X, int BK, int NT, bool KMAJOR, bool EDGE, int PAD>
 struct operand_tile {

@@ -1,0 +1,55 @@
+// Sums across the lanes of a wave64 with DPP (data-parallel primitives: an operand of a vector
+// instruction is taken from another lane of the same wavefront, no LDS traffic, no barrier).
+//
+// wave_group_sum<W>(v): the lanes of a wavefront are split into groups of W consecutive lanes (W a
+// power of two, 2..64); the LAST lane of every group returns the sum of its group's values, the other
+// lanes partial sums.  Steps: row_shr:1,2,4,8 add, within each row of 16 lanes, the value 1, 2, 4, 8
+// lanes to the left (lanes without such a neighbour add 0), which leaves the total of the window of
+// 2, 4, 8, 16 lanes that ends at a lane; row_bcast:15 adds lane 15 of rows 0 and 2 to every lane of
+// rows 1 and 3, row_bcast:31 adds lane 31 to rows 2 and 3 -- so lane 31 ends with the total of lanes
+// 0..31 and lane 63 with the total of the wavefront.
+//
+// block_group_sum<W>(v, scratch): groups of W = 128..1024 consecutive threads of a workgroup (whole
+// wavefronts); wavefront totals meet in LDS.  All threads of the workgroup must call it together.
+#ifndef TIRAMISU_AMD_WAVE_REDUCE_HIP_H
+#define TIRAMISU_AMD_WAVE_REDUCE_HIP_H
+#include <hip/hip_runtime.h>
+
+namespace twave {
+
+template <int CTRL, int ROW_MASK, bool ZERO_FILL>
+__device__ __forceinline__ float dpp_term(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, ZERO_FILL));
+}
+
+template <int W>
+__device__ __forceinline__ float wave_group_sum(float v) {
+    static_assert(W >= 2 && W <= 64 && (W & (W - 1)) == 0, "group width must be a power of two up to the wavefront size");
+    if (W >= 2) v += dpp_term<0x111, 0xf, true>(v);    // row_shr:1
+    if (W >= 4) v += dpp_term<0x112, 0xf, true>(v);    // row_shr:2
+    if (W >= 8) v += dpp_term<0x114, 0xf, true>(v);    // row_shr:4
+    if (W >= 16) v += dpp_term<0x118, 0xf, true>(v);   // row_shr:8
+    if (W >= 32) v += dpp_term<0x142, 0xa, false>(v);  // row_bcast:15 into rows 1 and 3
+    if (W >= 64) v += dpp_term<0x143, 0xc, false>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// `scratch` holds one float per wavefront of the workgroup; `linear` is the thread's linear id.
+template <int W>
+__device__ __forceinline__ float block_group_sum(float v, float *scratch, int linear) {
+    static_assert(W % 64 == 0 && W >= 128 && W <= 1024, "group width must be whole wavefronts");
+    v = wave_group_sum<64>(v);
+    if ((linear & 63) == 63) scratch[linear >> 6] = v;
+    __syncthreads();
+    float total = 0.f;
+    if ((linear % W) == W - 1) {
+        const int last = linear >> 6;
+#pragma unroll
+        for (int w = W / 64 - 1; w >= 0; w--) total += scratch[last - w];
+    }
+    __syncthreads();
+    return total;
+}
+
+}  // namespace twave
+#endif

@@ -18,8 +18,6 @@ using lir::node;
 using lir::node_kind;
 using lir::node_ptr;
 
-namespace {
-
 #ifndef TIRAMISU_AMD_KERNEL_DIR
 #define TIRAMISU_AMD_KERNEL_DIR "."
 #endif
@@ -28,6 +26,13 @@ std::string kernel_dir() {
     if (const char *e = std::getenv("TIRAMISU_AMD_KERNEL_DIR")) return e;
     return TIRAMISU_AMD_KERNEL_DIR;
 }
+
+void add_include_once(context &ctx, const std::string &line) {
+    if (ctx.include_once.insert(line).second) ctx.includes += line + "\n";
+}
+
+namespace {
+
 
 int env_int(const char *name, int dflt) {
     const char *e = std::getenv(name);
@@ -85,10 +90,6 @@ void leaves_under(const node_ptr &n, std::vector<node_ptr> &out, bool &has_cond)
         if (x->kind == node_kind::leaf) out.push_back(x);
         if (x->kind == node_kind::cond) has_cond = true;
     });
-}
-
-void add_include_once(context &ctx, const std::string &line) {
-    if (ctx.include_once.insert(line).second) ctx.includes += line + "\n";
 }
 
 }  // namespace
@@ -1055,6 +1056,10 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         !std::getenv("TIRAMISU_MFMA_NO_SPLITK")) {
         BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
         DEPTH = (int)std::min<long>(4, std::max<long>(1, Kl / BK - 1));   // latency-bound: ask for (up to) all slices at once
+        // a reduction of 1024 or more (several terms run as one loop): the loop is long enough to hide its own
+        // latencies, and four groups of wavefronts with 64-k slices and no extra slices in flight are faster
+        // (4-layer LSTM cell, 64x2048x1024 per layer: 1.30 ms per pass against 1.55 ms)
+        if ((long)products.size() * Kl >= 1024) { BK = 64; WGK = 4; DEPTH = 1; }
     }
     // at most one 64x64 tile per compute unit and a long reduction: two groups of wavefronts share each
     // (64-k) slice, so that every SIMD has two wavefronts to alternate between (1024^3: 20.6 us against 21.9)
@@ -1063,6 +1068,10 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         WGK = 2; BK = 64;
     }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
+    if (const char *e = std::getenv("TIRAMISU_MFMA_BM")) BM = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_BN")) BN = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_WGM")) WGM = std::atoi(e);
+    if (const char *e = std::getenv("TIRAMISU_MFMA_WGN")) WGN = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
@@ -1274,8 +1283,12 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
     int term = 0, ktab_words = 0;
     const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
+    // several product terms over plain operands: one pipelined loop over the concatenated reduction ranges
+    // (a call per term would drain and refill the pipeline between the terms)
+    bool merge_terms = !bf16 && operands.size() > 1 && lit && Kl % 4 == 0 && !std::getenv("TIRAMISU_MFMA_SEPARATE_TERMS");
+    for (auto &o : operands) merge_terms = merge_terms && o.first.linear && o.second.linear;
     for (auto &o : operands) {
-        body << "    {\n";
+        if (!merge_terms || term == 0) body << "    {\n";
         if (bf16) {
             used_buffers.insert(o.first.buf->get_name());
             used_buffers.insert(o.second.buf->get_name());
@@ -1287,7 +1300,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         }
         int which = 0;
         for (const operand_info *g : {&o.first, &o.second}) {
-            const char *nm = which == 0 ? "_A" : "_B";
+            const std::string nm_text = std::string(which == 0 ? "_A" : "_B") + (merge_terms ? std::to_string(term) : "");
+            const char *nm = nm_text.c_str();
             const group_info &rowg = which == 0 ? GM : GN;
             used_buffers.insert(g->buf->get_name());
             if (g->linear) {
@@ -1339,13 +1353,26 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
             }
             which++;
         }
-        if (with_consumer) {
-            body << "        const tgemm::regrouped_rows<decltype(_B), CFG::BN, " << UB << "> _Bq{_B, " << UE << "};\n";
-            body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _Bq, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
-        } else {
-            body << "        tgemm::tile_accumulate<CFG>(_acc, _A, _B, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
-        }
         term++;
+        if (merge_terms && term < (int)operands.size()) continue;
+        std::string a_name = "_A", b_name = "_B", k_text = "_K";
+        if (merge_terms) {
+            a_name = "_A0";
+            b_name = "_B0";
+            for (int t = 1; t < term; t++) {
+                for (std::string *nm : {&a_name, &b_name}) {
+                    const std::string next = std::string(nm == &a_name ? "_A" : "_B") + std::to_string(t), cat = *nm + "c";
+                    body << "        const tgemm::concat_k<decltype(" << *nm << "), decltype(" << next << ")> " << cat << "{" << *nm << ", " << next << ", " << t << " * _K};\n";
+                    *nm = cat;
+                }
+            }
+            k_text = std::to_string(term) + " * _K";
+        }
+        if (with_consumer) {
+            body << "        const tgemm::regrouped_rows<decltype(" << b_name << "), CFG::BN, " << UB << "> _Bq{" << b_name << ", " << UE << "};\n";
+            b_name = "_Bq";
+        }
+        body << "        tgemm::tile_accumulate<CFG>(_acc, " << a_name << ", " << b_name << ", " << k_text << ", _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
     }
     if (with_consumer)   // the finished tile, handed to the consumer's statements through LDS (behind the operand stages)
         body << "    float *_gt = _lds + CFG::LDS_BYTES / 4 + " << ktab_words << ";\n";

@@ -144,8 +144,10 @@ static void generate(int L, int B, int H, int S)
 int main()
 {
     generate(4, 64, 512, 100);   // benchmark configuration 5
+    if (std::getenv("LSTM_ONLY_FULL")) return 0;
     generate(2, 8, 32, 5);
     generate(1, 4, 16, 3);
     generate(3, 20, 64, 4);
+    generate(2, 64, 256, 6);     // whole 64x32 tiles with the reduction split over eight groups of wavefronts
     return 0;
 }
