@@ -38,6 +38,7 @@ import numpy as np  # noqa: E402
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 BF16_MFMA_PEAK_TFLOPS = 2500.0
+FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X vector fp32 (256 CUs x 128 lanes x 2 flops x 2.4 GHz): what a kernel without MFMA is priced against
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_by_kernel.md")
@@ -333,6 +334,21 @@ def bench_lstm(steps, warmup, with_cpu):
                           with_cpu, "unscheduled program, batch loop parallelized")   # one kernel does all the flops: the fused cell
 
 
+def bench_sgemm_cache_shared(steps, warmup, with_cpu):
+    """The reference's tuned cache_shared schedule (generator3) at 3072^3, kept on the schedule-faithful
+    emitter: VALU FMAs fed from LDS tiles.  Not one of the benchmark configurations and not part of
+    `--workload all`; it is here so that the emitter's LDS behaviour can be put under the profiler."""
+    M = N = K = 3072
+    rng = np.random.RandomState(30)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    C = np.zeros((M, N), np.float32)
+    out = _generic_bench("sgemm_cache_shared_3072", [("host", np.array([1.0, 0.0], np.float32)), A, B, C],
+                         2.0 * M * N * K, FP32_VALU_PEAK_TFLOPS, steps, warmup, False, "")
+    out["roofline"]["bound"] = "valu"
+    return out
+
+
 WORKLOADS = {
     "heat2d": lambda s, w, c: bench_heat2d(s, w, c),
     "sgemm1024": lambda s, w, c: bench_sgemm(1024, s, w, c),
@@ -358,7 +374,8 @@ def main():
     if runtime.wrappers().tiramisu_hip_device_count() < 1:
         sys.exit("no HIP device visible")
     WORKLOADS["copy"] = bench_copy   # calibration only, not part of "all"
-    names = [n for n in WORKLOADS if n != "copy"] if a.workload == "all" else [a.workload]
+    WORKLOADS["sgemm_cache_shared"] = bench_sgemm_cache_shared   # profiling of the schedule-faithful emitter only
+    names = [n for n in WORKLOADS if n not in ("copy", "sgemm_cache_shared")] if a.workload == "all" else [a.workload]
     results = {}
     for n in names:
         with_cpu = not a.no_cpu

@@ -244,11 +244,64 @@ struct generic_kernel_gen {
         return lir::simplify(lir::simplify(up - first) + 1);
     }
 
+    // ---- barriers of cache_shared.  Every LDS tile comes with a barrier before its cooperative copy (the
+    // previous contents are no longer read) and one after it (the new contents are visible), in the
+    // reference's order (tiramisu_core.cpp:9479-9515): two tiles filled at the same loop level give
+    //   sync  copy(B)  sync  sync  copy(A)  sync  compute.
+    // Copies of different tiles that read global memory only do not need a barrier between them, and two
+    // barriers in a row are one: the sequence is emitted as  sync  copy(B)  copy(A)  sync  compute.
+    static bool is_sync(const node_ptr &n) { return n->kind == node_kind::leaf && n->lkind == leaf_kind::sync; }
+
+    // the LDS tiles written by a statement list that consists of cooperative cache copies only (else: false)
+    bool tiles_filled_by(const std::vector<node_ptr> &nodes, std::set<std::string> &tiles) const {
+        bool only_copies = !nodes.empty();
+        for (auto &n : nodes)
+            lir::walk(n, [&](const node_ptr &x) {
+                if (x->kind != node_kind::leaf) return;
+                if (x->lkind != leaf_kind::assign || !x->comp || !x->comp->get_cache_consumer() || !x->lhs ||
+                    x->lhs->get_location() != memory_location::shared) { only_copies = false; return; }
+                x->rhs.visit([&](const expr &e) {
+                    if (e.get_expr_type() == e_op && e.get_op_type() == o_access &&
+                        f->get_buffers().at(e.get_name())->get_location() == memory_location::shared) only_copies = false;
+                });
+                tiles.insert(x->lhs->get_name());
+            });
+        return only_copies;
+    }
+
+    std::vector<node_ptr> without_redundant_barriers(const std::vector<node_ptr> &in) const {
+        if (std::getenv("TIRAMISU_HIP_KEEP_BARRIERS")) return in;
+        std::vector<node_ptr> flat, v;
+        std::function<void(const node_ptr &)> flatten = [&](const node_ptr &n) {
+            if (n && n->kind == node_kind::block) for (auto &c : n->children) flatten(c);
+            else if (n) flat.push_back(n);
+        };
+        for (auto &n : in) flatten(n);
+        for (auto &n : flat)
+            if (!(is_sync(n) && !v.empty() && is_sync(v.back()))) v.push_back(n);      // two barriers in a row
+        for (bool changed = true; changed;) {
+            changed = false;
+            std::vector<size_t> syncs;
+            for (size_t i = 0; i < v.size(); i++) if (is_sync(v[i])) syncs.push_back(i);
+            for (size_t s = 1; s + 1 < syncs.size() && !changed; s++) {
+                std::set<std::string> before, after;
+                const std::vector<node_ptr> left(v.begin() + syncs[s - 1] + 1, v.begin() + syncs[s]), right(v.begin() + syncs[s] + 1, v.begin() + syncs[s + 1]);
+                if (!tiles_filled_by(left, before) || !tiles_filled_by(right, after)) continue;
+                bool disjoint = true;
+                for (auto &t : before) if (after.count(t)) disjoint = false;
+                if (!disjoint) continue;
+                v.erase(v.begin() + syncs[s]);
+                changed = true;
+            }
+        }
+        return v;
+    }
+
     void emit(const node_ptr &n, int ind) {
         if (!n) return;
         switch (n->kind) {
         case node_kind::block:
-            for (auto &c : n->children) emit(c, ind);
+            for (auto &c : without_redundant_barriers(n->children)) emit(c, ind);
             break;
         case node_kind::cond:
             body << pad(ind) << "if (" << dev.print(n->condition) << ") {\n";
