@@ -50,6 +50,15 @@ def test_batch_of_64_rows_splits_k(K, tB):
     run(64, 96, K, 2.0, 0.0, tB=tB, seed=2)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 256, 8192), (128, 192, 4096), (100, 70, 2500), (640, 640, 4096), (64, 64, 65536)])
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, True)])
+def test_deep_reductions_split_k_over_workgroups(M, N, K, tA, tB):
+    # few 64x64 tiles and K >= 2048: chunks of K on different workgroups, partial tiles through the
+    # scratch workspace, the last workgroup of a tile adds them in chunk order
+    run(M, N, K, 1.0, 0.0, tA=tA, tB=tB)
+    run(M, N, K, 2.0, 1.0, tA=tA, tB=tB, pad=4, off=16, seed=3)
+
+
 @pytest.mark.parametrize("tA,tB", [(False, True), (True, False), (True, True)])
 def test_transposed_operands_padding_and_offsets(tA, tB):
     run(128, 192, 96, 1.0, 1.0, tA=tA, tB=tB)

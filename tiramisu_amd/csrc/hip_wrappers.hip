@@ -215,6 +215,118 @@ void dispatch_skinny(const float *A, const float *B, float *C, int M, int N, int
     }
 }
 
+// ---- deep reductions: the K range split over workgroups.
+// A problem with few C tiles and a long K (256 x 256 x 65536: sixteen 64x64 tiles) leaves most of the
+// chip idle when one workgroup walks the whole K range of a tile.  Here gridDim.y workgroups take a
+// chunk of K each for the same tile, write their partial tile to a scratch buffer, and the last one to
+// finish (a counter per tile) adds the partial tiles in chunk order -- so the result does not depend on
+// which workgroup came last -- and applies alpha / beta.  No workgroup waits for another.
+// Scratch layout: floats [tile][chunk][register quad][thread][4], then one 32-bit counter per tile
+// (zero before the launch; the last workgroup leaves it zero again).
+constexpr int SPLITK_TILE = 64, SPLITK_THREADS = 256, SPLITK_MAX_TILES = 128;
+constexpr uint64_t SPLITK_COUNTER_BYTES = SPLITK_MAX_TILES * sizeof(unsigned);
+
+template <class CFG>
+__global__ void __launch_bounds__(CFG::NT) sgemm_splitk_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                                float *__restrict__ C, int M, int N, int K, long lda, long ldb,
+                                                                long ldc, float alpha, float beta, int vec_ok, int chunk,
+                                                                float *__restrict__ partial, unsigned *__restrict__ counters) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    __shared__ unsigned ticket;
+    static_assert(CFG::WGK == 1 && CFG::TM == 1 && CFG::TN == 1, "one accumulator tile per wavefront");
+    int tm, tn;
+    const int tiles_n = (N + CFG::BN - 1) / CFG::BN;
+    tm = blockIdx.x / tiles_n;
+    tn = blockIdx.x % tiles_n;
+    const int z = blockIdx.y, Z = gridDim.y;
+    const int k0 = z * chunk, kc = min(chunk, K - k0);
+    tgemm::accumulators<CFG> acc;
+    acc.clear();
+    tgemm::linear_source<CFG::A_KMAJOR, CFG::EDGE> sa{A + (CFG::A_KMAJOR ? (long)k0 : (long)k0 * lda), lda, M, kc, vec_ok != 0};
+    tgemm::linear_source<CFG::B_KMAJOR, CFG::EDGE> sb{B + (CFG::B_KMAJOR ? (long)k0 : (long)k0 * ldb), ldb, N, kc, vec_ok != 0};
+    tgemm::tile_accumulate<CFG>(acc, sa, sb, kc, tm * CFG::BM, tn * CFG::BN, lds);
+    tgemm::f32x4 *mine = reinterpret_cast<tgemm::f32x4 *>(partial) + ((long)blockIdx.x * Z + z) * 4 * CFG::NT;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        mine[r * CFG::NT + threadIdx.x] = tgemm::f32x4{acc.t[0][0][4 * r], acc.t[0][0][4 * r + 1], acc.t[0][0][4 * r + 2], acc.t[0][0][4 * r + 3]};
+    __threadfence();                       // the partial tile is visible device-wide before the ticket is taken
+    __syncthreads();
+    if (threadIdx.x == 0) ticket = atomicAdd(&counters[blockIdx.x], 1u);
+    __syncthreads();
+    if (ticket != (unsigned)(Z - 1)) return;
+    __threadfence();                       // and the other workgroups' tiles are visible to this one
+    const tgemm::f32x4 *all = reinterpret_cast<const tgemm::f32x4 *>(partial) + (long)blockIdx.x * Z * 4 * CFG::NT;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        tgemm::f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < Z; c++) {
+            sum += all[((long)c * 4 + r) * CFG::NT + threadIdx.x];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc.t[0][0][4 * r + e] = sum[e];
+    }
+    tgemm::axpby_epilogue epi{C, ldc, alpha, beta};
+    tgemm::tile_epilogue<CFG>(acc, M, N, tm * CFG::BM, tn * CFG::BN, epi);
+    if (threadIdx.x == 0) counters[blockIdx.x] = 0;     // ready for the next launch
+}
+
+__global__ void clear_counters_kernel(unsigned *counters, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) counters[i] = 0;
+}
+
+// How a problem is split: chunks of K (a multiple of the 32-k slice) and the scratch it needs; chunks == 1: not split.
+struct splitk_plan {
+    int tiles = 0, chunks = 1, chunk = 0;
+    uint64_t scratch_bytes = 0;    // partial tiles + counters
+};
+
+splitk_plan plan_splitk(int M, int N, int K, uint64_t max_bytes) {
+    splitk_plan p;
+    p.tiles = ((M + SPLITK_TILE - 1) / SPLITK_TILE) * ((N + SPLITK_TILE - 1) / SPLITK_TILE);
+    if (p.tiles > SPLITK_MAX_TILES || K < 2048) return p;
+    // enough workgroups for every compute unit, at least 512 of K each
+    int chunks = std::min((256 + p.tiles - 1) / p.tiles, K / 512);
+    const uint64_t per_chunk = (uint64_t)p.tiles * SPLITK_TILE * SPLITK_TILE * sizeof(float);
+    while (chunks > 1 && per_chunk * chunks + SPLITK_COUNTER_BYTES > max_bytes) chunks--;
+    if (chunks < 2) return p;
+    p.chunk = ((K + chunks - 1) / chunks + 31) / 32 * 32;
+    p.chunks = (K + p.chunk - 1) / p.chunk;
+    p.scratch_bytes = per_chunk * p.chunks + SPLITK_COUNTER_BYTES;
+    return p;
+}
+
+template <bool AK, bool BK_, bool EDGE>
+void launch_splitk(const splitk_plan &p, const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
+                   float alpha, float beta, bool vec_ok, void *scratch) {
+    typedef tgemm::config<SPLITK_TILE, SPLITK_TILE, 32, 2, 2, AK, BK_, EDGE> CFG;
+    static_assert(CFG::NT == SPLITK_THREADS, "scratch layout assumes 256 threads");
+    unsigned *counters = reinterpret_cast<unsigned *>(scratch);
+    float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(scratch) + SPLITK_COUNTER_BYTES);
+    hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(SPLITK_MAX_TILES), 0, current_stream, counters, p.tiles);
+    hipLaunchKernelGGL((sgemm_splitk_kernel<CFG>), dim3(p.tiles, p.chunks), dim3(CFG::NT), CFG::LDS_BYTES, current_stream, A, B, C,
+                       M, N, K, lda, ldb, ldc, alpha, beta, vec_ok ? 1 : 0, p.chunk, partial, counters);
+    check(hipGetLastError(), "tiramisu_hip_sgemm");
+}
+
+void dispatch_splitk(const splitk_plan &p, bool tA, bool tB, bool edge, const float *A, const float *B, float *C, int M, int N, int K,
+                     long lda, long ldb, long ldc, float alpha, float beta, bool vec_ok, void *scratch) {
+#define SPLITK_CASE(AK, BKM)                                                                                              \
+    if (edge) launch_splitk<AK, BKM, true>(p, A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok, scratch);              \
+    else launch_splitk<AK, BKM, false>(p, A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok, scratch)
+    if (!tA && !tB) { SPLITK_CASE(true, false); }
+    else if (!tA && tB) { SPLITK_CASE(true, true); }
+    else if (tA && !tB) { SPLITK_CASE(false, false); }
+    else { SPLITK_CASE(false, true); }
+#undef SPLITK_CASE
+}
+
+// Scratch of the allocating entry point: one block per host thread (calls work on the thread's
+// current stream), grown on demand, kept until the process ends.
+thread_local void *splitk_workspace = nullptr;
+thread_local uint64_t splitk_workspace_bytes = 0;
+constexpr uint64_t SPLITK_WORKSPACE_LIMIT = (uint64_t)256 << 20;
+
 template <bool AK, bool BK_>
 void dispatch_edge(bool edge, const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb,
                    long ldc, float alpha, float beta, bool vec_ok) {
@@ -318,18 +430,18 @@ int32_t tiramisu_hip_stream_synchronize(int32_t) {
     return 0;
 }
 
-int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
-                       uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
-                       bool transposeA, bool transposeB) {
+static int sgemm_impl(const char *fn, float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
+                      float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
+                      bool transposeA, bool transposeB) {
     if (ldA == 0) ldA = transposeA ? M : K;
     if (ldB == 0) ldB = transposeB ? K : N;
     if (ldC == 0) ldC = N;
     if (M == 0 || N == 0) return 0;
-    scoped_record rec("tiramisu_hip_sgemm");
+    scoped_record rec(fn);
     const float *a = A + offsetA, *b = B + offsetB;
     float *c = C + offsetC;
     if (M > 0x7fffffffull || N > 0x7fffffffull || K > 0x7fffffffull) {
-        fprintf(stderr, "Error at %s: dimension exceeds 2^31-1\n", __FUNCTION__);
+        fprintf(stderr, "Error at %s: dimension exceeds 2^31-1\n", fn);
         exit(1);
     }
     const int m = (int)M, n = (int)N, k = (int)K;
@@ -340,12 +452,31 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
         hipLaunchKernelGGL(gemm_generic_kernel<float>, grd, blk, 0, current_stream, a, b, c, m, n, k,
                            transposeA ? 1L : (long)ldA, transposeA ? (long)ldA : 1L, transposeB ? 1L : (long)ldB,
                            transposeB ? (long)ldB : 1L, (long)ldC, alpha, beta);
-        check(hipGetLastError(), __FUNCTION__);
+        check(hipGetLastError(), fn);
         return 0;
     }
     if (skinny(m, n, k, vec_ok, transposeA)) {
         if (transposeB) dispatch_skinny<true>(a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta);
         else dispatch_skinny<false>(a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta);
+        return 0;
+    }
+    // few tiles, deep reduction: K split over workgroups through a scratch buffer
+    const splitk_plan plan = plan_splitk(m, n, k, SPLITK_WORKSPACE_LIMIT);
+    if (plan.chunks > 1) {
+        void *ws;
+        {
+            if (splitk_workspace_bytes < plan.scratch_bytes) {
+                if (splitk_workspace) {
+                    check(hipStreamSynchronize(current_stream), fn);
+                    check(hipFree(splitk_workspace), fn);
+                }
+                check(hipMalloc(&splitk_workspace, plan.scratch_bytes), fn);
+                splitk_workspace_bytes = plan.scratch_bytes;
+            }
+            ws = splitk_workspace;
+        }
+        const bool edge = !(vec_ok && m % SPLITK_TILE == 0 && n % SPLITK_TILE == 0 && plan.chunk % 32 == 0 && k % plan.chunk == 0);
+        dispatch_splitk(plan, transposeA, transposeB, edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok, ws);
         return 0;
     }
     const int bm = tile_for(m, n);
@@ -356,6 +487,12 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
     else if (transposeA && !transposeB) dispatch_edge<false, false>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
     else dispatch_edge<false, true>(edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok);
     return 0;
+}
+
+int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                       uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
+                       bool transposeA, bool transposeB) {
+    return sgemm_impl(__FUNCTION__, A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, offsetA, offsetB, offsetC, transposeA, transposeB);
 }
 
 int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha, double beta,
