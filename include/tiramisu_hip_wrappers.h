@@ -54,6 +54,21 @@ int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uin
 int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha,
                        double beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
                        uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
+/* tiramisu_hip_sgemm for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments,
+ * same kernels, bit-identical results; the difference is where deep reductions (at most 128 tiles of
+ * 64x64 and K >= 2048, whose K range is split over workgroups) keep their partial tiles and per-tile
+ * counters: tiramisu_hip_sgemm takes them from a per-thread workspace that it allocates and grows with
+ * hipMalloc, this entry point from a 4 MiB (+512 B of counters) array that lives in the library's code
+ * object, one copy per GPU, held until the process ends.  It calls no hipMalloc / hipFree.  A problem
+ * whose split needs more than the array holds (tiles x chunks x 16 KiB: e.g. 640 x 640 x 4096, 300
+ * partial tiles) is refused: a message on stderr, return value 1, nothing launched -- the one case in
+ * this library where a failure returns instead of ending the process.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race; serialise them.  The counters
+ * are cleared by a small kernel before every use.  Returns 0 on success. */
+int tiramisu_hip_sgemm_static_scratch(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
+                                      float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
+                                      uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
 
 /* ---- code objects and launches.  The reference links nvcc-compiled kernel wrappers
  *      (_kernel_N_wrapper, tiramisu_codegen_cuda.cpp:1288-1318) into the program; here

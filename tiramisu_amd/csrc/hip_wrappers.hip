@@ -327,6 +327,24 @@ thread_local void *splitk_workspace = nullptr;
 thread_local uint64_t splitk_workspace_bytes = 0;
 constexpr uint64_t SPLITK_WORKSPACE_LIMIT = (uint64_t)256 << 20;
 
+// Scratch of the entry point that allocates nothing: lives in the code object, one copy per device.
+constexpr uint64_t STATIC_SCRATCH_BYTES = ((uint64_t)4 << 20) + SPLITK_COUNTER_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+std::mutex static_scratch_mutex;
+std::map<int, void *> static_scratch_of_device;      // device -> address of its copy of `scratch`
+
+void *static_scratch_here() {
+    int device = 0;
+    check(hipGetDevice(&device), "tiramisu_hip_sgemm_static_scratch");
+    std::lock_guard<std::mutex> g(static_scratch_mutex);
+    auto it = static_scratch_of_device.find(device);
+    if (it != static_scratch_of_device.end()) return it->second;
+    void *ptr = nullptr;
+    check(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "tiramisu_hip_sgemm_static_scratch");
+    static_scratch_of_device[device] = ptr;
+    return ptr;
+}
+
 template <bool AK, bool BK_>
 void dispatch_edge(bool edge, const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb,
                    long ldc, float alpha, float beta, bool vec_ok) {
@@ -430,7 +448,9 @@ int32_t tiramisu_hip_stream_synchronize(int32_t) {
     return 0;
 }
 
-static int sgemm_impl(const char *fn, float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
+// Shared by the two single-precision entry points.  `static_scratch`: deep reductions take their scratch
+// from the code object's static array and nothing is allocated; else from the calling thread's workspace.
+static int sgemm_impl(const char *fn, bool static_scratch, float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
                       float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
                       bool transposeA, bool transposeB) {
     if (ldA == 0) ldA = transposeA ? M : K;
@@ -464,7 +484,15 @@ static int sgemm_impl(const char *fn, float *A, float *B, float *C, uint64_t M, 
     const splitk_plan plan = plan_splitk(m, n, k, SPLITK_WORKSPACE_LIMIT);
     if (plan.chunks > 1) {
         void *ws;
-        {
+        if (static_scratch) {
+            if (plan.scratch_bytes > STATIC_SCRATCH_BYTES) {
+                fprintf(stderr, "Error at %s: %d x %d x %d needs %llu bytes of scratch for its %d K chunks of %d tiles, the static array holds %llu; "
+                                "use tiramisu_hip_sgemm (which allocates) for this size\n", fn, m, n, k, (unsigned long long)plan.scratch_bytes,
+                        plan.chunks, plan.tiles, (unsigned long long)STATIC_SCRATCH_BYTES);
+                return 1;
+            }
+            ws = static_scratch_here();
+        } else {
             if (splitk_workspace_bytes < plan.scratch_bytes) {
                 if (splitk_workspace) {
                     check(hipStreamSynchronize(current_stream), fn);
@@ -492,7 +520,13 @@ static int sgemm_impl(const char *fn, float *A, float *B, float *C, uint64_t M, 
 int tiramisu_hip_sgemm(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
                        uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
                        bool transposeA, bool transposeB) {
-    return sgemm_impl(__FUNCTION__, A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, offsetA, offsetB, offsetC, transposeA, transposeB);
+    return sgemm_impl(__FUNCTION__, false, A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, offsetA, offsetB, offsetC, transposeA, transposeB);
+}
+
+int tiramisu_hip_sgemm_static_scratch(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha, float beta,
+                                      uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
+                                      bool transposeA, bool transposeB) {
+    return sgemm_impl(__FUNCTION__, true, A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, offsetA, offsetB, offsetC, transposeA, transposeB);
 }
 
 int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha, double beta,

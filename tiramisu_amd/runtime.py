@@ -108,6 +108,7 @@ def wrappers():
         u64 = ctypes.c_uint64
         lib.tiramisu_hip_sgemm.argtypes = [ctypes.c_void_p] * 3 + [u64] * 3 + [ctypes.c_float] * 2 + \
             [u64] * 6 + [ctypes.c_bool] * 2
+        lib.tiramisu_hip_sgemm_static_scratch.argtypes = lib.tiramisu_hip_sgemm.argtypes
         lib.tiramisu_hip_dgemm.argtypes = [ctypes.c_void_p] * 3 + [u64] * 3 + [ctypes.c_double] * 2 + \
             [u64] * 6 + [ctypes.c_bool] * 2
         _wrappers = lib
