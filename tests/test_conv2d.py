@@ -42,6 +42,25 @@ def make_inputs(s, seed, integer):
     return xp, w, b
 
 
+def kernel_descriptions(s):
+    lib = os.path.join(PROGRAMS, "build", "lib%s.so" % name_of(s))
+    return [k["how"] for k in runtime.manifest_of(lib, name_of(s))["kernels"]]
+
+
+def test_which_kernel_each_shape_gets():
+    """The benchmark shape and the small shape with whole tiles take the sliding-window kernel (input staged in LDS
+    by channel blocks); the benchmark's 1568 tiles do not divide by the 512 resident workgroups, so its last 32 tiles
+    are cut into pieces.  The ragged shapes take the gathering kernel."""
+    full, = kernel_descriptions((32, 64, 64, 112))
+    assert "sliding window of 9 taps staged in LDS by blocks of 8 channels" in full
+    assert "take tiles from a queue, the last tiles cut into 8 pieces" in full
+    small, = kernel_descriptions((2, 8, 64, 16))
+    assert "sliding window of 9 taps" in small and "cut into" not in small
+    for s in [(1, 3, 5, 12), (3, 4, 32, 8)]:
+        how, = kernel_descriptions(s)
+        assert "gathered operand" in how and "guarded edges" in how
+
+
 # ---------------------------------------------------------------- oracle pins
 
 def test_oracle_matches_seven_loops():

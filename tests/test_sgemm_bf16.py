@@ -15,7 +15,7 @@ from tiramisu_amd import runtime
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
-SMALL = [(128, 192, 128), (48, 40, 24), (1024, 1280, 512)]
+SMALL = [(128, 192, 128), (48, 40, 24), (200, 150, 100), (1024, 1280, 512)]
 RTOL = 2e-2
 
 
@@ -47,6 +47,17 @@ def test_bf16_rounding_helper():
     assert to_bf16(tie)[0] == 0x3F80
     tie2 = np.array([0x3F818000], np.uint32).view(np.float32)
     assert to_bf16(tie2)[0] == 0x3F82
+
+
+@pytest.mark.parametrize("M,N,K,what", [(128, 192, 128, "tile 64x64x64, whole tiles"), (48, 40, 24, "tile 64x64x64, guarded edges"),
+                                        (200, 150, 100, "tile 64x64x64, guarded edges"), (1024, 1280, 512, "tile 128x128x32, whole tiles"),
+                                        (4096, 4096, 4096, "tile 256x256x32, whole tiles")])
+def test_every_shape_gets_the_bf16_mfma_kernel(M, N, K, what):
+    """Ragged shapes and unaligned rows take the 64x64 tile with guarded loads instead of falling back
+    to the schedule-faithful (VALU) kernel."""
+    import json
+    kernels = json.load(open(os.path.join(PROGRAMS, "build", name_of(M, N, K) + ".o.json")))["kernels"]
+    assert len(kernels) == 1 and "v_mfma_f32_32x32x16_bf16" in kernels[0]["how"] and what in kernels[0]["how"]
 
 
 @pytest.mark.parametrize("M,N,K", SMALL)

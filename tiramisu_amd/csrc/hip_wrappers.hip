@@ -19,6 +19,7 @@
 
 #include "../../include/tiramisu_hip_wrappers.h"
 #include "kernels/gemm_mfma.hip.h"
+#include "kernels/target_gfx950.h"
 
 namespace {
 
@@ -163,23 +164,8 @@ void launch_mfma(const float *A, const float *B, float *C, int M, int N, int K, 
     check(hipGetLastError(), "tiramisu_hip_sgemm");
 }
 
-// The square C tile whose launch is modelled fastest: a compute unit works through
-// ceil(tiles / 256) tiles, each costing its area over the share of the MFMA rate that a tile of
-// that size sustains.  256 and 192 are for whole tiles only (3072 = 16 x 192: one per unit).
-int tile_for(int M, int N) {
-    struct candidate { int tile; double rate; bool whole_only; };
-    const candidate cands[] = {{256, 1.0, true}, {192, 0.9, true}, {128, 0.8, false}, {64, 0.68, false}};
-    double best = 0;
-    int tile = 64;
-    for (const candidate &c : cands) {
-        if (c.whole_only && (M % c.tile != 0 || N % c.tile != 0)) continue;
-        if (c.tile == 128 && M < 128) continue;
-        const long tiles = (long)((M + c.tile - 1) / c.tile) * ((N + c.tile - 1) / c.tile);
-        const double cost = (double)((tiles + 255) / 256) * c.tile * c.tile / c.rate;
-        if (best == 0 || cost < best) { best = cost; tile = c.tile; }
-    }
-    return tile;
-}
+// The square C tile whose launch is modelled fastest on this machine.
+int tile_for(int M, int N) { return ttarget::square_tile_for(M, N); }
 
 template <bool AK, bool BK_, bool EDGE>
 void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K, long lda, long ldb, long ldc,
@@ -201,7 +187,7 @@ void dispatch_tile(const float *A, const float *B, float *C, int M, int N, int K
 // cells): 64x32 tiles, 8 groups of wavefronts share the K range of each tile and reduce through
 // LDS, and up to four K-slices are requested ahead (the launch is latency-bound).
 bool skinny(int M, int N, int K, bool vec_ok, bool transposeA) {
-    return !transposeA && vec_ok && M == 64 && (N + 63) / 64 <= 64 && N % 32 == 0 && K % 128 == 0 && K >= 256;
+    return !transposeA && vec_ok && M == 64 && (N + 63) / 64 <= ttarget::COMPUTE_UNITS / 4 && N % 32 == 0 && K % 128 == 0 && K >= 256;
 }
 
 template <bool BK_>
@@ -248,25 +234,35 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_splitk_kernel(const float *__re
     tgemm::f32x4 *mine = reinterpret_cast<tgemm::f32x4 *>(partial) + ((long)blockIdx.x * Z + z) * 4 * CFG::NT;
 #pragma unroll
     for (int r = 0; r < 4; r++)
-        mine[r * CFG::NT + threadIdx.x] = tgemm::f32x4{acc.t[0][0][4 * r], acc.t[0][0][4 * r + 1], acc.t[0][0][4 * r + 2], acc.t[0][0][4 * r + 3]};
-    __threadfence();                       // the partial tile is visible device-wide before the ticket is taken
+        tgemm::store_handed_over(mine + r * CFG::NT + threadIdx.x, tgemm::f32x4{acc.t[0][0][4 * r], acc.t[0][0][4 * r + 1], acc.t[0][0][4 * r + 2], acc.t[0][0][4 * r + 3]});
+    tgemm::handed_over_stores_done();      // the partial tile is in memory before the ticket is taken
     __syncthreads();
     if (threadIdx.x == 0) ticket = atomicAdd(&counters[blockIdx.x], 1u);
     __syncthreads();
     if (ticket != (unsigned)(Z - 1)) return;
-    __threadfence();                       // and the other workgroups' tiles are visible to this one
+    tgemm::handed_over_loads_begin();
     const tgemm::f32x4 *all = reinterpret_cast<const tgemm::f32x4 *>(partial) + (long)blockIdx.x * Z * 4 * CFG::NT;
+    // four chunks' partial tiles are requested before the first is added (one round trip to memory per four
+    // chunks); they are added in chunk order, whichever workgroup arrives last
+    tgemm::f32x4 sum[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int c0 = 0; c0 < Z; c0 += 4) {
+        tgemm::f32x4 part[4][4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        tgemm::f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int c = 0; c < Z; c++) {
-            sum += all[((long)c * 4 + r) * CFG::NT + threadIdx.x];
-        }
+        for (int cc = 0; cc < 4; cc++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) acc.t[0][0][4 * r + e] = sum[e];
+            for (int r = 0; r < 4; r++)
+                if (c0 + cc < Z) part[cc][r] = tgemm::load_handed_over(all + ((long)(c0 + cc) * 4 + r) * CFG::NT + threadIdx.x);
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                if (c0 + cc < Z) sum[r] += part[cc][r];
     }
-    tgemm::axpby_epilogue epi{C, ldc, alpha, beta};
-    tgemm::tile_epilogue<CFG>(acc, M, N, tm * CFG::BM, tn * CFG::BN, epi);
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc.t[0][0][4 * r + e] = sum[r][e];
+    tgemm::tile_epilogue<CFG>(acc, M, N, tm * CFG::BM, tn * CFG::BN, tgemm::axpby_value{C, ldc, alpha, beta}, tgemm::axpby_store{C, ldc});
     if (threadIdx.x == 0) counters[blockIdx.x] = 0;     // ready for the next launch
 }
 
@@ -286,7 +282,7 @@ splitk_plan plan_splitk(int M, int N, int K, uint64_t max_bytes) {
     p.tiles = ((M + SPLITK_TILE - 1) / SPLITK_TILE) * ((N + SPLITK_TILE - 1) / SPLITK_TILE);
     if (p.tiles > SPLITK_MAX_TILES || K < 2048) return p;
     // enough workgroups for every compute unit, at least 512 of K each
-    int chunks = std::min((256 + p.tiles - 1) / p.tiles, K / 512);
+    int chunks = std::min((ttarget::COMPUTE_UNITS + p.tiles - 1) / p.tiles, K / 512);
     const uint64_t per_chunk = (uint64_t)p.tiles * SPLITK_TILE * SPLITK_TILE * sizeof(float);
     while (chunks > 1 && per_chunk * chunks + SPLITK_COUNTER_BYTES > max_bytes) chunks--;
     if (chunks < 2) return p;
@@ -585,7 +581,7 @@ void *tiramisu_hip_module_get_global(void *module, const char *name, uint64_t by
 int tiramisu_hip_launch(void *function, const uint32_t grid[3], const uint32_t block[3], uint32_t dynamic_lds_bytes,
                         void **args) {
     if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return 0;  // empty iteration space
-    if ((uint64_t)block[0] * block[1] * block[2] > 1024) {
+    if ((uint64_t)block[0] * block[1] * block[2] > (uint64_t)ttarget::MAX_THREADS_PER_WORKGROUP) {
         fprintf(stderr, "Error at %s: thread block %ux%ux%u exceeds 1024 threads\n", __FUNCTION__, block[0], block[1], block[2]);
         exit(1);
     }

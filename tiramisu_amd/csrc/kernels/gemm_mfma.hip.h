@@ -28,12 +28,40 @@
 #include <stdint.h>
 #include <type_traits>
 
+#include "target_gfx950.h"
+
 namespace tgemm {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));   // 4-byte aligned 16-byte load
+
+// Data handed from one workgroup to another within a launch (partial tiles of a reduction cut over workgroups):
+// written through to memory and read from there, as agent-scope atomic accesses of 8 bytes.  The compute dies of
+// the GPU have an L2 cache each, so ordinary stores would need the writer's whole L2 written back (what an
+// agent-scope release fence does) and the reader's invalidated; with these accesses the writer only has to wait
+// for its own stores (handed_over_stores_done) before it announces them with an atomic counter, and the reader,
+// once it has seen the counter, reads what the writers wrote.
+__device__ __forceinline__ void store_handed_over(f32x4 *p, f32x4 v) {
+    typedef unsigned long long u64;
+    union { f32x4 v; u64 u[2]; } x;
+    x.v = v;
+    __hip_atomic_store(reinterpret_cast<u64 *>(p), x.u[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(reinterpret_cast<u64 *>(p) + 1, x.u[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 load_handed_over(const f32x4 *p) {
+    typedef unsigned long long u64;
+    union { f32x4 v; u64 u[2]; } x;
+    u64 *q = reinterpret_cast<u64 *>(const_cast<f32x4 *>(p));
+    x.u[0] = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    x.u[1] = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return x.v;
+}
+// every store_handed_over of this wavefront has reached memory when this returns
+__device__ __forceinline__ void handed_over_stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+// no load_handed_over is moved ahead of this point (placed behind the counter's read)
+__device__ __forceinline__ void handed_over_loads_begin() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
 // An operand stored with one unit stride: element (x, k) lives at base[x*ld + k] (KMAJOR) or
 // base[k*ld + x].  With EDGE, elements outside XE x KE read as zero and rows need not be
@@ -147,7 +175,7 @@ struct operand_tile {
 __device__ __forceinline__ void tile_of_block(int tiles_m, int tiles_n, int &tm, int &tn) {
     const int total = tiles_m * tiles_n;
     int id = blockIdx.x;
-    constexpr int XCDS = 8;
+    constexpr int XCDS = ttarget::XCDS;
     if (total % XCDS == 0) id = (id % XCDS) * (total / XCDS) + id / XCDS;
     constexpr int GROUP = 8;
     const int per_group = GROUP * tiles_n;
@@ -404,26 +432,61 @@ __device__ __forceinline__ void tile_epilogue(const accumulators<CFG> &acc, int 
             }
 }
 
-template <class CFG, class EPI>
+// The epilogue in two passes: value(row, column, sum) returns what the element's store will write (it may read
+// memory), store(row, column, v) writes it.  Loads and stores are counted by one in-order counter (vmcnt): a load
+// issued behind a store can only be waited for together with that store's acknowledgement, so a tile whose
+// elements load and store in turn pays a round trip to memory per element.  Here the values of a group of
+// accumulator tiles (64 elements per lane: what the loads of the first pass may keep in registers) are all
+// computed before the group's first store is issued: one round trip per group.
+template <class CFG, class VALUE, class STORE>
+__device__ __forceinline__ void tile_epilogue(accumulators<CFG> &acc, int M, int N, int m0, int n0, VALUE value, STORE store) {
+    const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % (CFG::WGM * CFG::WGN);
+    const int wm = wave / CFG::WGN, wn = wave % CFG::WGN;
+    const int l32 = lane & 31, h = lane >> 5;
+    constexpr int TILES = CFG::TM * CFG::TN, GROUP = 4;
+#pragma unroll
+    for (int g0 = 0; g0 < TILES; g0 += GROUP)
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+            for (int g = g0; g < g0 + GROUP && g < TILES; g++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int i = g / CFG::TN, j = g % CFG::TN;
+                    const int row = m0 + wm * CFG::WM + i * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+                    const int col = n0 + wn * CFG::WN + j * 32 + l32;
+                    if (!CFG::EDGE || (row < M && col < N)) {
+                        if (pass == 0) acc.t[i][j][r] = value(row, col, acc.t[i][j][r]);
+                        else store(row, col, acc.t[i][j][r]);
+                    }
+                }
+}
+
+template <class CFG, class VALUE, class STORE>
 __device__ __forceinline__ void tile_mainloop(const float *__restrict__ A, long lda, const float *__restrict__ B,
                                               long ldb, int M, int N, int K, int m0, int n0, bool vec_ok,
-                                              float *lds, EPI epi) {
+                                              float *lds, VALUE value, STORE store) {
     accumulators<CFG> acc;
     acc.clear();
     linear_source<CFG::A_KMAJOR, CFG::EDGE> sa{A, lda, M, K, vec_ok};
     linear_source<CFG::B_KMAJOR, CFG::EDGE> sb{B, ldb, N, K, vec_ok};
     tile_accumulate<CFG>(acc, sa, sb, K, m0, n0, lds);
-    if (tile_reduce_k<CFG>(acc, lds)) tile_epilogue<CFG>(acc, M, N, m0, n0, epi);
+    if (tile_reduce_k<CFG>(acc, lds)) tile_epilogue<CFG>(acc, M, N, m0, n0, value, store);
 }
 
-struct axpby_epilogue {
-    float *C;
+// C = alpha * sum + beta * C as the two passes of tile_epilogue
+struct axpby_value {
+    const float *C;
     long ldc;
     float alpha, beta;
-    __device__ __forceinline__ void operator()(int row, int col, float v) const {
-        float *p = C + (long)row * ldc + col;
-        *p = (beta == 0.f) ? alpha * v : alpha * v + beta * *p;
+    __device__ __forceinline__ float operator()(int row, int col, float v) const {
+        return (beta == 0.f) ? alpha * v : alpha * v + beta * C[(long)row * ldc + col];
     }
+};
+struct axpby_store {
+    float *C;
+    long ldc;
+    __device__ __forceinline__ void operator()(int row, int col, float v) const { C[(long)row * ldc + col] = v; }
 };
 
 template <class CFG>
@@ -433,8 +496,8 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_kernel(const float *__restrict_
     extern __shared__ __attribute__((aligned(16))) float lds[];
     int tm, tn;
     tile_of_block((M + CFG::BM - 1) / CFG::BM, (N + CFG::BN - 1) / CFG::BN, tm, tn);
-    axpby_epilogue epi{C, ldc, alpha, beta};
-    tile_mainloop<CFG>(A, lda, B, ldb, M, N, K, tm * CFG::BM, tn * CFG::BN, vec_ok != 0, lds, epi);
+    tile_mainloop<CFG>(A, lda, B, ldb, M, N, K, tm * CFG::BM, tn * CFG::BN, vec_ok != 0, lds, axpby_value{C, ldc, alpha, beta},
+                       axpby_store{C, ldc});
 }
 
 }  // namespace tgemm

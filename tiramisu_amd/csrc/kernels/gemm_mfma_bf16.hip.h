@@ -15,8 +15,10 @@
 //     write every fourth column) and keeps the reads conflict-free.
 //   * Row m of k-group kq of A sits at position m ^ swz(kq) for the same reason (the lanes that
 //     store the k-groups of one row are 4096 bytes apart).
-// Whole tiles only: M % BM == 0, N % BN == 0, K % BK == 0, rows of A 16-byte and rows of B 8-byte
-// aligned (the emitter checks).  Large tiles use the second variant further down
+// With EDGE the tile may hang over the M x N x K problem and rows need not be aligned: loads outside
+// read as zero (element loads where a 16-byte / 8-byte piece is not whole or not aligned), and the
+// epilogue skips elements outside.  Without it: M % BM == 0, N % BN == 0, K % BK == 0, rows of A 16-byte
+// and rows of B 8-byte aligned (the emitter checks).  Large tiles use the second variant further down
 // (tile_accumulate_bf16_direct: slices loaded straight into an LDS ring); this one serves 64x64 tiles.
 #ifndef TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
 #define TIRAMISU_AMD_GEMM_MFMA_BF16_HIP_H
@@ -28,10 +30,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2), aligned(4)));
 
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
+template <int BM_, int BN_, int BK_, int WGM_, int WGN_, bool EDGE_ = false>
 struct config_bf16 {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WGM = WGM_, WGN = WGN_;
-    static constexpr bool EDGE = false;
+    static constexpr bool EDGE = EDGE_;
     static constexpr int NT = 64 * WGM * WGN;
     static constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
     static constexpr int A_WORDS = (BK / 8) * BM * 4;    // 32-bit words per stage
@@ -47,8 +49,11 @@ struct config_bf16 {
 
 template <class CFG>
 __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, const uint16_t *__restrict__ A, long lda,
-                                                     const uint16_t *__restrict__ B, long ldb, int K, int m0, int n0,
+                                                     const uint16_t *__restrict__ B, long ldb, int M, int N, int K, int m0, int n0,
                                                      uint32_t *lds) {
+    // whole 16-byte pieces of A / 8-byte pieces of B may be loaded as such
+    const bool vec_a = !CFG::EDGE || ((lda % 8 == 0) && ((uintptr_t)A % 16 == 0));
+    const bool vec_b = !CFG::EDGE || ((ldb % 4 == 0) && ((uintptr_t)B % 8 == 0));
     constexpr int TM = CFG::TM, TN = CFG::TN, BK = CFG::BK, BM = CFG::BM, BN = CFG::BN, NT = CFG::NT;
     constexpr int NVA = CFG::NVA, NVB = CFG::NVB;
     constexpr int Q = BK / 16;                      // MFMA steps (fragment sets) per slice
@@ -71,7 +76,15 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
 #pragma unroll
         for (int v = 0; v < NVA; v++) {
             const int idx = t + NT * v, kq = idx % (BK / 8), m = idx / (BK / 8);
-            ra[v] = *reinterpret_cast<const u32x4 *>(A + (long)(m0 + m) * lda + k0 + 8 * kq);
+            const uint16_t *p = A + (long)(m0 + m) * lda + k0 + 8 * kq;
+            if (!CFG::EDGE || (vec_a && m0 + m < M && k0 + 8 * kq + 7 < K)) {
+                ra[v] = *reinterpret_cast<const u32x4 *>(p);
+            } else {
+                uint16_t e[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) e[i] = (m0 + m < M && k0 + 8 * kq + i < K) ? p[i] : (uint16_t)0;
+                ra[v] = u32x4{e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16), e[4] | ((uint32_t)e[5] << 16), e[6] | ((uint32_t)e[7] << 16)};
+            }
         }
     };
     auto col_pos = [](int n) -> int { return n ^ ((n >> 3) & 7); };
@@ -82,7 +95,16 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
             if (CFG::UNITS_B % NT == 0 || idx < CFG::UNITS_B) {
                 const uint16_t *p = B + (long)(k0 + 8 * kq) * ldb + n0 + 4 * n4;
 #pragma unroll
-                for (int i = 0; i < 8; i++) rb[v][i] = *reinterpret_cast<const u32x2 *>(p + i * ldb);
+                for (int i = 0; i < 8; i++) {
+                    if (!CFG::EDGE || (vec_b && k0 + 8 * kq + i < K && n0 + 4 * n4 + 3 < N)) {
+                        rb[v][i] = *reinterpret_cast<const u32x2 *>(p + i * ldb);
+                    } else {
+                        uint16_t e[4];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) e[c] = (k0 + 8 * kq + i < K && n0 + 4 * n4 + c < N) ? p[i * ldb + c] : (uint16_t)0;
+                        rb[v][i] = u32x2{e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16)};
+                    }
+                }
             }
         }
     };
@@ -140,7 +162,7 @@ __device__ __forceinline__ void tile_accumulate_bf16(accumulators<CFG> &acc, con
     // loads of the slice after it; the barrier sits before the last set, whose matrix instructions
     // cover the first fragment reads of the next slice.  Memory instructions are dealt out between
     // the matrix instructions with scheduling groups.
-    const int KT = K / BK;
+    const int KT = CFG::EDGE ? (K + BK - 1) / BK : K / BK;
     load_a(0);
     load_b(0);
     store_a(0);

@@ -48,6 +48,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "target_gfx950.h"
+
 #define ST_HY (ST_R * ST_RAD)                       /* halo rows */
 #define ST_HX ((ST_R * ST_RAD + 3) / 4 * 4)         /* halo columns, multiple of 4 */
 #define ST_LH (ST_W * ST_RPT)
@@ -261,8 +263,9 @@ ST_NAME(float *__restrict__ planes, const int src_plane)
     constexpr int IW = ST_IBX1 - ST_IBX0 + 1;
     constexpr int nb = ST_NI;
 #if ST_XCD
-    const int xcd = b % 8, per = nb / 8, extra = nb % 8;
-    const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / 8;
+    constexpr int XCDS = ttarget::XCDS;
+    const int xcd = b % XCDS, per = nb / XCDS, extra = nb % XCDS;
+    const int tile = xcd * per + (xcd < extra ? xcd : extra) + b / XCDS;
 #else
     const int tile = b;
 #endif

@@ -3,11 +3,13 @@
 // domains and store relations, with isl where sets and maps are compared -- that the nest is of
 // its kind, and only then replaces it by kernels shaped for gfx950.  Anything that fails a check
 // falls back to the generic emitter, which reproduces the reference's behaviour.
+#include <algorithm>
 #include <cstdlib>
 #include <sstream>
 
 #include "hip_backend.h"
 #include <tiramisu/isl_api.h>
+#include "kernels/target_gfx950.h"
 #include "util.h"
 
 namespace tiramisu {
@@ -1032,27 +1034,16 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     if (lit) {
         if (Ml <= 64 && Nl >= 256 * 256) { BM = 64; BN = 256; WGM = 1; WGN = 4; }   // short, very wide (convolutions)
         else {
-            // square tiles: the one whose launch is modelled fastest.  A compute unit works through
-            // ceil(tiles / 256) tiles, each costing its area over the fraction of the MFMA rate that
-            // a tile of that size sustains (larger tiles re-read less through LDS).  256 and 192
-            // are for whole tiles only; 192 is what makes 3072 = 16 x 192 one tile per compute unit.
-            struct candidate { int tile; double rate; bool whole_only; };
-            const candidate cands[] = {{256, 1.0, true}, {192, 0.9, true}, {128, 0.8, false}, {64, 0.68, false}};
-            double best = 0;
-            for (const candidate &c : cands) {
-                if (c.whole_only && (Ml % c.tile != 0 || Nl % c.tile != 0)) continue;
-                if (c.tile == 128 && Ml < 128) continue;
-                const long tiles = ((Ml + c.tile - 1) / c.tile) * ((Nl + c.tile - 1) / c.tile);
-                const double cost = (double)((tiles + 255) / 256) * c.tile * c.tile / c.rate;
-                if (best == 0 || cost < best) { best = cost; BM = BN = c.tile; }
-            }
+            // square tiles: the one whose launch is modelled fastest on this machine (kernels/target_gfx950.h);
+            // 192 is what makes 3072 = 16 x 192 one tile per compute unit
+            BM = BN = ttarget::square_tile_for(Ml, Nl);
             PADX = BM == 256 ? 0 : 1;
         }
     }
     if (BM == 64 && BN == 64) BK = 32;   // one 32x32 tile per wavefront: longer slices, fewer barriers per flop
     // few C tiles but a long reduction (a batch-sized M against wide weights, as in recurrent cells):
     // 64x32 tiles, and 8 groups of wavefronts share the K range of each tile
-    if (lit && !bf16 && BM == 64 && BN == 64 && Ml <= 64 && ((Nl + 63) / 64) <= 64 && Nl % 32 == 0 && Kl % 128 == 0 && Kl >= 256 &&
+    if (lit && !bf16 && BM == 64 && BN == 64 && Ml <= 64 && ((Nl + 63) / 64) <= ttarget::COMPUTE_UNITS / 4 && Nl % 32 == 0 && Kl % 128 == 0 && Kl >= 256 &&
         !std::getenv("TIRAMISU_MFMA_NO_SPLITK")) {
         BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
         DEPTH = (int)std::min<long>(4, std::max<long>(1, Kl / BK - 1));   // latency-bound: ask for (up to) all slices at once
@@ -1064,7 +1055,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     // at most one 64x64 tile per compute unit and a long reduction: two groups of wavefronts share each
     // (64-k) slice, so that every SIMD has two wavefronts to alternate between (1024^3: 20.6 us against 21.9)
     if (lit && !bf16 && BM == 64 && BN == 64 && WGK == 1 && Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0 && Kl >= 512 &&
-        (Ml / 64) * (Nl / 64) <= 256) {
+        (Ml / 64) * (Nl / 64) <= ttarget::COMPUTE_UNITS) {
         WGK = 2; BK = 64;
     }
     if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
@@ -1076,29 +1067,36 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     if (const char *e = std::getenv("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
     if (const char *e = std::getenv("TIRAMISU_MFMA_WGK")) WGK = std::atoi(e);
+    bool bf16_edge = false;
     if (bf16) {
-        // whole tiles of the bf16 kernel only; anything else stays on the schedule-faithful emitter
-        if (!lit) return reject(24);
-        // 256x256 when that fills the chip, else 128x128 (both load their slices straight into LDS), else 64x64
-        if ((Ml / 256) * (Nl / 256) >= 192 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 32 == 0) { BM = BN = 256; BK = 32; }
-        else if (Ml % 128 == 0 && Nl % 128 == 0 && Kl % 32 == 0 && (Ml / 128) * (Nl / 128) >= 48) { BM = BN = 128; BK = 32; }
-        else if (Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0) { BM = BN = 64; BK = 64; }
-        else return reject(24);
-        WGM = WGN = 2;
+        // 256x256 when that fills the chip, else 128x128 (both load their slices straight into LDS and want whole
+        // tiles, 16-byte aligned rows and operands below 2 GiB), else 64x64 -- with guarded loads when tiles hang
+        // over the problem, sizes are known at run time only, or rows are not aligned
+        for (auto &o : operands)
+            if (!o.first.linear || !o.second.linear || !o.first.kmajor || o.second.kmajor) return reject(25);
+        bool aligned = true, small_enough = true;
         for (auto &o : operands) {
             long v;
-            if (!o.first.linear || !o.second.linear || !o.first.kmajor || o.second.kmajor) return reject(25);
             for (const operand_info *g : {&o.first, &o.second})
-                if (!literal_value(g->ld, v) || v % 8 != 0 || !literal_value(g->base, v) || v % 8 != 0) return reject(25);
-            // the large tiles address their operands with 32-bit byte offsets (buffer loads)
+                if (!literal_value(g->ld, v) || v % 8 != 0 || !multiple_of(g->base, 8)) aligned = false;
             long lda = 0, ldb = 0;
-            literal_value(o.first.ld, lda);
-            literal_value(o.second.ld, ldb);
-            if (BM >= 128 && ((double)Ml * lda * 2 >= 2147483648.0 || (double)Kl * ldb * 2 >= 2147483648.0)) { BM = BN = 64; BK = 64; }
+            if (lit && literal_value(o.first.ld, lda) && literal_value(o.second.ld, ldb)) {
+                if ((double)Ml * lda * 2 >= 2147483648.0 || (double)Kl * ldb * 2 >= 2147483648.0) small_enough = false;
+            } else {
+                small_enough = false;
+            }
         }
-        if (BM == 64 && Kl % 64 != 0) return reject(24);
+        WGM = WGN = 2;
+        if (lit && aligned && small_enough && (Ml / 256) * (Nl / 256) >= 3 * ttarget::COMPUTE_UNITS / 4 && Ml % 256 == 0 && Nl % 256 == 0 && Kl % 32 == 0) { BM = BN = 256; BK = 32; }
+        else if (lit && aligned && small_enough && Ml % 128 == 0 && Nl % 128 == 0 && Kl % 32 == 0 && (Ml / 128) * (Nl / 128) >= 3 * ttarget::COMPUTE_UNITS / 16) { BM = BN = 128; BK = 32; }
+        else {
+            BM = BN = 64;
+            BK = 64;
+            bf16_edge = !(lit && aligned && Ml % 64 == 0 && Nl % 64 == 0 && Kl % 64 == 0);
+        }
     }
     bool edge = !(lit && Ml % BM == 0 && Nl % BN == 0 && Kl % BK == 0);
+    if (bf16) edge = bf16_edge;
     for (auto &o : operands)
         for (const operand_info *g : {&o.first, &o.second}) {
             long v;
@@ -1113,6 +1111,85 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         if (BN % G != 0 || UB == 0 || UE % UB != 0 || Nl % BN != 0) return reject(35);
         for (auto &o : operands)
             if (!o.second.linear || (!o.second.kmajor && UB % 4 != 0)) return reject(35);
+    }
+
+    // ---- a gathered B operand that is a sliding window (the implicit GEMM of a convolution): k = (channel,
+    // taps...) with the channel outermost, offset = f(position) + channel * stride + tap offset.  When the piece
+    // of memory that a tile's positions and all taps touch per channel is short, blocks of channels are staged
+    // in LDS and the operand is read from there (kernels/gemm_mfma_window.hip.h); else the gather stays as it is.
+    bool windowed = false;
+    int win_cb = 0, win_taps = 0, win_floats = 0;
+    long win_chan_stride = 0, win_channels = 0, win_x_elements = 0;
+    std::vector<long> win_tap_offsets;
+    int win_splits = 1;                  // pieces that each tile of the last, incomplete round is cut into
+    long win_grid = 0, win_scratch_floats = 0, win_counters = 0;
+    int win_resident = 1;                // workgroups that share a compute unit
+    std::string window_call_head;
+    if (!bf16 && !with_consumer && lit && operands.size() == 1 && operands[0].first.linear && operands[0].first.kmajor &&
+        !operands[0].second.linear && GK.dims.size() >= 2 && GK.literal && GN.literal && Ml % BM == 0 && Nl % BN == 0 && WGK == 1 &&
+        !std::getenv("TIRAMISU_MFMA_NO_WINDOW")) {
+        const operand_info &xo = operands[0].second;
+        std::vector<long> ck, cn;
+        bool ok = true;
+        long v;
+        for (int p : GK.dims) { ok = ok && literal_value(xo.coef.at(p), v); ck.push_back(v); }
+        for (int p : GN.dims) { ok = ok && literal_value(xo.coef.at(p), v); cn.push_back(v); }
+        long base_lit = 0, lda_lit = 0, abase_lit = 0;
+        ok = ok && literal_value(xo.base, base_lit) && base_lit % 4 == 0 && literal_value(operands[0].first.ld, lda_lit) && lda_lit % 4 == 0 &&
+             literal_value(operands[0].first.base, abase_lit) && abase_lit % 4 == 0 && xo.buf->has_constant_extents();
+        if (ok && ck[0] % 4 == 0 && ck[0] > 0) {
+            win_channels = GK.ext[0];
+            win_chan_stride = ck[0];
+            win_taps = 1;
+            for (size_t d = 1; d < GK.dims.size(); d++) win_taps *= (int)GK.ext[d];
+            for (int t = 0; t < win_taps; t++) {
+                long off = 0, rest = t;
+                for (int d = (int)GK.dims.size() - 1; d >= 1; d--) { off += (rest % GK.ext[d]) * ck[d]; rest /= GK.ext[d]; }
+                if (off < 0) ok = false;
+                win_tap_offsets.push_back(off);
+            }
+            auto position_offset = [&](long pflat) {
+                long off = 0, rest = pflat;
+                for (int d = (int)GN.dims.size() - 1; d >= 0; d--) { off += (rest % GN.ext[d]) * cn[d]; rest /= GN.ext[d]; }
+                return off;
+            };
+            long need = 0;
+            const long max_tap = *std::max_element(win_tap_offsets.begin(), win_tap_offsets.end());
+            for (long n0 = 0; n0 < Nl && ok; n0 += BN) {
+                const long f0 = position_offset(n0) & ~3L;
+                for (long pp = n0; pp < n0 + BN; pp++) {
+                    const long fpos = position_offset(pp);
+                    if (fpos < f0) ok = false;              // positions must not run backwards within a tile
+                    need = std::max(need, fpos + max_tap - f0 + 1);
+                }
+            }
+            const int cb_max = env_int("TIRAMISU_MFMA_WINDOW_CB", 8);
+            for (int cb : {8, 4, 2})
+                if (win_cb == 0 && cb <= cb_max && win_channels % cb == 0 && (cb * win_taps) % 4 == 0) win_cb = cb;
+            win_floats = (int)((need + 31) / 64 * 64 + 32);      // = 32 mod 64: the two halves of a wavefront on disjoint banks
+            if (win_floats < need) win_floats += 64;
+            long cnt = 1;
+            for (auto &d : xo.buf->get_dim_sizes()) cnt *= lir::simplify(d).get_int_val();
+            win_x_elements = cnt - base_lit;
+            const long stage_bytes = ((long)win_cb * (win_taps * BM + 32) + (long)win_cb * win_floats) * 4;
+            windowed = ok && win_cb > 0 && win_taps <= 64 && (win_taps * BM) % 64 == 0 && 2 * stage_bytes + 64 <= ttarget::LDS_BYTES_PER_CU && cnt < 2147483648L;
+            if (windowed) {
+                // as many workgroups as the chip holds take tiles from a queue; the tiles left over after the last
+                // full round of the grid are cut along the channel blocks into short pieces that fill the end
+                const long tiles = (Ml / BM) * (Nl / BN), blocks = win_channels / win_cb;
+                // two workgroups per compute unit when their LDS fits: one's tile boundaries (epilogue stores, the wait
+                // for the first block) are covered by the other's matrix instructions
+                win_resident = 2 * (2 * stage_bytes + 64) <= ttarget::LDS_BYTES_PER_CU ? env_int("TIRAMISU_MFMA_WINDOW_RESIDENT", 2) : 1;
+                win_grid = std::min<long>(tiles, (long)ttarget::COMPUTE_UNITS * win_resident);
+                const long rest = tiles % win_grid;
+                if (rest > 0 && tiles > win_grid && !std::getenv("TIRAMISU_MFMA_NO_TAIL_SPLIT")) win_splits = (int)std::min<long>(std::min<long>(blocks, 2 * win_grid / rest), 16);
+                if (win_splits < 2) win_splits = 1;
+                // partial tiles of the pieces, a counter per remaining tile, the work queue's two counters
+                const long cut = win_splits > 1 ? rest : 0;
+                win_counters = cut + 2;
+                win_scratch_floats = cut * win_splits * BM * BN + win_counters;
+            }
+        }
     }
 
     // ---- kernel text
@@ -1130,7 +1207,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     // ---- the consumer's statements, once per point of the tile.  A value that the point itself stored
     // earlier is taken from its register instead of memory; a temporary of the function that nothing else
     // in the program reads is then not stored at all.
-    std::ostringstream consumer_text;
+    std::ostringstream consumer_text, consumer_loads_text;
     std::set<std::string> dead;                 // buffers whose stores are dropped
     if (with_consumer) {
         struct stmt { const buffer *lhs; std::vector<expr> idx; std::string value, decl; primitive_t type; };
@@ -1141,6 +1218,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         plain.fct = f;
         plain.device = true;
         std::set<int> groups_used;
+        std::vector<std::pair<std::string, expr>> hoisted;      // (variable, load) of what the points read from memory
         // an element as a text that is the same for every statement of a point: row and unit by their role,
         // outer dimensions by their value in terms of the host loops
         auto element_key = [&](size_t n, const buffer *b, const std::vector<expr> &index) {
@@ -1188,7 +1266,11 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
                     if (!never_the_same(w, n, x.get_access())) okx = false;
                 }
                 loaded.insert(x.get_name());
-                return x;
+                // what a point still reads from memory is read before any point of the thread stores (see below)
+                const std::string name = "_in" + std::to_string(hoisted.size());
+                hoisted.push_back({name, x.substitute(X.subs)});
+                locals.insert(name);
+                return var(x.get_data_type(), name);
             }).substitute(X.subs);
             if (!okx) return reject(36);
             stmt st;
@@ -1223,12 +1305,30 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
             if (!loaded.count(st.lhs->get_name()) && only_used_here(st.lhs)) dead.insert(st.lhs->get_name());
         if (only_used_here(acc_buf)) dead.insert(acc_buf->get_name());
         const std::string m_var = U.dims[Mg[0]].kvar;
+        // A thread handles _POINTS points.  Two passes: first everything the points read from memory (elements that
+        // no point of the launch stores, or the point's own before it stores it), then values and stores.  Loads and
+        // stores are counted by one in-order counter, so a point's load issued behind the previous point's stores
+        // would wait for those stores to be acknowledged: a round trip to memory per point instead of one in all.
+        std::ostringstream point;
+        point << "        const int _p = threadIdx.x + _i * CFG::NT;\n";
+        point << "        if (_p >= CFG::BM * " << UB << ") continue;\n";
+        point << "        const int _lr = _p / " << UB << ", _lu = _p % " << UB << ";\n";
+        if (edge) point << "        if (_tm * CFG::BM + _lr >= _M) continue;\n";
+        point << "        const int32_t " << m_var << " = _tm * CFG::BM + _lr + (" << dev.print(U.dims[Mg[0]].lo.substitute(U.subs)) << ");\n";
+        point << "        const int32_t _u = _tn * " << UB << " + _lu + (" << u_lo << ");\n";
+        // (the loads do not depend on the contraction: they are issued before it and arrive while it runs)
+        consumer_loads_text << "    constexpr int _POINTS = (CFG::BM * " << UB << " + CFG::NT - 1) / CFG::NT;\n";
+        for (auto &hl : hoisted)
+            consumer_loads_text << "    " << primitive_c_name(hl.second.get_data_type()) << " " << hl.first << "_of[_POINTS];\n";
+        if (!hoisted.empty()) {
+            consumer_loads_text << "#pragma unroll\n    for (int _i = 0; _i < _POINTS; _i++) {\n" << point.str();
+            for (auto &hl : hoisted) consumer_loads_text << "        " << hl.first << "_of[_i] = " << dev.print(hl.second) << ";\n";
+            consumer_loads_text << "    }\n";
+        }
         consumer_text << "    __syncthreads();\n";
-        consumer_text << "    for (int _p = threadIdx.x; _p < CFG::BM * " << UB << "; _p += CFG::NT) {\n";
-        consumer_text << "        const int _lr = _p / " << UB << ", _lu = _p % " << UB << ";\n";
-        if (edge) consumer_text << "        if (_tm * CFG::BM + _lr >= _M) continue;\n";
-        consumer_text << "        const int32_t " << m_var << " = _tm * CFG::BM + _lr + (" << dev.print(U.dims[Mg[0]].lo.substitute(U.subs)) << ");\n";
-        consumer_text << "        const int32_t _u = _tn * " << UB << " + _lu + (" << u_lo << ");\n";
+        consumer_text << "#pragma unroll\n    for (int _i = 0; _i < _POINTS; _i++) {\n" << point.str();
+        for (auto &hl : hoisted)
+            consumer_text << "        const " << primitive_c_name(hl.second.get_data_type()) << " " << hl.first << " = " << hl.first << "_of[_i];\n";
         for (int q : groups_used)
             consumer_text << "        const float _g" << q << " = _gt[_lr * (CFG::BN + 1) + " << q * UB << " + _lu];\n";
         for (auto &st : stmts) {
@@ -1273,14 +1373,14 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         body << "    extern __shared__ __attribute__((aligned(16))) uint32_t _lds[];\n";
         // large tiles: slices go straight from global memory into a four-stage LDS ring
         if (BM >= 128) body << "    typedef tgemm::config_bf16_direct<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << ", 4> CFG;\n";
-        else body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << "> CFG;\n";
+        else body << "    typedef tgemm::config_bf16<" << BM << ", " << BN << ", " << BK << ", " << WGM << ", " << WGN << ", " << (edge ? "true" : "false") << "> CFG;\n";
     } else {
         body << "    extern __shared__ __attribute__((aligned(16))) float _lds[];\n";
         body << "    typedef " << cfg << " CFG;\n";
     }
     body << "    const int _M = " << dev.print(Me) << ", _N = " << dev.print(Ne) << ", _K = " << dev.print(Ke) << ";\n";
     body << "    int _tm, _tn;\n    tgemm::tile_of_block((_M + CFG::BM - 1) / CFG::BM, (_N + CFG::BN - 1) / CFG::BN, _tm, _tn);\n";
-    body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n";
+    body << "    tgemm::accumulators<CFG> _acc;\n    _acc.clear();\n" << consumer_loads_text.str();
     int term = 0, ktab_words = 0;
     const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
     // several product terms over plain operands: one pipelined loop over the concatenated reduction ranges
@@ -1294,7 +1394,26 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
             used_buffers.insert(o.second.buf->get_name());
             body << "        tgemm::tile_accumulate_bf16" << (BM >= 128 ? "_direct" : "") << "<CFG>(_acc, " << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), "
                  << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + (" << dev.print(o.second.base) << "), " << dev.print(o.second.ld)
-                 << (BM >= 128 ? ", _M, _N" : "") << ", _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+                 << ", _M, _N, _K, _tm * CFG::BM, _tn * CFG::BN, _lds);\n    }\n";
+            term++;
+            continue;
+        }
+        if (windowed) {
+            used_buffers.insert(o.first.buf->get_name());
+            used_buffers.insert(o.second.buf->get_name());
+            pre << "struct " << kname << "_taps {\n    static __device__ __forceinline__ constexpr int at(int t) {\n        return ";
+            for (int t = 0; t + 1 < win_taps; t++) pre << "t == " << t << " ? " << win_tap_offsets[t] << " : ";
+            pre << win_tap_offsets[win_taps - 1] << ";\n    }\n};\n";
+            pre << "struct " << kname << "_pos {\n    __device__ __forceinline__ long operator()(int _x) const {\n" << digits(GN, "_x", "        ", false) << "        return 0";
+            for (int p : GN.dims) pre << " + (long)" << U.dims[p].kvar << " * " << dev.print(o.second.coef.at(p));
+            pre << ";\n    }\n};\n";
+            std::ostringstream call;
+            call << "    tgemm::contraction_window<CFG, " << win_cb << ", " << win_taps << ", " << win_floats << ", " << env_int("TIRAMISU_MFMA_WINDOW_AHEAD", 2) << ", " << win_splits << ", " << kname << "_taps>("
+                 << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), " << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + ("
+                 << dev.print(o.second.base) << "), " << win_x_elements << "L, " << kname << "_pos(), " << win_chan_stride << "L, " << win_channels
+                 << ", _M, _N, _tail_scratch, _lds, ";
+            window_call_head = call.str();
+            body << "    }\n";
             term++;
             continue;
         }
@@ -1376,50 +1495,81 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     }
     if (with_consumer)   // the finished tile, handed to the consumer's statements through LDS (behind the operand stages)
         body << "    float *_gt = _lds + CFG::LDS_BYTES / 4 + " << ktab_words << ";\n";
-    if (WGK > 1) body << "    if (tgemm::tile_reduce_k<CFG>(_acc, _lds))\n";
-    body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, [&](int _r, int _c, float _sum) {\n";
+    // The element-wise tail of a tile: `_accv` = initial value + sum, then the store of the accumulator element and/or of the
+    // fused epilogue's value.  With a single store the tail is printed as two functions, value and store, and
+    // tile_epilogue runs the first over the whole tile before the second: loads and stores are counted by one in-order
+    // counter, so a load behind a store can only be waited for together with that store's acknowledgement, and
+    // element-by-element the tile would pay one round trip to memory per element.
+    std::string digit_text;
     if (with_consumer) {
-        body << digits(GM, "_r", "        ", true);
-        body << "        const int _cq = tgemm::regrouped_index<CFG::BN, " << UB << ">(_c, " << UE << ");\n";
-        body << digits(GN, "_cq", "        ", true);
+        digit_text = digits(GM, "_r", "        ", true);
+        digit_text += "        const int _cq = tgemm::regrouped_index<CFG::BN, " + std::to_string(UB) + ">(_c, " + std::to_string(UE) + ");\n";
+        digit_text += digits(GN, "_cq", "        ", true);
     } else {
-        body << digits(GM, "_r", "        ", true) << digits(GN, "_c", "        ", true);
+        digit_text = digits(GM, "_r", "        ", true) + digits(GN, "_c", "        ", true);
     }
     std::vector<expr> acc_index;
     for (auto &e : U.leaf->lhs_index) acc_index.push_back(e.substitute(U.subs));
+    std::string accv_text;
     if (has_init) {
         expr init = cs[ii].leaf->rhs.substitute(cs[ii].subs);
         expr z = lir::simplify(init);
-        if (z.is_constant() && z.get_double_val() == 0.0) body << "        float _accv = _sum;\n";
-        else body << "        float _accv = " << dev.print(init) << " + _sum;\n";
+        if (z.is_constant() && z.get_double_val() == 0.0) accv_text = "        float _accv = _sum;\n";
+        else accv_text = "        float _accv = " + dev.print(init) + " + _sum;\n";
     } else {
-        body << "        float _accv = " << dev.element(acc_buf, acc_index) << " + _sum;\n";
+        accv_text = "        float _accv = " + dev.element(acc_buf, acc_index) + " + _sum;\n";
     }
-    if (!acc_private && !dead.count(acc_buf->get_name()) &&
-        !(has_epi && cs[ei].leaf->lhs == acc_buf && same_element(expr(o_access, acc_buf->get_name(), leaves[ei]->lhs_index, p_float32), acc_buf, ureal->lhs_index)))
-        body << "        " << dev.store(acc_buf, acc_index, "_accv", p_float32) << "\n";
-    if (with_consumer) body << "        _gt[(_r - _tm * CFG::BM) * (CFG::BN + 1) + (_c - _tn * CFG::BN)] = _accv;\n";
+    if (with_consumer) accv_text += "        _gt[(_r - _tm * CFG::BM) * (CFG::BN + 1) + (_c - _tn * CFG::BN)] = _accv;\n";
+    const bool acc_stored = !acc_private && !dead.count(acc_buf->get_name()) &&
+        !(has_epi && cs[ei].leaf->lhs == acc_buf && same_element(expr(o_access, acc_buf->get_name(), leaves[ei]->lhs_index, p_float32), acc_buf, ureal->lhs_index));
+    std::string epi_value_text, epi_store_text, epi_one_pass_text;   // of the fused epilogue: its value (reads _accv), its store of `_v`, both in one
+    bool epi_is_float = true;
     if (has_epi) {
         canon &E = cs[ei];
         std::vector<expr> ix;
         for (auto &e : E.leaf->lhs_index) ix.push_back(e.substitute(E.subs));
         expr val = replace_acc(E.leaf->rhs.substitute(E.subs));
-        body << "        " << dev.store(E.leaf->lhs, ix, dev.print(val), val.get_data_type()) << "\n";
+        epi_is_float = val.get_data_type() == p_float32;
+        epi_value_text = dev.print(val);
+        epi_store_text = dev.store(E.leaf->lhs, ix, "_v", val.get_data_type());
+        epi_one_pass_text = dev.store(E.leaf->lhs, ix, epi_value_text, val.get_data_type());
     }
-    body << "    });\n";
+    const bool two_pass = !(acc_stored && has_epi) && epi_is_float && !std::getenv("TIRAMISU_MFMA_ONE_PASS_EPILOGUE");
+    if (two_pass) {
+        body << "    auto _epi_value = [&](int _r, int _c, float _sum) -> float {\n" << digit_text << accv_text;
+        body << "        return " << (has_epi ? epi_value_text : std::string("_accv")) << ";\n    };\n";
+        body << "    auto _epi_store = [&](int _r, int _c, float _v) {\n" << digit_text;
+        if (has_epi) body << "        " << epi_store_text << "\n";
+        else if (acc_stored) body << "        " << dev.store(acc_buf, acc_index, "_v", p_float32) << "\n";
+        body << "    };\n";
+    } else {
+        body << "    auto _epi = [&](int _r, int _c, float _sum) {\n" << digit_text << accv_text;
+        if (acc_stored) body << "        " << dev.store(acc_buf, acc_index, "_accv", p_float32) << "\n";
+        if (has_epi) body << "        " << epi_one_pass_text << "\n";
+        body << "    };\n";
+    }
+    const std::string epi_args = two_pass ? "_epi_value, _epi_store" : "_epi";
+    if (windowed) {
+        body << window_call_head << epi_args << ");\n";
+    } else {
+        if (WGK > 1) body << "    if (tgemm::tile_reduce_k<CFG>(_acc, _lds))\n    ";
+        body << "    tgemm::tile_epilogue<CFG>(_acc, _M, _N, _tm * CFG::BM, _tn * CFG::BN, " << epi_args << ");\n";
+    }
     body << consumer_text.str();
 
     kernel k;
     k.name = kname;
     bool any_gather = false;
     for (auto &o : operands) any_gather = any_gather || !o.first.linear || !o.second.linear;
-    k.how = std::string("mfma-contraction: ") + (bf16 ? (BM >= 128 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
+    k.how = std::string("mfma-contraction: ") + (bf16 ? (BM >= 128 ? "v_mfma_f32_32x32x16_bf16, slices loaded straight into LDS, " : "v_mfma_f32_32x32x16_bf16, ") : "v_mfma_f32_32x32x2_f32, ") + (windowed ? "implicit GEMM, sliding window of " + std::to_string(win_taps) + " taps staged in LDS by blocks of " + std::to_string(win_cb) + " channels, " :
+                                                                                      any_gather ? "implicit GEMM (gathered operand), " : "") + "M " +
             std::to_string(Mg.size()) + " dim(s) x N " + std::to_string(Ng.size()) + " x K " + std::to_string(Kg.size()) + ", tile " +
             std::to_string(BM) + "x" + std::to_string(BN) + "x" + std::to_string(BK) + (edge ? ", guarded edges" : ", whole tiles") + ", " +
             std::to_string(operands.size()) + " product term(s)" + (has_init ? ", fused initialisation" : "") + (has_epi ? ", fused epilogue" : "") +
             (with_consumer ? ", " + std::to_string(xs.size()) + " point-wise statement(s) of the following nest fused (" + std::to_string(G) + " column group(s) per unit, " +
                                  std::to_string(dead.size()) + " temporaries kept in registers)" : "") +
-            (batched ? ", iterations of the parallel host loop as gridDim.z" : "");
+            (batched ? ", iterations of the parallel host loop as gridDim.z" : "") +
+            (windowed ? ", " + std::to_string(win_resident) + " workgroup(s) per compute unit take tiles from a queue" + (win_splits > 1 ? ", the last tiles cut into " + std::to_string(win_splits) + " pieces" : std::string()) : std::string());
     std::ostringstream host;
     host << "    {\n";
     // With a batched launch the values of the outer dimensions depend on blockIdx.z: they are computed
@@ -1468,6 +1618,19 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         if (b->get_location() != memory_location::global) return reject(22);
         k.params.push_back({true, nm, b->get_elements_type()});
     }
+    if (windowed) {
+        // scratch for the pieces of the last round's tiles and their counters: one block per host thread (calls
+        // work on the thread's current stream), allocated at the first call and kept; the counters start at zero
+        // and every launch leaves them at zero
+        k.params.push_back({true, "_tail_scratch", p_float32});
+        k.grid[0] = std::to_string(win_grid);
+        host << "        static thread_local float *_tail_scratch = nullptr;\n";
+        host << "        if (!_tail_scratch) {\n";
+        host << "            _tail_scratch = (float *)tiramisu_hip_malloc((uint64_t)" << win_scratch_floats << " * sizeof(float));\n";
+        host << "            static const uint32_t _zeros[" << win_counters << "] = {};\n";
+        host << "            tiramisu_hip_memcpy_to_device((void *)(_tail_scratch + " << (win_scratch_floats - win_counters) << "), (void *)_zeros, sizeof(_zeros));\n";
+        host << "        }\n";
+    }
     k.block[0] = std::to_string(NT);
     // two LDS stages of an A and a B slice
     {
@@ -1477,10 +1640,13 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         if (bf16) k.lds_bytes = std::to_string((BM >= 128 ? 4 : 2) * (BK / 8) * (BM + BN) * 4 * 4);   // four-stage ring for the large tiles
         else if (ktab_words) k.lds_bytes = std::to_string(2 * (rowA + rowB) * 4 + ktab_words * 4);
         if (with_consumer) k.lds_bytes = std::to_string(std::stol(k.lds_bytes) + BM * (BN + 1) * 4);
+        if (windowed) k.lds_bytes = std::to_string(2 * ((long)win_cb * (win_taps * BM + 32) + (long)win_cb * win_floats) * 4);
     }
     std::ostringstream src;
     src << pre.str();
-    src << "extern \"C\" __global__ void __launch_bounds__(" << NT << ") " << k.name << "(";
+    src << "extern \"C\" __global__ void __launch_bounds__(" << NT;
+    if (windowed && win_resident > 1) src << ", " << win_resident * (NT / 64) / 4;       // waves per SIMD: bounds the registers
+    src << ") " << k.name << "(";
     for (size_t i = 0; i < k.params.size(); i++) {
         auto &p = k.params[i];
         src << (i ? ", " : "");
@@ -1491,6 +1657,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     k.source = src.str();
     add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma.hip.h\"");
     if (bf16) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_bf16.hip.h\"");
+    if (windowed) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_window.hip.h\"");
     host << launch_text(k, "        ") << "    }\n";
     plan.kernels.push_back(k);
     plan.host_code = host.str();

@@ -15,6 +15,7 @@
 // CPU schedule (-DTIRAMISU_TARGET_CPU): parallelize n and co, vectorize x by 8 (the tags of
 // conv_layer_generator_tiramisu.cpp:110-112,172-173).
 // One generated function per shape: conv2d_<N>x<Cin>x<Cout>x<H>.
+#include <cstdlib>
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -86,6 +87,10 @@ static void generate(int NB, int CI, int CO, int H)
 
 int main()
 {
+    if (const char *nb = std::getenv("CONV_ONLY_FULL")) {   // experiments: the benchmark shape alone, with another batch size
+        generate(std::atoi(nb) > 1 ? std::atoi(nb) : 32, 64, 64, 112);
+        return 0;
+    }
     generate(32, 64, 64, 112);   // benchmark configuration 4
     generate(2, 8, 64, 16);
     generate(1, 3, 5, 12);       // ragged in every group

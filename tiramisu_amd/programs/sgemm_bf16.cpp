@@ -73,6 +73,7 @@ int main()
     generate(3072, 4096, 160);    // 256x256 tiles, five K-slices: one steady-state turn of the four-stage ring, then the drain
     generate(1024, 1280, 512);    // 128x128 tiles
     generate(128, 192, 128);      // whole 64x64x64 tiles: MFMA path
-    generate(48, 40, 24);         // no whole tiles: schedule-faithful kernel
+    generate(48, 40, 24);         // one ragged 64x64 tile: MFMA path with guarded loads
+    generate(200, 150, 100);      // ragged in every direction, rows of neither operand 16-byte aligned
     return 0;
 }
