@@ -32,15 +32,18 @@ namespace tgemm {
 // unit, by their LDS footprint) and they take work items from a queue: first the whole tiles -- all tiles but
 // R = T mod G, G = gridDim.x --, then the R remaining tiles cut into SPLITS pieces each along the channel blocks
 // (1568 tiles, 512 workgroups: 1536 whole tiles, then 32 tiles as 256 pieces), so that the end of the launch is
-// filled with short items.  Workgroup w starts with item w; further items come from an atomic counter, one item
-// ahead, because the first block of the next item is already travelling while the current item's last block is
-// multiplied.  Two workgroups of a compute unit share its matrix pipeline unevenly; with a fixed list per
-// workgroup the slower one would finish its list alone, at a workgroup's solo rate.
-// The pieces of a tile meet in `scratch`: partial tiles, one counter per remaining tile, then the queue's
-// counter and a counter of finished workgroups (all counters zero between launches; the last workgroup to
-// finish zeroes the queue).  The workgroup whose piece arrives last adds the pieces in piece order and runs the
+// filled with short items.  Items come from atomic counters, one item ahead, because the first block of the next
+// item is already travelling while the current item's last block is multiplied.  Two workgroups of a compute unit
+// share its matrix pipeline unevenly; with a fixed list per workgroup the slower one would finish its list alone,
+// at a workgroup's solo rate.  The whole tiles are dealt to the XCDs in contiguous ranges with a counter each
+// (workgroup w runs on XCD w mod 8): the windows of neighbouring tiles overlap -- 544 floats per channel for 256
+// positions here -- and are fetched once per L2 when neighbours run on the same XCD at about the same time.  A
+// workgroup whose XCD has no whole tile left takes pieces, from one counter for all.
+// The pieces of a tile meet in `scratch`: partial tiles, one counter per remaining tile, then the piece queue, a
+// counter of finished workgroups and the XCDs' queues (all counters zero between launches; the last workgroup to
+// finish zeroes the queues).  The workgroup whose piece arrives last adds the pieces in piece order and runs the
 // epilogue, so the result does not depend on the order of arrival.
-template <class CFG, int CB, int TAPS, int WIN, int AHEAD, int SPLITS, class TAP_OFFSETS, class POS, class VALUE, class STORE>
+template <class CFG, int CB, int TAPS, int WIN, int AHEAD, int SPLITS, bool BY_XCD, class TAP_OFFSETS, class POS, class VALUE, class STORE>
 __device__ __forceinline__ void contraction_window(const float *__restrict__ A, long lda, const float *__restrict__ X, long x_elements,
                                                    const POS &pos, long chan_stride, int channels, int M, int N,
                                                    float *__restrict__ scratch, float *lds, VALUE value, STORE store) {
@@ -177,7 +180,7 @@ __device__ __forceinline__ void contraction_window(const float *__restrict__ A, 
     constexpr int QUADS = TM * TN * 4;
     f32x4 *pieces = reinterpret_cast<f32x4 *>(scratch);
     unsigned *counters = reinterpret_cast<unsigned *>(scratch + (long)rest * splits * BM * BN);
-    unsigned *queue = counters + rest, *finished = queue + 1;
+    unsigned *piece_queue = counters + rest, *finished = piece_queue + 1, *xcd_queue = finished + 1;
     auto finish_piece = [&](int q, int m0, int n0) {
         const int rt = (q - whole) / splits, z = (q - whole) % splits;
         f32x4 *mine = pieces + ((long)rt * splits + z) * QUADS * NT;
@@ -223,7 +226,14 @@ __device__ __forceinline__ void contraction_window(const float *__restrict__ A, 
     };
 
     __shared__ int next_item;
-    int cur = w;                                   // G <= whole: every workgroup has a first item
+    // this workgroup's group (its XCD), its place there, the group's range of whole tiles
+    const int groups = BY_XCD && G % ttarget::XCDS == 0 ? ttarget::XCDS : 1, x = w % groups, in_group = G / groups;
+    const int lo = (int)((long)x * whole / groups), hi = (int)((long)(x + 1) * whole / groups);
+    auto take_item = [&]() {
+        const int i = in_group + (int)atomicAdd(xcd_queue + x, 1u);
+        return lo + i < hi ? lo + i : whole + (int)atomicAdd(piece_queue, 1u);
+    };
+    int cur = lo + w / groups;                     // G <= whole: every workgroup has a first item
     int m0, n0;
     aim_loads_at(item_tile(cur));
     aim_tile_at(item_tile(cur), m0, n0);
@@ -236,7 +246,7 @@ __device__ __forceinline__ void contraction_window(const float *__restrict__ A, 
     int stage = 0;
     while (cur < items) {
         // the item after this one (a barrier lies between this write and the previous item's read: block() has one)
-        if (t == 0) next_item = G + (int)atomicAdd(queue, 1u);
+        if (t == 0) next_item = take_item();
         __syncthreads();
         const int next = next_item;
         // all blocks but the last: nothing but the block pipeline in this loop
@@ -259,8 +269,9 @@ __device__ __forceinline__ void contraction_window(const float *__restrict__ A, 
     }
     // the last workgroup to run out of items leaves the queue ready for the next launch
     if (t == 0 && atomicAdd(finished, 1u) == (unsigned)(G - 1)) {
-        *queue = 0;
+        *piece_queue = 0;
         *finished = 0;
+        for (int g = 0; g < groups; g++) xcd_queue[g] = 0;
     }
 }
 

@@ -1184,9 +1184,10 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
                 const long rest = tiles % win_grid;
                 if (rest > 0 && tiles > win_grid && !std::getenv("TIRAMISU_MFMA_NO_TAIL_SPLIT")) win_splits = (int)std::min<long>(std::min<long>(blocks, 2 * win_grid / rest), 16);
                 if (win_splits < 2) win_splits = 1;
-                // partial tiles of the pieces, a counter per remaining tile, the work queue's two counters
+                // partial tiles of the pieces, a counter per remaining tile, the work queues' counters (pieces,
+                // finished workgroups, one per XCD)
                 const long cut = win_splits > 1 ? rest : 0;
-                win_counters = cut + 2;
+                win_counters = cut + 2 + ttarget::XCDS;
                 win_scratch_floats = cut * win_splits * BM * BN + win_counters;
             }
         }
@@ -1408,7 +1409,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
             for (int p : GN.dims) pre << " + (long)" << U.dims[p].kvar << " * " << dev.print(o.second.coef.at(p));
             pre << ";\n    }\n};\n";
             std::ostringstream call;
-            call << "    tgemm::contraction_window<CFG, " << win_cb << ", " << win_taps << ", " << win_floats << ", " << env_int("TIRAMISU_MFMA_WINDOW_AHEAD", 2) << ", " << win_splits << ", " << kname << "_taps>("
+            call << "    tgemm::contraction_window<CFG, " << win_cb << ", " << win_taps << ", " << win_floats << ", " << env_int("TIRAMISU_MFMA_WINDOW_AHEAD", 2) << ", " << win_splits << ", " << (env_int("TIRAMISU_MFMA_WINDOW_XCD_QUEUES", 1) ? "true" : "false") << ", " << kname << "_taps>("
                  << o.first.buf->get_name() << " + (" << dev.print(o.first.base) << "), " << dev.print(o.first.ld) << ", " << o.second.buf->get_name() << " + ("
                  << dev.print(o.second.base) << "), " << win_x_elements << "L, " << kname << "_pos(), " << win_chan_stride << "L, " << win_channels
                  << ", _M, _N, _tail_scratch, _lds, ";
