@@ -167,6 +167,13 @@ public:
       * (reference: tiramisu_function.cpp:1458-1511, tiramisu_core.cpp:2268-2335). */
     void allocate_and_map_buffers_automatically();
     void dump_dep_graph();
+    /** Infer iteration domains from consumers: starting from the computations that nothing reads, a
+      * computation's domain becomes what its consumers read of it (joined with the domain it was declared
+      * with, unless that was unbounded); computations with several definitions keep theirs
+      * (reference: tiramisu_function.cpp:624-747). */
+    void compute_bounds();
+    /** Computations that no other computation reads (reference: tiramisu_function.cpp:503-615). */
+    std::vector<computation *> get_live_out_computations();
     /** Print the iteration domains / the time-space domains (domain mapped through the schedule) of all
       * computations (reference: core.h:1071-1109). */
     void dump_iteration_domain() const;
@@ -232,6 +239,8 @@ public:
     void set_auto_deallocate(bool v) { auto_deallocate = v; }
     bool has_constant_extents() const;
     function *get_function() const { return fct; }
+    /** Reference: tiramisu_core.cpp:8159-8167. */
+    void set_dim_size(int dim, int size);
 
     /** Memory-space tags (reference: tiramisu_core.cpp:8913-8936). */
     void tag_gpu_global() { location = memory_location::global; }
@@ -305,6 +314,9 @@ protected:
     void assert_names_not_assigned(const std::vector<std::string> &names) const;
     void separate_and_split(int level, int factor, const std::string &outer,
                             const std::string &inner, bool &split_applied);
+    computation *copy_as(const std::string &new_name);
+    void separate_by_text(int dim, const std::string &bound_text, const std::string &params);
+    std::vector<computation *> duplicates;
 
 public:
     static const var root;
@@ -339,6 +351,10 @@ public:
     const expr &get_predicate() const { return predicate; }
     primitive_t get_data_type() const { return data_type; }
     int get_iteration_domain_dimensions_number() const;
+    /** Lowest and highest value of iteration-domain dimension \p dim among the iterations that this computation
+      * executes (its iteration domain restricted by its schedule: separated pieces and duplicates execute a
+      * part); false when there is none or the range is not a pair of constants. */
+    bool executed_range(int dim, long &lowest, long &highest) const;
     int get_loop_levels_number() const { return (int)level_names.size(); }
     const std::vector<std::string> &get_loop_level_names() const { return level_names; }
     const std::vector<std::string> &get_iteration_domain_dimension_names() const { return iterator_names_; }
@@ -468,6 +484,37 @@ public:
     void tag_unroll_level(var L, int F);
     void tag_unroll_level(int L);
     void tag_unroll_level(int L, int F);
+    // ---- separation, redundant computation, storage folding ----
+    /** Cut this computation in two at loop level \p dim: it keeps the iterations below
+      * lower_bound + v * floor(N / v) -- whole groups of v -- and a new definition (get_update(k)), scheduled
+      * after it at that level, takes the rest (reference: tiramisu_core.cpp:746-870). */
+    void separate(int dim, expr N, int v, expr lower_bound);
+    void separate(int dim, expr N, int v) { separate(dim, N, v, expr((int32_t)0)); }
+    /** Cut at the given points of loop level \p level: this computation keeps [.., p0), new definitions take
+      * [p0, p1), ..., [p(n-1), max) (reference: tiramisu_core.cpp:872-1010). */
+    void separate_at(var level, std::vector<expr> separate_points, expr max);
+    /** separate() at the loop's own bounds, then split the full part by \p sizeX counting from the loop's lower
+      * bound; false when the loop is not longer than sizeX and nothing was split
+      * (reference: tiramisu_core.cpp:6103-6240). */
+    bool separateAndSplit(var L0, int sizeX);
+    bool separateAndSplit(var L0, int sizeX, var L0_outer, var L0_inner);
+    bool separateAndSplit(int L0, int sizeX);
+    virtual void split_with_lower_bound(int L0, int sizeX, std::string lower_bound);
+    /** A copy of this computation (same expression, data mapping and schedule) restricted to the given part of
+      * the iteration domain and / or of the time-space domain; scheduled on its own from then on
+      * (reference: tiramisu_core.cpp:3244-3310).  select(k) returns the k-th duplicate (0: this computation). */
+    computation *duplicate(std::string domain_constraints, std::string range_constraints);
+    computation *select(int duplicate_id);
+    /** Compute this computation inside the loop nest of \p consumer at loop level \p L: ordered before the
+      * consumer there, and whatever the consumer's iterations of that level read that this computation does not
+      * produce in the same iteration is computed again by a duplicate, shifted into that iteration
+      * (reference: tiramisu_core.cpp:5262-5660). */
+    void compute_at(computation &consumer, var L);
+    void compute_at(computation &consumer, int L);
+    /** Store dimension \p dim of this computation's buffer modulo \p f: the buffer keeps f entries there
+      * (reference: tiramisu_core.cpp:8169-8260). */
+    virtual void storage_fold(var dim, int f);
+
     void set_low_level_schedule(std::string map_str);
     void apply_transformation_on_schedule(std::string map_str);
     void set_loop_level_names(std::vector<std::string> names);

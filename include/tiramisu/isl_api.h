@@ -115,6 +115,9 @@ isl_set *isl_set_lexmax(isl_set *set);
 isl_bool isl_set_is_singleton(isl_set *set);
 isl_val *isl_set_plain_get_val_if_fixed(isl_set *set, enum isl_dim_type type, unsigned pos);
 isl_val *isl_set_count_val(isl_set *set);
+isl_bool isl_set_plain_is_universe(isl_set *set);
+isl_size isl_pw_aff_n_piece(isl_pw_aff *pwaff);
+isl_set *isl_set_remove_redundancies(isl_set *set);
 
 // maps
 isl_map *isl_map_read_from_str(isl_ctx *ctx, const char *str);

@@ -56,6 +56,8 @@ std::string expr_to_isl_str(const expr &e, bool &ok) {
     }
 }
 
+static std::string single_piece_text(isl_pw_aff *pa);
+
 static std::string params_prefix(const std::vector<std::string> &params) {
     if (params.empty()) return "";
     return "[" + join(params, ", ") + "] -> ";
@@ -789,6 +791,9 @@ void computation::assert_names_not_assigned(const std::vector<std::string> &name
 void computation::apply_on_range(const std::string &t) {
     isl_map *m = isl_map_read_from_str(ctx, t.c_str());
     if (!m) ERROR("cannot parse schedule transformation " + t, true);
+    // dimensions that align_schedules() appended (zeros behind the last level) are dropped again first
+    const int have = (int)isl_map_dim(schedule, isl_dim_out), takes = (int)isl_map_dim(m, isl_dim_in);
+    if (have > takes) schedule = isl_map_project_out(schedule, isl_dim_out, takes, have - takes);
     schedule = isl_map_apply_range(schedule, m);
 }
 
@@ -1050,10 +1055,18 @@ void computation::tag_unroll_level(var L, int F) { tag_unroll_level(get_loop_lev
 // separates a remainder computation when the extent is not a multiple of the factor
 // (tiramisu_core.cpp:1238-1370); here the inner loop simply keeps a min() bound on the last
 // tile, which executes the same iterations in the same order.
+// vectorize / unroll: the loop is cut into whole groups of `factor` iterations, which are split, and a remainder
+// that a definition of its own computes (reference: tiramisu_core.cpp:1238-1274 -> separateAndSplit); where the
+// loop's bounds are not single affine expressions of the parameters the loop is split as a whole and the inner
+// loop keeps a min() bound on the last group.
 void computation::separate_and_split(int level, int factor, const std::string &outer, const std::string &inner,
                                      bool &split_applied) {
     isl_set *ts = isl_set_apply(isl_set_copy(iteration_domain), isl_map_copy(schedule));
-    int p = dynamic_pos(level);
+    const int p = dynamic_pos(level), n = (int)level_names.size();
+    isl_set *level_values = isl_set_project_out(isl_set_copy(ts), isl_dim_set, p + 1, 2 * n + 2 - (p + 1));
+    level_values = isl_set_project_out(level_values, isl_dim_set, 0, p);
+    const bool separable = !single_piece_text(isl_set_dim_max(isl_set_copy(level_values), 0)).empty() &&
+                           !single_piece_text(isl_set_dim_min(level_values, 0)).empty() && !std::getenv("TIRAMISU_NO_SEPARATION");
     isl_val *mx = isl_set_dim_max_val(isl_set_copy(ts), p);
     isl_val *mn = isl_set_dim_min_val(ts, p);
     long extent = -1;
@@ -1062,11 +1075,11 @@ void computation::separate_and_split(int level, int factor, const std::string &o
     isl_val_free(mx);
     isl_val_free(mn);
     split_applied = !(extent > 0 && extent <= factor);
-    if (split_applied) {
-        split(level, factor);
-        level_names[level] = outer;
-        level_names[level + 1] = inner;
-    }
+    if (!split_applied) return;
+    if (separable) separateAndSplit(level, factor);
+    else split(level, factor);
+    level_names[level] = outer;
+    level_names[level + 1] = inner;
 }
 
 void computation::vectorize(var L, int v, var L_outer, var L_inner) {
@@ -1416,6 +1429,407 @@ bool computation::shared_caches_cover_reads() const {
     const bool covered = isl_map_is_empty(violations) == isl_bool_true;
     isl_map_free(violations);
     return covered;
+}
+
+// ------------------------------------------------------------------ separation, duplicates, compute_at, storage folding
+
+static std::string function_params(function *f) { return params_prefix(f->get_invariant_names()); }
+
+// the time-space tuple of a schedule with n levels as variables x0 ... x(2n+1)
+static std::string time_space_tuple(int levels) {
+    std::vector<std::string> v;
+    range_vars(levels, v);
+    return "[" + join(v, ",") + "]";
+}
+
+bool computation::executed_range(int dim, long &lowest, long &highest) const {
+    isl_set *points = isl_map_domain(isl_map_intersect_domain(isl_map_copy(schedule), isl_set_copy(iteration_domain)));
+    bool ok = isl_set_is_empty(points) != isl_bool_true && dim >= 0 && dim < (int)isl_set_dim(points, isl_dim_set);
+    if (ok) {
+        isl_val *a = isl_set_dim_min_val(isl_set_copy(points), dim), *b = isl_set_dim_max_val(isl_set_copy(points), dim);
+        ok = a && b && isl_val_is_int(a) == isl_bool_true && isl_val_is_int(b) == isl_bool_true;
+        if (ok) { lowest = isl_val_get_num_si(a); highest = isl_val_get_num_si(b); }
+        isl_val_free(a);
+        isl_val_free(b);
+    }
+    isl_set_free(points);
+    return ok;
+}
+
+void buffer::set_dim_size(int dim, int size) {
+    if (dim < 0 || dim >= (int)dim_sizes.size() || size <= 0) ERROR("set_dim_size: bad dimension or size for buffer " + name, true);
+    dim_sizes[dim] = expr((int32_t)size);
+}
+
+// A copy of this computation under another name: same iteration domain, expression, schedule, level names and
+// data mapping; a definition of the same first definition, so accesses to it keep reading through that one.
+computation *computation::copy_as(const std::string &new_name) {
+    isl_set *dom = isl_set_set_tuple_name(isl_set_copy(iteration_domain), new_name.c_str());
+    char *text = isl_set_to_str(dom);
+    computation *c = new computation(std::string(text), expression, schedule_this, data_type, fct);
+    free(text);
+    isl_set_free(dom);
+    c->iterator_names_ = iterator_names_;
+    c->level_names = level_names;
+    c->declared_vars = declared_vars;
+    if (c->schedule) isl_map_free(c->schedule);
+    c->schedule = isl_map_set_tuple_name(isl_map_copy(schedule), isl_dim_in, new_name.c_str());
+    if (access) c->access = isl_map_set_tuple_name(isl_map_copy(access), isl_dim_in, new_name.c_str());
+    c->predicate = predicate;
+    c->associated_let_stmts = associated_let_stmts;
+    c->is_let = is_let;
+    c->inline_ = inline_;
+    c->first_definition = get_first_definition();
+    return c;
+}
+
+// Cut at loop level `dim`: this computation keeps the time-space points with x(dim) < bound, a new definition
+// takes x(dim) >= bound and runs after this one at that level.
+void computation::separate_by_text(int dim, const std::string &bound, const std::string &params) {
+    const int n = (int)level_names.size();
+    if (dim < 0 || dim >= n) ERROR("separate: level out of range for " + name, true);
+    const std::string x = "x" + std::to_string(dynamic_pos(dim));
+    const std::string full = params + "{ " + time_space_tuple(n) + " : " + x + " < " + bound + " }";
+    const std::string rest = params + "{ " + time_space_tuple(n) + " : " + x + " >= " + bound + " }";
+    isl_set *rest_set = isl_set_read_from_str(ctx, rest.c_str());
+    if (!rest_set) ERROR("separate: cannot parse " + rest, true);
+    isl_map *there = isl_map_intersect_range(isl_map_intersect_domain(isl_map_copy(schedule), isl_set_copy(iteration_domain)), rest_set);
+    const bool empty = isl_map_is_empty(there) == isl_bool_true;
+    isl_map_free(there);
+    if (!empty) {
+        computation *first = get_first_definition();
+        computation *c = copy_as("_" + first->name + "_update_" + std::to_string(first->updates.size() + 1));
+        first->updates.push_back(c);
+        c->add_schedule_constraint("", rest);
+        c->after(*this, dim);
+    }
+    add_schedule_constraint("", full);
+}
+
+void computation::separate(int dim, expr N, int v, expr lower_bound) {
+    bool ok = true;
+    const std::string n_text = expr_to_isl_str(N, ok), lower = expr_to_isl_str(lower_bound, ok);
+    if (!ok || v < 1) ERROR("separate: the loop extent and lower bound must be affine, the factor positive (" + name + ")", true);
+    separate_by_text(dim, "(" + std::to_string(v) + " * floor((" + n_text + ") / " + std::to_string(v) + ") + (" + lower + "))", function_params(fct));
+}
+
+void computation::separate_at(var level, std::vector<expr> separate_points, expr max) {
+    if (separate_points.empty()) ERROR("separate_at: no separation point given for " + name, true);
+    const int dim = get_loop_level_number_from_dimension_name(level.get_name());
+    const int n = (int)level_names.size();
+    const std::string x = "x" + std::to_string(dynamic_pos(dim)), params = function_params(fct);
+    bool ok = true;
+    std::vector<std::string> cut;
+    for (auto &pt : separate_points) cut.push_back("(" + expr_to_isl_str(pt, ok) + ")");
+    cut.push_back("(" + expr_to_isl_str(max, ok) + ")");
+    if (!ok) ERROR("separate_at: separation points must be affine (" + name + ")", true);
+    computation *first = get_first_definition();
+    computation *previous = this;
+    for (size_t k = 0; k + 1 < cut.size(); k++) {
+        const std::string piece = params + "{ " + time_space_tuple(n) + " : " + x + " >= " + cut[k] + " and " + x + " < " + cut[k + 1] + " }";
+        isl_set *piece_set = isl_set_read_from_str(ctx, piece.c_str());
+        if (!piece_set) ERROR("separate_at: cannot parse " + piece, true);
+        isl_map *there = isl_map_intersect_range(isl_map_intersect_domain(isl_map_copy(schedule), isl_set_copy(iteration_domain)), piece_set);
+        const bool empty = isl_map_is_empty(there) == isl_bool_true;
+        isl_map_free(there);
+        if (empty) continue;
+        computation *c = copy_as("_" + first->name + "_update_" + std::to_string(first->updates.size() + 1));
+        first->updates.push_back(c);
+        c->add_schedule_constraint("", piece);
+        c->after(*previous, dim);
+        previous = c;
+    }
+    add_schedule_constraint("", params + "{ " + time_space_tuple(n) + " : " + x + " < " + cut[0] + " }");
+}
+
+// "(text)" of the single affine piece of a bound, empty when the bound is piecewise
+static std::string single_piece_text(isl_pw_aff *pa) {
+    std::string out;
+    if (pa && isl_pw_aff_n_piece(pa) == 1) {
+        char *t = isl_pw_aff_to_str(pa);          // "[N] -> { [(-1 + N)] }"
+        std::string s = t ? t : "";
+        free(t);
+        const size_t a = s.find("[("), b = s.rfind(")]");
+        if (a != std::string::npos && b != std::string::npos && b > a && s.find(" : ", a) == std::string::npos) out = s.substr(a + 1, b - a);
+    }
+    if (pa) isl_pw_aff_free(pa);
+    return out;
+}
+
+void computation::split_with_lower_bound(int L0, int sizeX, std::string lower_bound) {
+    const int n = (int)level_names.size();
+    if (L0 < 0 || L0 >= n) ERROR("split: level out of range for " + name, true);
+    if (sizeX < 1) ERROR("split: factor must be positive", true);
+    std::vector<std::string> in, out;
+    range_vars(n, in);
+    const std::string d = "(" + in[dynamic_pos(L0)] + " - (" + lower_bound + "))", f = std::to_string(sizeX);
+    for (int i = 0; i < (int)in.size(); i++) {
+        if (i != dynamic_pos(L0)) { out.push_back(in[i]); continue; }
+        out.push_back("floor(" + d + " / " + f + ")");
+        out.push_back("0");
+        out.push_back(d + " mod " + f);
+    }
+    apply_on_range(function_params(fct) + "{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+    level_names.insert(level_names.begin() + L0 + 1, fct->generate_new_name(level_names[L0] + "_in"));
+}
+
+bool computation::separateAndSplit(int L0, int v) {
+    const int n = (int)level_names.size();
+    if (L0 < 0 || L0 >= n) ERROR("separateAndSplit: level out of range for " + name, true);
+    isl_set *ts = isl_set_apply(isl_set_copy(iteration_domain), isl_map_copy(schedule));
+    const int p = dynamic_pos(L0);
+    // a loop of at most v iterations stays as it is
+    isl_val *mx = isl_set_dim_max_val(isl_set_copy(ts), p), *mn = isl_set_dim_min_val(isl_set_copy(ts), p);
+    long extent = -1;
+    if (mx && mn && isl_val_is_int(mx) == isl_bool_true && isl_val_is_int(mn) == isl_bool_true) extent = isl_val_get_num_si(mx) - isl_val_get_num_si(mn) + 1;
+    isl_val_free(mx);
+    isl_val_free(mn);
+    if (extent > 0 && extent <= v) { isl_set_free(ts); return false; }
+    // bounds of the level in terms of the parameters alone
+    isl_set *level_values = isl_set_project_out(isl_set_copy(ts), isl_dim_set, p + 1, 2 * n + 2 - (p + 1));
+    level_values = isl_set_project_out(level_values, isl_dim_set, 0, p);
+    const std::string upper = single_piece_text(isl_set_dim_max(isl_set_copy(level_values), 0));
+    const std::string lower = single_piece_text(isl_set_dim_min(level_values, 0));
+    isl_set_free(ts);
+    if (upper.empty() || lower.empty()) ERROR("separateAndSplit: the bounds of level " + level_names[L0] + " of " + name + " are not single affine expressions of the parameters", true);
+    const std::string count = "(" + upper + " - " + lower + " + 1)", f = std::to_string(v);
+    std::vector<std::string> params;
+    for (int i = 0; i < (int)isl_map_dim(schedule, isl_dim_param); i++) params.push_back(isl_map_get_dim_name(schedule, isl_dim_param, i));
+    for (auto &nm : fct->get_invariant_names()) if (std::find(params.begin(), params.end(), nm) == params.end()) params.push_back(nm);
+    separate_by_text(L0, "(" + f + " * floor(" + count + " / " + f + ") + " + lower + ")", params_prefix(params));
+    split_with_lower_bound(L0, v, lower);
+    return true;
+}
+
+bool computation::separateAndSplit(var L0, int sizeX, var L0_outer, var L0_inner) {
+    const int l = get_loop_level_number_from_dimension_name(L0.get_name());
+    assert_names_not_assigned({L0_outer.get_name(), L0_inner.get_name()});
+    const bool split_happened = separateAndSplit(l, sizeX);
+    level_names[l] = L0_outer.get_name();
+    if (split_happened) level_names[l + 1] = L0_inner.get_name();
+    return split_happened;
+}
+
+bool computation::separateAndSplit(var L0, int sizeX) {
+    return separateAndSplit(L0, sizeX, var(fct->generate_new_name(L0.get_name() + "_so")), var(fct->generate_new_name(L0.get_name() + "_si")));
+}
+
+computation *computation::duplicate(std::string domain_constraints, std::string range_constraints) {
+    fct->align_schedules();
+    computation *first = get_first_definition();
+    computation *c = copy_as("_" + first->name + "_dup_" + std::to_string(first->duplicates.size() + 1));
+    first->duplicates.push_back(c);
+    if (!domain_constraints.empty()) {
+        isl_set *d = isl_set_read_from_str(ctx, domain_constraints.c_str());
+        if (!d) ERROR("duplicate: cannot parse " + domain_constraints, true);
+        d = isl_set_set_tuple_name(d, c->name.c_str());
+        c->schedule = isl_map_intersect_domain(c->schedule, d);
+    }
+    c->add_schedule_constraint("", range_constraints);
+    // the duplicate's number goes into the first time-space dimension
+    std::vector<std::string> in, out;
+    range_vars((int)c->level_names.size(), in);
+    out = in;
+    out[0] = std::to_string(first->duplicates.size());
+    c->apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
+    return c;
+}
+
+computation *computation::select(int duplicate_id) {
+    computation *first = get_first_definition();
+    if (duplicate_id == 0) return this;
+    if (duplicate_id < 0 || duplicate_id > (int)first->duplicates.size()) ERROR("select: " + name + " has no duplicate number " + std::to_string(duplicate_id), true);
+    return first->duplicates[duplicate_id - 1];
+}
+
+// { consumer[iterators] -> producer[indices] } for every read of `producer` in the consumer's expression and predicate
+static isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain = true) {
+    function *f = consumer.get_function();
+    const std::string wanted = producer.get_first_definition()->get_name();
+    std::vector<std::string> pieces;
+    bool ok = true;
+    auto collect = [&](const expr &e) {
+        if (!e.is_defined()) return;
+        e.visit([&](const expr &x) {
+            if (x.get_expr_type() != e_op || x.get_op_type() != o_access || x.get_name() != wanted) return;
+            std::vector<std::string> idx;
+            for (auto &i : x.get_access()) idx.push_back(expr_to_isl_str(i, ok));
+            pieces.push_back(consumer.get_name() + "[" + join(consumer.get_iteration_domain_dimension_names(), ",") + "] -> " + producer.get_name() + "[" + join(idx, ",") + "]");
+        });
+    };
+    collect(consumer.get_expr());
+    collect(consumer.get_predicate());
+    if (!ok) ERROR("an index of " + wanted + " in " + consumer.get_name() + " is not affine", true);
+    if (pieces.empty()) return nullptr;
+    isl_map *all = nullptr;
+    for (auto &pc : pieces) {
+        isl_map *m = isl_map_read_from_str(f->get_isl_ctx(), (function_params(f) + "{ " + pc + " }").c_str());
+        if (!m) ERROR("cannot parse read relation " + pc, true);
+        all = all ? isl_map_union(all, m) : m;
+    }
+    all = isl_map_intersect_domain(all, isl_set_copy(consumer.get_iteration_domain()));
+    return within_producer_domain ? isl_map_intersect_range(all, isl_set_copy(producer.get_iteration_domain())) : all;
+}
+
+std::vector<computation *> function::get_live_out_computations() {
+    std::vector<computation *> out;
+    for (auto c : body) {
+        if (c->is_inline_computation() || !c->get_expr().is_defined() && !c->should_schedule_this_computation()) continue;
+        const std::string nm = c->get_first_definition()->get_name();
+        bool is_read = false;
+        for (auto k : body) {
+            if (k->get_first_definition() == c->get_first_definition()) continue;
+            for (const expr *e : {&k->get_expr(), &k->get_predicate()})
+                if (e->is_defined()) e->visit([&](const expr &x) { if (x.get_expr_type() == e_op && x.get_op_type() == o_access && x.get_name() == nm) is_read = true; });
+        }
+        if (!is_read) out.push_back(c);
+    }
+    return out;
+}
+
+void function::compute_bounds() {
+    std::map<computation *, isl_set *> frontier;
+    for (auto c : get_live_out_computations()) frontier[c] = isl_set_copy(c->get_iteration_domain());
+    for (size_t round = 0; round <= body.size() && !frontier.empty(); round++) {
+        std::map<computation *, isl_set *> next;
+        for (auto &fr : frontier) {
+            for (auto p : body) {
+                if (p->get_first_definition() == fr.first->get_first_definition()) continue;       // a computation reading itself adds nothing
+                if (!p->is_first_definition() || !p->get_updates().empty()) continue;               // several definitions: the user's domains stay
+                isl_map *m = reads_of(*fr.first, *p, false);
+                if (!m) continue;
+                isl_set *needed = isl_set_apply(isl_set_copy(fr.second), m);
+                if (isl_set_is_empty(needed) == isl_bool_true) { isl_set_free(needed); continue; }
+                next[p] = next.count(p) ? isl_set_union(next[p], needed) : needed;
+            }
+            isl_set_free(fr.second);
+        }
+        for (auto &nx : next) {
+            computation *p = nx.first;
+            isl_set *dom = isl_set_plain_is_universe(p->iteration_domain) == isl_bool_true
+                               ? isl_set_copy(nx.second) : isl_set_union(isl_set_copy(p->iteration_domain), isl_set_copy(nx.second));
+            dom = isl_set_coalesce(dom);
+            dom = isl_set_set_tuple_name(dom, p->name.c_str());
+            for (size_t d = 0; d < p->iterator_names_.size(); d++) dom = isl_set_set_dim_name(dom, isl_dim_set, (unsigned)d, p->iterator_names_[d].c_str());
+            isl_set_free(p->iteration_domain);
+            p->iteration_domain = dom;
+        }
+        frontier = next;
+    }
+    for (auto &fr : frontier) isl_set_free(fr.second);
+}
+
+void computation::compute_at(computation &consumer, var L) {
+    compute_at(consumer, consumer.get_loop_level_number_from_dimension_name(L.get_name()));
+}
+
+void computation::compute_at(computation &consumer, int L) {
+    fct->align_schedules();
+    const int n = (int)isl_map_dim(schedule, isl_dim_out);                  // 2 * levels + 2, the same for both now
+    if (L < root_dimension || dynamic_pos(L) >= n) ERROR("compute_at: level out of range for " + consumer.name, true);
+    // `first`, the head of the chain that ends in this computation, goes right before the consumer: behind the
+    // consumer's present predecessor if it has one
+    auto chain_before_consumer = [&](computation *first) {
+        computation *q = consumer.get_predecessor();
+        if (q && q != this && q != first) {
+            const int level_q = fct->sched_graph[q][&consumer];
+            fct->sched_graph[q].erase(&consumer);
+            fct->sched_graph_reversed[&consumer].erase(q);
+            first->after(*q, level_q);
+        }
+        consumer.after(*this, L);
+    };
+    isl_map *reads = reads_of(consumer, *this);
+    if (!reads || L == root_dimension) {
+        // nothing read (or the whole nests one after the other): ordering only
+        if (reads) isl_map_free(reads);
+        chain_before_consumer(this);
+        return;
+    }
+    // reads, consumer and producer in time-space coordinates; the loops down to L pinned to parameters _T0 ... _TL
+    reads = isl_map_apply_range(isl_map_apply_domain(reads, isl_map_copy(consumer.schedule)), isl_map_copy(schedule));
+    std::vector<std::string> vars, t_names, pins, distances;
+    for (int i = 0; i < n; i++) vars.push_back("x" + std::to_string(i));
+    for (int i = 0; i <= L; i++) {
+        t_names.push_back("_T" + std::to_string(i));
+        pins.push_back(vars[dynamic_pos(i)] + " = " + t_names.back());
+        distances.push_back(vars[dynamic_pos(i)] + " - " + t_names.back());
+    }
+    const std::string t_params = "[" + join(t_names, ",") + "] -> ";
+    isl_set *pin = isl_set_read_from_str(ctx, (t_params + "{ [" + join(vars, ",") + "] : " + join(pins, " and ") + " }").c_str());
+    isl_set *consumer_ts = isl_set_intersect(isl_set_apply(isl_set_copy(consumer.iteration_domain), isl_map_copy(consumer.schedule)), isl_set_copy(pin));
+    isl_set *produced = isl_set_intersect(isl_set_apply(isl_set_copy(iteration_domain), isl_map_copy(schedule)), pin);
+    isl_set *needed = isl_set_apply(consumer_ts, reads);
+    isl_set *missing = isl_set_coalesce(isl_set_subtract(needed, produced));
+    if (isl_set_is_empty(missing) == isl_bool_true) {
+        isl_set_free(missing);
+        chain_before_consumer(this);
+        return;
+    }
+    // How far, per level, the missing points lie from the iteration that needs them: the set of distance vectors
+    // (x(level) - _T(level)) must be a few constant vectors.
+    isl_set *vectors = isl_set_apply(isl_set_copy(missing),
+                                     isl_map_read_from_str(ctx, (t_params + "{ [" + join(vars, ",") + "] -> [" + join(distances, ",") + "] }").c_str()));
+    vectors = isl_set_project_out(vectors, isl_dim_param, 0, isl_set_dim(vectors, isl_dim_param));
+    std::vector<std::vector<int>> found;
+    while (isl_set_is_empty(vectors) != isl_bool_true) {
+        if (found.size() == 32) ERROR("compute_at: what " + consumer.name + " reads of " + name + " outside its own iterations is not at a few fixed distances", true);
+        isl_set *pt = isl_set_lexmin(isl_set_copy(vectors));
+        std::vector<int> v;
+        for (int i = 0; i <= L; i++) {
+            isl_val *c = isl_set_plain_get_val_if_fixed(pt, isl_dim_set, i);
+            if (!c || isl_val_is_int(c) != isl_bool_true) ERROR("compute_at: what " + consumer.name + " reads of " + name + " outside its own iterations is not at fixed distances", true);
+            v.push_back((int)isl_val_get_num_si(c));
+            isl_val_free(c);
+        }
+        found.push_back(v);
+        vectors = isl_set_subtract(vectors, pt);
+    }
+    isl_set_free(vectors);
+    // One duplicate computes every missing point, once, early enough for all its readers: at the largest distance
+    // per level (a point read from distances c1 and c2 is computed at its own time minus max(c1, c2), which is
+    // not later than either reader).  The buffer keeps it for the later readers.
+    std::vector<int> farthest = found[0];
+    for (auto &v : found)
+        for (int i = 0; i <= L; i++) farthest[i] = std::max(farthest[i], v[i]);
+    for (auto &t : t_names)
+        for (int i = 0; i < (int)isl_set_dim(missing, isl_dim_param); i++)
+            if (t == isl_set_get_dim_name(missing, isl_dim_param, i)) { missing = isl_set_project_out(missing, isl_dim_param, i, 1); break; }
+    char *text = isl_set_to_str(missing);
+    computation *redundant = duplicate("", text);
+    free(text);
+    for (int i = 0; i <= L; i++)
+        if (farthest[i] != 0) redundant->shift(i, -farthest[i]);
+    after(*redundant, L);
+    computation *head = redundant;
+    isl_set_free(missing);
+    chain_before_consumer(head);
+}
+
+void computation::storage_fold(var L0, int factor) {
+    if (!access) ERROR("storage_fold: " + name + " has no data mapping yet", true);
+    if (factor < 1) ERROR("storage_fold: factor must be positive", true);
+    const int d = get_loop_level_number_from_dimension_name(L0.get_name());
+    const int n = (int)isl_map_dim(access, isl_dim_out);
+    if (d < 0 || d >= n) ERROR("storage_fold: " + L0.get_name() + " is not a dimension of the buffer of " + name, true);
+    buffer *b = get_buffer();
+    b->set_dim_size(d, factor);
+    std::vector<std::string> in, out;
+    for (int i = 0; i < n; i++) {
+        in.push_back("o" + std::to_string(i));
+        out.push_back(i == d ? in.back() + " mod " + std::to_string(factor) : in.back());
+    }
+    const std::string bn = b->get_name();
+    isl_map *fold = isl_map_read_from_str(ctx, ("{ " + bn + "[" + join(in, ",") + "] -> " + bn + "[" + join(out, ",") + "] }").c_str());
+    // every definition and duplicate of this computation that stores in the buffer stores folded: the buffer has
+    // shrunk for all of them
+    computation *first = get_first_definition();
+    std::vector<computation *> all{first};
+    all.insert(all.end(), first->updates.begin(), first->updates.end());
+    all.insert(all.end(), first->duplicates.begin(), first->duplicates.end());
+    for (auto c : all)
+        if (c->access && isl_map_get_tuple_name(c->access, isl_dim_out) == bn) c->access = isl_map_apply_range(c->access, isl_map_copy(fold));
+    isl_map_free(fold);
 }
 
 void computation::gen_time_space_domain() {
