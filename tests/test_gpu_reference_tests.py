@@ -49,7 +49,7 @@ def test_transpose_gpu_tile(programs_dir):
 
 def test_gemm_register_tile(programs_dir):
     rng = np.random.RandomState(170)
-    A, B, C = ints(rng, (128, 96)), ints(rng, (96, 192)), ints(rng, (128, 192))
+    A, B, C = ints(rng, (96, 100)), ints(rng, (100, 180)), ints(rng, (96, 180))
     expected = ref.gemm_accumulate(A, B, C)
     C_cpu = C.copy()
     cpu_variant(programs_dir, "gemm_register_tile")(A, B, C_cpu)

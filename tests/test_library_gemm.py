@@ -82,9 +82,15 @@ def test_seeded_sweep_of_shapes():
         run(M, N, K, alpha, beta, tA=tA, tB=tB, pad=pad, off=off, seed=case)
 
 
-@pytest.mark.parametrize("M,N,K,tA,tB", [(70, 50, 30, False, False), (64, 96, 128, True, False), (33, 65, 17, False, True), (128, 128, 64, True, True)])
+DOUBLE_CASES = [(70, 50, 30, False, False), (64, 96, 128, True, False), (33, 65, 17, False, True), (128, 128, 64, True, True),
+                # enough 128 x 128 tiles for the large-tile kernel, ragged in M, N and K, all four transposition cases
+                (1500, 1430, 250, False, False), (1500, 1430, 250, True, False), (1500, 1430, 250, False, True), (1411, 1600, 77, True, True),
+                (1, 1, 1, False, False), (17, 3000, 5, False, False)]
+
+
+@pytest.mark.parametrize("M,N,K,tA,tB", DOUBLE_CASES)
 def test_double_precision(M, N, K, tA, tB):
-    # tiramisu_hip_dgemm (replaces tiramisu_cublas_dgemm, tiramisu_cuda_wrappers.cpp:117-162)
+    # tiramisu_hip_dgemm (replaces tiramisu_cublas_dgemm, tiramisu_cuda_wrappers.cpp:117-162): fp64 matrix instructions
     from gpu_util import DeviceArray
     rng = np.random.RandomState(M * K)
     A = rng.uniform(-1, 1, (K, M) if tA else (M, K))
@@ -94,6 +100,29 @@ def test_double_precision(M, N, K, tA, tB):
     dA, dB, dC = DeviceArray(A), DeviceArray(B), DeviceArray(C)
     runtime.wrappers().tiramisu_hip_dgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 1.5, 0.5, 0, 0, 0, 0, 0, 0, tA, tB)
     assert np.max(np.abs(dC.download() - expected)) <= 1e-12 * K
+    # integer-valued data: exact, whatever the order of the sums
+    A, B, C = np.rint(A * 8), np.rint(B * 8), np.rint(C * 8)
+    dA, dB, dC = DeviceArray(A), DeviceArray(B), DeviceArray(C)
+    runtime.wrappers().tiramisu_hip_dgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 2.0, 0.0, 0, 0, 0, 0, 0, 0, tA, tB)
+    assert np.array_equal(dC.download(), 2.0 * ((A.T if tA else A) @ (B.T if tB else B)))
+
+
+def test_double_precision_leading_dimensions_and_offsets():
+    # operands inside larger allocations: leading dimensions wider than the rows, element offsets, beta = 1
+    from gpu_util import DeviceArray
+    rng = np.random.RandomState(9)
+    M, N, K, lda, ldb, ldc, oa, ob, oc = 90, 70, 40, 47, 75, 80, 5, 11, 3
+    bufA = np.rint(rng.uniform(-4, 4, oa + M * lda))
+    bufB = np.rint(rng.uniform(-4, 4, ob + K * ldb))
+    bufC = np.rint(rng.uniform(-4, 4, oc + M * ldc))
+    A = bufA[oa:oa + M * lda].reshape(M, lda)[:, :K]
+    B = bufB[ob:ob + K * ldb].reshape(K, ldb)[:, :N]
+    expected = bufC.copy()
+    view = expected[oc:oc + M * ldc].reshape(M, ldc)
+    view[:, :N] = -1.0 * (A @ B) + view[:, :N]
+    dA, dB, dC = DeviceArray(bufA), DeviceArray(bufB), DeviceArray(bufC)
+    runtime.wrappers().tiramisu_hip_dgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, -1.0, 1.0, lda, ldb, ldc, oa, ob, oc, False, False)
+    assert np.array_equal(dC.download(), expected)         # the padding between rows is untouched
 
 
 def test_freed_device_blocks_are_reused():

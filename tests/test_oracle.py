@@ -87,7 +87,7 @@ def test_cpu_transpose():
 
 def test_cpu_gemm_register_tile():
     rng = np.random.RandomState(170)
-    A, B, C = ints(rng, (128, 96)), ints(rng, (96, 192)), ints(rng, (128, 192))
+    A, B, C = ints(rng, (96, 100)), ints(rng, (100, 180)), ints(rng, (96, 180))
     expected = ref.gemm_accumulate(A, B, C)
     cpu_program("gemm_register_tile")(A, B, C)
     assert np.array_equal(C, expected)

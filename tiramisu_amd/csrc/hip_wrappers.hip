@@ -19,6 +19,7 @@
 
 #include "../../include/tiramisu_hip_wrappers.h"
 #include "kernels/gemm_mfma.hip.h"
+#include "kernels/gemm_mfma_f64.hip.h"
 #include "kernels/target_gfx950.h"
 
 namespace {
@@ -348,6 +349,36 @@ void dispatch_edge(bool edge, const float *A, const float *B, float *C, int M, i
     else dispatch_tile<AK, BK_, false>(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, vec_ok);
 }
 
+template <class S, bool A_KFAST, bool B_NFAST>
+void launch_dgemm_kernel(const double *A, const double *B, double *C, int M, int N, int K, long sam, long sak, long sbk, long sbn, long ldc,
+                                double alpha, double beta) {
+    auto kernel = tgemm64::dgemm_kernel<S, A_KFAST, B_NFAST>;
+    // the large tile's two LDS stages exceed the 64 KiB that a launch gets without asking (once per device)
+    static std::atomic<unsigned long long> asked{0};
+    if (S::LDS_BYTES > 64 * 1024) {
+        int device = 0;
+        check(hipGetDevice(&device), "tiramisu_hip_dgemm");
+        const unsigned long long bit = 1ull << (device & 63);
+        if (!(asked.load() & bit)) {
+            check(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES), "tiramisu_hip_dgemm");
+            asked.fetch_or(bit);
+        }
+    }
+    const unsigned tiles = (unsigned)(((M + S::BM - 1) / S::BM) * ((N + S::BN - 1) / S::BN));
+    hipLaunchKernelGGL(kernel, dim3(tiles), dim3(S::NT), S::LDS_BYTES, current_stream, A, B, C, M, N, K, sam, sak, sbk, sbn, ldc, alpha, beta);
+    check(hipGetLastError(), "tiramisu_hip_dgemm");
+}
+
+template <class S>
+void launch_dgemm(bool transposeA, bool transposeB, const double *A, const double *B, double *C, int M, int N, int K, long sam, long sak,
+                         long sbk, long sbn, long ldc, double alpha, double beta) {
+    // A's k is the unit stride unless A is transposed; B's n is unless B is transposed
+    if (!transposeA && !transposeB) launch_dgemm_kernel<S, true, true>(A, B, C, M, N, K, sam, sak, sbk, sbn, ldc, alpha, beta);
+    else if (!transposeA && transposeB) launch_dgemm_kernel<S, true, false>(A, B, C, M, N, K, sam, sak, sbk, sbn, ldc, alpha, beta);
+    else if (transposeA && !transposeB) launch_dgemm_kernel<S, false, true>(A, B, C, M, N, K, sam, sak, sbk, sbn, ldc, alpha, beta);
+    else launch_dgemm_kernel<S, false, false>(A, B, C, M, N, K, sam, sak, sbk, sbn, ldc, alpha, beta);
+}
+
 }  // namespace
 
 extern "C" {
@@ -537,12 +568,15 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
         fprintf(stderr, "Error at %s: dimension exceeds 2^31-1\n", __FUNCTION__);
         exit(1);
     }
-    dim3 blk(16, 16), grd((unsigned)((N + 15) / 16), (unsigned)((M + 15) / 16));
-    hipLaunchKernelGGL(gemm_generic_kernel<double>, grd, blk, 0, current_stream, (const double *)(A + offsetA),
-                       (const double *)(B + offsetB), C + offsetC, (int)M, (int)N, (int)K,
-                       transposeA ? 1L : (long)ldA, transposeA ? (long)ldA : 1L, transposeB ? 1L : (long)ldB,
-                       transposeB ? (long)ldB : 1L, (long)ldC, alpha, beta);
-    check(hipGetLastError(), __FUNCTION__);
+    const double *a = A + offsetA, *b = B + offsetB;
+    double *c = C + offsetC;
+    // element (m, k) of op(A) and (k, n) of op(B) through two strides each
+    const long sam = transposeA ? 1L : (long)ldA, sak = transposeA ? (long)ldA : 1L;
+    const long sbk = transposeB ? 1L : (long)ldB, sbn = transposeB ? (long)ldB : 1L;
+    // 128 x 128 tiles when they give every compute unit work, else 64 x 64
+    const long big = (long)((M + 127) / 128) * (long)((N + 127) / 128);
+    if (big >= ttarget::COMPUTE_UNITS / 2) launch_dgemm<tgemm64::shape<4, 2, 2, 4>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
+    else launch_dgemm<tgemm64::shape<2, 2, 2, 2>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
     return 0;
 }
 
