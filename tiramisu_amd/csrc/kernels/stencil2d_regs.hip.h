@@ -63,15 +63,17 @@
 #define TIRAMISU_AMD_STENCIL2D_REGS_COMMON
 typedef float st_f4 __attribute__((ext_vector_type(4)));
 
-// lane i receives lane i-1's value (lane 0 keeps its own)
+// lane i receives lane i-1's value; lane 0, which has no such neighbour, reads 0 (its cells next to the region's
+// edge are stale from the first step on and never written).  With nothing to keep for the lanes out of range, the
+// compiler folds the shift into the add that consumes it (v_add_f32_dpp) instead of issuing a move.
 __device__ __forceinline__ float st_from_left(float v) {
     const int i = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, 0x138 /* wave_shr:1 */, 0xf, 0xf, true));
 }
-// lane i receives lane i+1's value (lane 63 keeps its own)
+// lane i receives lane i+1's value; lane 63 reads 0
 __device__ __forceinline__ float st_from_right(float v) {
     const int i = __builtin_bit_cast(int, v);
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, i, 0x130 /* wave_shl:1 */, 0xf, 0xf, true));
 }
 
 // Four cells of row gy starting at column gx (a multiple of 4) of a plane of NY x NX cells;
@@ -145,34 +147,20 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
         }
 #pragma unroll
         for (int r = 0; r < RPT; r++) ext[ST_RAD + r] = cur[r];
-        // the ST_RAD cells left and right of every quad, from the adjacent lanes
-        float lf[RPT + 2 * ST_RAD][ST_RAD], rt[RPT + 2 * ST_RAD][ST_RAD];
-#pragma unroll
-        for (int j = 0; j < RPT + 2 * ST_RAD; j++)
-#pragma unroll
-            for (int i = 0; i < ST_RAD; i++) {
-                lf[j][i] = st_from_left(ext[j][4 - ST_RAD + i]);
-                rt[j][i] = st_from_right(ext[j][i]);
-            }
 #pragma unroll
         for (int r = 0; r < RPT; r++) {
-            // window of old values around the quad: rows -RAD..RAD, columns -RAD..3+RAD
-            float w[2 * ST_RAD + 1][4 + 2 * ST_RAD];
-#pragma unroll
-            for (int dy = -ST_RAD; dy <= ST_RAD; dy++) {
-                const int j = r + ST_RAD + dy;
-#pragma unroll
-                for (int e = 0; e < 4; e++) w[dy + ST_RAD][ST_RAD + e] = ext[j][e];
-#pragma unroll
-                for (int i = 0; i < ST_RAD; i++) {
-                    w[dy + ST_RAD][i] = lf[j][i];
-                    w[dy + ST_RAD][ST_RAD + 4 + i] = rt[j][i];
-                }
-            }
+            // Old value at row r + dy, column e + dx of the quad (columns -RAD .. 3 + RAD): columns outside the quad
+            // come from the adjacent lane.  The shift is written where the value is used, once per use: the compiler
+            // folds a lane shift into the add that consumes it (v_add_f32_dpp) only when the two are a few
+            // instructions apart, and a shift folded that way costs no instruction.
+            auto old_at = [&](int dy, int col) -> float {
+                const st_f4 &row = ext[r + ST_RAD + dy];
+                return col < 0 ? st_from_left(row[4 + col]) : col > 3 ? st_from_right(row[col - 4]) : row[col];
+            };
             const bool row_in = !EDGE || (gy0 + r >= ST_Y0 && gy0 + r <= ST_Y1);
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-#define ST_AT(dy, dx) w[(dy) + ST_RAD][e + (dx) + ST_RAD]
+#define ST_AT(dy, dx) old_at((dy), e + (dx))
                 const float computed = (ST_EXPR);
 #undef ST_AT
                 if (EDGE) {

@@ -9,6 +9,8 @@
 // vectorize x by 8.  One generated function per (N, STEPS) instance: heat2d_<N>x<STEPS>.
 #include <tiramisu/tiramisu.h>
 
+#include <cstdlib>
+
 using namespace tiramisu;
 
 static void generate(int N, int STEPS)
@@ -40,6 +42,7 @@ static void generate(int N, int STEPS)
 int main()
 {
     generate(8192, 32);   // the benchmark configuration
+    if (std::getenv("HEAT2D_ONLY_FULL")) return 0;   // for sweeps over the emitter's knobs
     generate(1024, 8);
     generate(1030, 9);    // rows not a multiple of 4 elements with interior tiles: unaligned strips
     generate(256, 1);

@@ -13,6 +13,8 @@
 // One generated function per size: sgemm_<M>x<N>x<K>.
 #include <tiramisu/tiramisu.h>
 
+#include <cstdlib>
+
 using namespace tiramisu;
 
 static void generate(int M, int N, int K)
@@ -75,6 +77,11 @@ static void generate(int M, int N, int K)
 
 int main()
 {
+    // SGEMM_ONLY_CUBE=<n>: only the n x n x n instance (for sweeps over the emitter's knobs)
+    if (const char *n = std::getenv("SGEMM_ONLY_CUBE")) {
+        generate(std::atoi(n), std::atoi(n), std::atoi(n));
+        return 0;
+    }
     generate(1024, 1024, 1024);   // benchmark configuration 1
     generate(4096, 4096, 4096);   // benchmark configuration 3 (fp32)
     generate(256, 256, 64);
