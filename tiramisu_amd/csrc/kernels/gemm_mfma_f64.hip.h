@@ -25,9 +25,9 @@ namespace tgemm64 {
 
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 
-constexpr int BK = 16, PAD = 4;
+constexpr int BK = 16;
 
-template <int TM_, int TN_, int WGM_, int WGN_>
+template <int TM_, int TN_, int WGM_, int WGN_, int PAD = 4>
 struct shape {
     static constexpr int TM = TM_, TN = TN_, WGM = WGM_, WGN = WGN_;
     static constexpr int NT = 64 * WGM * WGN;
@@ -39,9 +39,11 @@ struct shape {
     static_assert((BM * BK) % NT == 0 && (BN * BK) % NT == 0, "slice parts divide over the threads");
 };
 
+// The second launch bound (wavefronts per SIMD) holds the kernel to the registers that let two workgroups share a
+// compute unit: at 136 registers instead of 128 a single workgroup is resident and the kernel is a quarter slower.
 // A_KFAST: consecutive k of A are adjacent in memory (stride_ak == 1), else consecutive m are; likewise B_NFAST.
 template <class S, bool A_KFAST, bool B_NFAST>
-__global__ void __launch_bounds__(S::NT) dgemm_kernel(const double *__restrict__ A, const double *__restrict__ B, double *__restrict__ C, int M, int N,
+__global__ void __launch_bounds__(S::NT, S::NT / 128) dgemm_kernel(const double *__restrict__ A, const double *__restrict__ B, double *__restrict__ C, int M, int N,
                                                    int K, long stride_am, long stride_ak, long stride_bk, long stride_bn, long ldc, double alpha,
                                                    double beta) {
     constexpr int TM = S::TM, TN = S::TN, NT = S::NT;
