@@ -6,6 +6,8 @@
 // sgemm_bf16_<M>x<N>x<K>.
 #include <tiramisu/tiramisu.h>
 
+#include <cstdlib>
+
 using namespace tiramisu;
 
 static void generate(int M, int N, int K)
@@ -69,6 +71,7 @@ static void generate(int M, int N, int K)
 int main()
 {
     generate(4096, 4096, 4096);   // benchmark configuration 3, bf16-input variant
+    if (std::getenv("SGEMM_BF16_ONLY_FULL")) return 0;   // for sweeps over the emitter's knobs
     generate(4096, 3072, 32);     // 256x256 tiles, a single K-slice
     generate(3072, 4096, 160);    // 256x256 tiles, five K-slices: one steady-state turn of the four-stage ring, then the drain
     generate(1024, 1280, 512);    // 128x128 tiles
