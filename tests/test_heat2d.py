@@ -30,6 +30,21 @@ def cpu_program(n, steps):
 
 # ---------------------------------------------------------------- oracle pins (no GPU)
 
+def test_launch_plan_of_the_full_size_program():
+    """32 steps are three launches: odd chunks between the two planes, the last of them into a third plane,
+    and a final launch that writes the last step and the last but one into the two planes."""
+    import json
+    import re
+    base = os.path.join(PROGRAMS, "build", "heat2d_8192x32.o")
+    ranges = [(int(a), int(b)) for a, b in re.findall(r"_st_src = \d+;  // steps (\d+)\.\.(\d+)", open(base + ".host.cpp").read())]
+    assert ranges[0][0] == 1 and ranges[-1][1] == 32 and len(ranges) == 3
+    assert all(a[1] + 1 == b[0] for a, b in zip(ranges, ranges[1:]))
+    assert all((b - a + 1) % 2 == 1 for a, b in ranges[:-1])
+    hows = [k["how"] for k in json.load(open(base + ".json"))["kernels"] if "interior tiles" in k["how"]]
+    assert sum("into a third plane" in h and "from" not in h for h in hows) == 1
+    assert sum("from a third plane into both planes" in h for h in hows) == 1
+
+
 def test_oracle_matches_python_loops():
     g = initial_grid(9, 1)
     assert np.array_equal(ref.heat2d(g, 3), ref.heat2d_loops(g, 3))
@@ -93,9 +108,10 @@ def test_gpu_matches_oracle(n, steps):
 
 
 @pytest.mark.gpu
-def test_gpu_boundaries_of_both_planes_are_respected():
-    # the two planes hold different fixed boundary values: even steps read plane 1's boundary
-    n, steps = 66, 7
+@pytest.mark.parametrize("n,steps", [(66, 7), (130, 4), (1030, 9), (20, 2)])
+def test_gpu_boundaries_of_both_planes_are_respected(n, steps):
+    # the two planes hold different fixed boundary values: even steps read plane 1's boundary (with three
+    # steps or more the launches go through a third plane, which has to show the right plane's fixed cells)
     rng = np.random.RandomState(5)
     planes = rng.uniform(0, 1, (2, n, n)).astype(np.float32)
     expected = ref.heat2d(planes[0], steps, boundary_other=planes[1])

@@ -8,7 +8,7 @@ import glob
 import os
 import re
 
-SIGNATURE = re.compile(r'^extern "C" __global__ void __launch_bounds__\((\d+)\)\s*(?:__attribute__\(\([^)]*\)\)\s*)?(_kernel_(\d+))\(([^)]*)\)', re.M)
+SIGNATURE = re.compile(r'^extern "C" __global__ void __launch_bounds__\((\d+)(?:, \d+)?\)\s*(?:__attribute__\(\([^)]*\)\)\s*)?(_kernel_(\d+))\(([^)]*)\)', re.M)
 
 
 def kernels_of(path):

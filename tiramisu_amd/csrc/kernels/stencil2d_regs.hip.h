@@ -23,15 +23,24 @@
 // fixed cells keeps the other plane's values of its strip in registers (read once; no launch ever
 // writes those cells) and swaps the two values of a fixed cell at every step.  That costs registers
 // and checks, so each launch is split in two kernels: ST_NAME for the tiles whose staged region
-// lies inside the iteration domain (no checks at all), ST_NAME_EDGE for the others.  Both read
-// plane `src` and write plane `1-src` (disjoint cells), which requires ST_R to be odd; the host
-// code composes the time loop from odd chunks.
+// lies inside the iteration domain (no checks at all), ST_NAME_EDGE for the others.
+//
+// Where the values come from and go to (ST_MODE), `p` being the plane that holds the source step:
+//   0  read plane p, write plane 1-p (disjoint cells): ST_R must be odd;
+//   1  read plane p, write a third plane `temp` that stands in for plane 1-p (ST_R odd), fixed cells included,
+//      so that a later launch finds there all it reads;
+//   2  read `temp` (standing in for plane p) and write both planes: the values after ST_R - 1 steps to the plane
+//      of that step's parity and those after ST_R steps to the other one.  Neither plane is read except for its
+//      fixed cells, so ST_R may be even and the time loop can end with a fused launch that leaves both planes
+//      exactly as the un-tiled loop does.
+// The host code composes the time loop from such launches.
 //
 // Macros supplied by the emitter before this file is included:
 //   ST_NAME            kernel name
 //   ST_NY, ST_NX       plane extents (rows, columns)
 //   ST_Y0, ST_Y1, ST_X0, ST_X1   inclusive bounds of the iteration domain
-//   ST_R               time steps fused in one launch (odd)
+//   ST_R               time steps fused in one launch
+//   ST_MODE            0, 1 or 2: see above
 //   ST_RAD             stencil radius (<= 4, <= ST_RPT)
 //   ST_W               wavefronts per workgroup
 //   ST_RPT             rows per thread
@@ -58,6 +67,15 @@
 #define ST_TW (ST_LW - 2 * ST_HX)
 #define ST_CAT2(a, b) a##b
 #define ST_CAT(a, b) ST_CAT2(a, b)
+
+// The planes of a launch.  Plane src_plane holds (or `temp` stands in for) the source step; after ST_R steps the
+// values belong in plane (src_plane + ST_R) % 2.
+#define ST_PLANE(p) (planes + (size_t)(p) * ST_NY * ST_NX)
+#define ST_PLANES                                                                                              \
+    const float *__restrict__ src = ST_MODE == 2 ? temp : ST_PLANE(src_plane);                                 \
+    float *__restrict__ dst = ST_MODE == 1 ? temp : ST_PLANE((src_plane + ST_R) & 1);                          \
+    float *__restrict__ dst_prev = ST_MODE == 2 ? ST_PLANE((src_plane + ST_R - 1) & 1) : nullptr;              \
+    const float *fixed_other = ST_PLANE(1 - src_plane);
 
 #ifndef TIRAMISU_AMD_STENCIL2D_REGS_COMMON
 #define TIRAMISU_AMD_STENCIL2D_REGS_COMMON
@@ -103,9 +121,11 @@ __device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx
 
 // One workgroup advances the region of ST_W*RPT rows whose centre starts at plane row `oy`, column
 // `ox`, and writes the centre rows below `row_end`.
+// `fixed_other`: the plane whose fixed cells show at the steps of the other parity than the source's; `dst_prev`:
+// where the values of the last step but one go (mode 2 only).
 template <bool EDGE, int RPT>
-__device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int oy, int ox,
-                                                        int row_end) {
+__device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict__ src, float *__restrict__ dst, float *__restrict__ dst_prev,
+                                                        const float *fixed_other, st_f4 *xch, int oy, int ox, int row_end) {
     // values stay in registers from one step to the next: without this the multiply that ends a
     // step would be fused with an add of the next one, and results would differ from the
     // un-tiled program's
@@ -121,7 +141,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
 #pragma unroll
     for (int r = 0; r < RPT; r++) {
         cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
-        if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(dst, gy0 + r, gx);
+        if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(fixed_other, gy0 + r, gx);
     }
 
     // xch[parity][wave][top|bottom][row][lane]
@@ -129,9 +149,32 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
         return xch + ((((parity * ST_W + w) * 2 + side) * ST_RAD + i) * 64 + lane);
     };
 
+    // ---- write the tile centre: the cells of the domain, or in mode 1 all cells of the plane (a fixed cell then
+    // holds the value of the plane that `to` stands in for)
+    constexpr int WY0 = ST_MODE == 1 ? 0 : ST_Y0, WY1 = ST_MODE == 1 ? ST_NY - 1 : ST_Y1;
+    constexpr int WX0 = ST_MODE == 1 ? 0 : ST_X0, WX1 = ST_MODE == 1 ? ST_NX - 1 : ST_X1;
+    auto store_centre = [&](float *__restrict__ to) {
+        if (4 * lane >= ST_HX && 4 * lane < ST_HX + ST_TW) {
+#pragma unroll
+            for (int r = 0; r < RPT; r++) {
+                const int row = wave * RPT + r, gy = gy0 + r;
+                if (row < ST_HY || row >= ST_HY + CENTRE_ROWS || gy >= row_end) continue;
+                if (EDGE && (gy < WY0 || gy > WY1)) continue;
+                if ((ST_NX % 4 == 0) && (!EDGE || (gx >= WX0 && gx + 3 <= WX1))) {
+                    *reinterpret_cast<st_f4 *>(to + (size_t)gy * ST_NX + gx) = cur[r];
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (!EDGE || (gx + e >= WX0 && gx + e <= WX1)) to[(size_t)gy * ST_NX + gx + e] = cur[r][e];
+                }
+            }
+        }
+    };
+
 #pragma unroll
     for (int s = 1; s <= ST_R; s++) {
         const int parity = s & 1;
+        if (ST_MODE == 2 && s == ST_R) store_centre(dst_prev);   // the values after ST_R - 1 steps
 #pragma unroll
         for (int i = 0; i < ST_RAD; i++) {
             *slot(parity, wave, 0, i) = cur[i];
@@ -176,22 +219,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
         }
     }
 
-    // ---- write the tile centre (cells of the domain only)
-    if (4 * lane >= ST_HX && 4 * lane < ST_HX + ST_TW) {
-#pragma unroll
-        for (int r = 0; r < RPT; r++) {
-            const int row = wave * RPT + r, gy = gy0 + r;
-            if (row < ST_HY || row >= ST_HY + CENTRE_ROWS || gy >= row_end) continue;
-            if (EDGE && (gy < ST_Y0 || gy > ST_Y1)) continue;
-            if ((ST_NX % 4 == 0) && (!EDGE || (gx >= ST_X0 && gx + 3 <= ST_X1))) {
-                *reinterpret_cast<st_f4 *>(dst + (size_t)gy * ST_NX + gx) = cur[r];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (!EDGE || (gx + e >= ST_X0 && gx + e <= ST_X1)) dst[(size_t)gy * ST_NX + gx + e] = cur[r][e];
-            }
-        }
-    }
+    store_centre(dst);
 }
 
 // The tiles outside the interior rectangle, in the order: full tile rows above the interior
@@ -201,7 +229,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
 // strip) instead of one heavy workgroup per tile.  eb is the index of the slice.
 #define ST_TH_EDGE (ST_W * ST_RPT_EDGE - 2 * ST_HY)
 #define ST_EDGE_SUB ((ST_TH + ST_TH_EDGE - 1) / ST_TH_EDGE)
-static __device__ __forceinline__ void ST_CAT(ST_NAME, _edge_slice)(const float *__restrict__ src, float *__restrict__ dst, st_f4 *xch, int eb)
+static __device__ __forceinline__ void ST_CAT(ST_NAME, _edge_slice)(const float *__restrict__ src, float *__restrict__ dst,
+                                                                     float *__restrict__ dst_prev, const float *fixed_other, st_f4 *xch, int eb)
 {
     constexpr int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
     constexpr int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
@@ -220,7 +249,7 @@ static __device__ __forceinline__ void ST_CAT(ST_NAME, _edge_slice)(const float 
         by = ST_IBY0 + e / (SIDE > 0 ? SIDE : 1);
         bx = c < ST_IBX0 ? c : ST_IBX1 + 1 + (c - ST_IBX0);
     }
-    ST_CAT(ST_NAME, _sweep)<true, ST_RPT_EDGE>(src, dst, xch, by * ST_TH + sub * ST_TH_EDGE, bx * ST_TW, (by + 1) * ST_TH);
+    ST_CAT(ST_NAME, _sweep)<true, ST_RPT_EDGE>(src, dst, dst_prev, fixed_other, xch, by * ST_TH + sub * ST_TH_EDGE, bx * ST_TW, (by + 1) * ST_TH);
 }
 
 // Interior tiles: one workgroup per tile of the rectangle [ST_IBX0, ST_IBX1] x [ST_IBY0, ST_IBY1],
@@ -233,16 +262,16 @@ extern "C" __global__ void __launch_bounds__(64 * ST_W)
 #if ST_OCC > 0
 __attribute__((amdgpu_waves_per_eu(ST_OCC)))
 #endif
-ST_NAME(float *__restrict__ planes, const int src_plane)
+ST_NAME(float *planes, const int src_plane, float *temp)
 {
     static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
+    static_assert(ST_MODE == 2 ? ST_R >= 2 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
     __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
-    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
-    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
+    ST_PLANES
     const int b = blockIdx.x;
 #if ST_MERGE
     if (b >= ST_NI) {
-        ST_CAT(ST_NAME, _edge_slice)(src, dst, xch, b - ST_NI);
+        ST_CAT(ST_NAME, _edge_slice)(src, dst, dst_prev, fixed_other, xch, b - ST_NI);
         return;
     }
 #endif
@@ -257,22 +286,23 @@ ST_NAME(float *__restrict__ planes, const int src_plane)
 #else
     const int tile = b;
 #endif
-    ST_CAT(ST_NAME, _sweep)<false, ST_RPT>(src, dst, xch, (ST_IBY0 + tile / IW) * ST_TH, (ST_IBX0 + tile % IW) * ST_TW, ST_NY);
+    ST_CAT(ST_NAME, _sweep)<false, ST_RPT>(src, dst, dst_prev, fixed_other, xch, (ST_IBY0 + tile / IW) * ST_TH, (ST_IBX0 + tile % IW) * ST_TW, ST_NY);
 }
 
 // The edge slices as a launch of their own (used when the launches are not merged).
 extern "C" __global__ void __launch_bounds__(64 * ST_W)
-ST_NAME_EDGE(float *__restrict__ planes, const int src_plane)
+ST_NAME_EDGE(float *planes, const int src_plane, float *temp)
 {
     __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
-    const float *__restrict__ src = planes + (size_t)src_plane * ST_NY * ST_NX;
-    float *__restrict__ dst = planes + (size_t)(1 - src_plane) * ST_NY * ST_NX;
-    ST_CAT(ST_NAME, _edge_slice)(src, dst, xch, blockIdx.x);
+    ST_PLANES
+    ST_CAT(ST_NAME, _edge_slice)(src, dst, dst_prev, fixed_other, xch, blockIdx.x);
 }
 #undef ST_NI
 #undef ST_TH_EDGE
 #undef ST_EDGE_SUB
 
+#undef ST_PLANE
+#undef ST_PLANES
 #undef ST_HY
 #undef ST_HX
 #undef ST_LH

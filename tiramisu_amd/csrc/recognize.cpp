@@ -177,47 +177,81 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     if (!literal_box(S, lo, hi)) return false;
     if (lo[1] - radius < 0 || hi[1] + radius > NY - 1 || lo[2] - radius < 0 || hi[2] + radius > NX - 1) return false;
 
-    // ---- plan: odd chunks for all steps but the last, then the last step alone, so that on
-    // return both planes hold exactly what the un-tiled loop leaves there
+    // ---- plan.  On return both planes must hold exactly what the un-tiled loop leaves there: the last step in
+    // one, the last but one in the other.  A launch between the two planes advances an odd number of steps.
+    //  * With a third plane (allocated once per host thread, kept): odd chunks between the planes, the last of
+    //    them into the third plane, and a final launch that reads the third plane and writes both planes (the
+    //    values of its last step but one and of its last step), so no launch is spent on a single step.
+    //  * Without (fewer than 3 steps, or TIRAMISU_STENCIL_TEMP_PLANE=0): odd chunks for all steps but the last,
+    //    then the last step alone.
     const long T0 = lo[0], T1 = hi[0];
     const long steps = T1 - T0 + 1;
     // region staged by one workgroup: WAVES*ROWS rows by 256 columns (kernels/stencil2d_regs.hip.h)
     const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", 11);
     if (WAVES < 1 || WAVES > 16 || ROWS < radius || ROWS > 32) return false;
     const int LH = WAVES * ROWS, LW = 256;
-    int rmax = env_int("TIRAMISU_STENCIL_STEPS", 11);
+    // most steps of one launch; a launch between the two planes takes the largest odd number below.  12: the final
+    // launch writes two planes and has HBM time to cover one step more than the 11 of the others
+    int rcap = env_int("TIRAMISU_STENCIL_STEPS", 12);
     // keep at least half of the staged rows and columns as the tile
-    while (rmax > 1 && (4 * rmax * radius > LH || 4 * ((rmax * radius + 3) / 4 * 4) > LW)) rmax -= 1;
-    if (rmax % 2 == 0) rmax -= 1;
-    if (rmax < 1) rmax = 1;
+    while (rcap > 1 && (4 * rcap * radius > LH || 4 * ((rcap * radius + 3) / 4 * 4) > LW)) rcap -= 1;
+    if (rcap < 1) rcap = 1;
+    const int rmax = rcap % 2 == 0 ? rcap - 1 : rcap;
     if (2 * radius >= LH) return false;
-    std::vector<std::pair<long, int>> chunks;  // (first step, number of steps)
-    long t = T0, rem = steps - 1;
-    while (rem > 0) {
-        int c = (int)std::min<long>(rmax, rem);
-        if (c % 2 == 0) c -= 1;
-        chunks.push_back({t, c});
-        t += c;
-        rem -= c;
+    struct chunk { long first; int steps; int mode; };   // first step, number of steps, kernel mode (stencil2d_regs.hip.h)
+    auto odd_chunks = [&](long first, long count) {
+        std::vector<chunk> out;
+        while (count > 0) {
+            int c = (int)std::min<long>(rmax, count);
+            if (c % 2 == 0) c -= 1;
+            out.push_back({first, c, 0});
+            first += c;
+            count -= c;
+        }
+        return out;
+    };
+    std::vector<chunk> chunks;
+    const bool temp_plane = steps >= 3 && env_int("TIRAMISU_STENCIL_TEMP_PLANE", 1) != 0;
+    if (temp_plane) {
+        // the final launch's length: the one that needs the fewest launches (the longest of those)
+        int best = 2;
+        size_t best_n = 0;
+        for (int fin = (int)std::min<long>(rcap, steps - 1); fin >= 2; fin--) {
+            const size_t n = odd_chunks(T0, steps - fin).size();
+            if (best_n == 0 || n < best_n) { best = fin; best_n = n; }
+        }
+        chunks = odd_chunks(T0, steps - best);
+        chunks.back().mode = 1;
+        chunks.push_back({T0 + steps - best, best, 2});
+    } else {
+        chunks = odd_chunks(T0, steps - 1);
+        chunks.push_back({T0 + steps - 1, 1, 0});
     }
-    chunks.push_back({t, 1});
 
     c_printer dev;
     dev.fct = f;
     dev.device = true;
     const std::string point_text = dev.print(point);
-    std::map<int, std::pair<kernel, kernel>> by_steps;   // (interior tiles, tiles on the fixed boundary)
+    std::map<std::pair<int, int>, std::pair<kernel, kernel>> by_steps;   // (steps, mode) -> (interior tiles, tiles on the fixed boundary)
     std::ostringstream host;
     auto ceil_div = [](long a, long b) { return a >= 0 ? (a + b - 1) / b : -((-a) / b); };
     auto floor_div = [](long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); };
     // one launch per chunk: the boundary slices ride behind the interior tiles (TIRAMISU_STENCIL_MERGE=0: two launches)
     const bool merge = env_int("TIRAMISU_STENCIL_MERGE", 1) != 0;
+    static const char *const mode_text[] = {"", ", into a third plane", ", from a third plane into both planes"};
+    host << "    {\n";
+    if (temp_plane)
+        host << "        static thread_local float *_st_temp = nullptr;   // third plane: allocated at the first call, kept\n"
+             << "        if (!_st_temp) _st_temp = (float *)tiramisu_hip_malloc((uint64_t)" << NY << " * " << NX << " * sizeof(float));\n";
+    else
+        host << "        float *_st_temp = nullptr;\n";
     for (auto &ch : chunks) {
-        if (!by_steps.count(ch.second)) {
+        const std::pair<int, int> key(ch.steps, ch.mode);
+        if (!by_steps.count(key)) {
             kernel k, ke;
             k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
             ke.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
-            const int HY = ch.second * radius, HX = (ch.second * radius + 3) / 4 * 4;
+            const int HY = ch.steps * radius, HX = (ch.steps * radius + 3) / 4 * 4;
             const int TH = LH - 2 * HY, TW = LW - 2 * HX;
             const long GX = (NX + TW - 1) / TW, GY = (NY + TH - 1) / TH;
             // tiles whose staged region [b*T - H, b*T - H + L) lies inside the iteration domain
@@ -229,9 +263,9 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
             int rows_edge = ROWS / 2;
             if (rows_edge < radius || WAVES * rows_edge - 2 * HY < 8) rows_edge = ROWS;
             const int TH_edge = WAVES * rows_edge - 2 * HY, edge_sub = (TH + TH_edge - 1) / TH_edge;
-            k.how = "stencil: " + std::to_string(ch.second) + " time step(s) per launch, radius " + std::to_string(radius) +
+            k.how = "stencil: " + std::to_string(ch.steps) + " time step(s) per launch, radius " + std::to_string(radius) +
                     ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + " in registers, " + std::to_string(WAVES) +
-                    " wavefronts x " + std::to_string(ROWS) + " rows, " + std::to_string(interior) + " interior tiles";
+                    " wavefronts x " + std::to_string(ROWS) + " rows, " + std::to_string(interior) + " interior tiles" + mode_text[ch.mode];
             ke.how = "stencil: the " + std::to_string(edge_tiles) + " tiles of " + k.name + "'s launch that touch the fixed boundary, in " +
                      std::to_string(edge_sub) + " slice(s) of " + std::to_string(TH_edge) + " rows each" +
                      (merge ? " (carried by " + k.name + "'s launch, after its interior tiles)" : "");
@@ -241,28 +275,29 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
               << "\n#define ST_GX " << GX << "\n#define ST_GY " << GY << "\n#define ST_IBX0 " << bx0 << "\n#define ST_IBX1 " << bx1
               << "\n#define ST_IBY0 " << by0 << "\n#define ST_IBY1 " << by1 << "\n#define ST_W " << WAVES
               << "\n#define ST_MERGE " << (merge ? 1 : 0) << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0)
-              << "\n#define ST_RPT " << ROWS << "\n#define ST_RPT_EDGE " << rows_edge << "\n#define ST_R " << ch.second << "\n#define ST_RAD " << radius
+              << "\n#define ST_RPT " << ROWS << "\n#define ST_RPT_EDGE " << rows_edge << "\n#define ST_R " << ch.steps << "\n#define ST_MODE " << ch.mode << "\n#define ST_RAD " << radius
               << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
               << "#undef ST_NAME\n#undef ST_NAME_EDGE\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n"
               << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n"
-              << "#undef ST_MERGE\n#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_RAD\n#undef ST_EXPR\n";
+              << "#undef ST_MERGE\n#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_MODE\n#undef ST_RAD\n#undef ST_EXPR\n";
             k.source = s.str();            // both kernels come from the one inclusion
             ke.source = "";
             for (kernel *q : {&k, &ke}) {
-                q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}};
+                q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}, {true, "_st_temp", p_float32}};
                 q->block[0] = std::to_string(64 * WAVES);
             }
             k.grid[0] = std::to_string(merge ? interior + edge_tiles * edge_sub : interior);
             ke.grid[0] = std::to_string(merge ? 0 : edge_tiles * edge_sub);
-            by_steps[ch.second] = {k, ke};
+            by_steps[key] = {k, ke};
         }
         const long src = (((ch.first - 1) % 2) + 2) % 2;
-        auto &pr = by_steps[ch.second];
-        host << "    {\n        const int32_t _st_src = " << src << ";  // steps " << ch.first << ".." << ch.first + ch.second - 1 << "\n";
-        if (pr.first.grid[0] != "0") host << launch_text(pr.first, "        ");
-        if (pr.second.grid[0] != "0") host << launch_text(pr.second, "        ");
-        host << "    }\n";
+        auto &pr = by_steps[key];
+        host << "        {\n            const int32_t _st_src = " << src << ";  // steps " << ch.first << ".." << ch.first + ch.steps - 1 << "\n";
+        if (pr.first.grid[0] != "0") host << launch_text(pr.first, "            ");
+        if (pr.second.grid[0] != "0") host << launch_text(pr.second, "            ");
+        host << "        }\n";
     }
+    host << "    }\n";
     for (auto &kv : by_steps) { plan.kernels.push_back(kv.second.first); plan.kernels.push_back(kv.second.second); }
     plan.host_code = host.str();
     return true;
@@ -1623,7 +1658,10 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         // scratch for the pieces of the last round's tiles and their counters: one block per host thread (calls
         // work on the thread's current stream), allocated at the first call and kept; the counters start at zero
         // and every launch leaves them at zero
-        k.params.push_back({true, "_tail_scratch", p_float32});
+        // (buffer parameters stay sorted by name)
+        auto at = k.params.begin();
+        while (at != k.params.end() && (!at->is_buffer || at->name < "_tail_scratch")) ++at;
+        k.params.insert(at, {true, "_tail_scratch", p_float32});
         k.grid[0] = std::to_string(win_grid);
         host << "        static thread_local float *_tail_scratch = nullptr;\n";
         host << "        if (!_tail_scratch) {\n";
