@@ -58,8 +58,13 @@ __device__ __forceinline__ f32x4 load_handed_over(const f32x4 *p) {
     x.u[1] = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return x.v;
 }
-// every store_handed_over of this wavefront has reached memory when this returns
-__device__ __forceinline__ void handed_over_stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+// every store_handed_over of this wavefront has reached memory when this returns.  The wait is written out: a
+// release fence at workgroup scope orders the stores for the wavefronts of this compute unit only and, outside
+// thread-group-split mode, waits for nothing (a reader on another die then sees the counter before the data).
+__device__ __forceinline__ void handed_over_stores_done() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), leaving expcnt and lgkmcnt alone
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
 // no load_handed_over is moved ahead of this point (placed behind the counter's read)
 __device__ __forceinline__ void handed_over_loads_begin() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
 
