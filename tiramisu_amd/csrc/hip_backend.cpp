@@ -77,11 +77,98 @@ struct generic_kernel_gen {
                 if (n->lkind == leaf_kind::let) inner.insert(n->comp->get_name());
             }
         });
+        choose_lane_dimension(root);
         if (!std::getenv("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
             std::vector<node_ptr> stack;
             find_reductions(root, stack);
         }
     }
+
+    // ---- which thread-mapped loop runs along the lanes.  The front-end numbers the tagged thread levels from
+    // the innermost outwards (x, y, z: tiramisu_codegen_cuda.cpp:560-617), whatever the accesses look like: a
+    // program that tiles (i, j) with i the contiguous index of its buffers -- the image pipelines of
+    // benchmarks/halide all do -- gets threadIdx.x on the strided index, and the 64 lanes of a wavefront touch 16
+    // rows.  Which hardware index carries which tagged loop is not part of the program's meaning (the threads of
+    // a block are unordered), so the kernel may renumber: the dimension in which most accesses to memory have
+    // unit stride becomes x.  Not done when some statement stores to memory at an element that does not involve
+    // every thread loop around it (a sum or a broadcast across threads: the lowering of those is tied to x).
+    void choose_lane_dimension(const node_ptr &root) {
+        if (std::getenv("TIRAMISU_HIP_KEEP_THREAD_DIMENSIONS")) return;
+        int used = 0;
+        for (int d = 0; d < 3; d++) used += loops_per_dim[1][d] > 0;
+        if (used < 2) return;
+        long score[3] = {0, 0, 0};
+        bool veto = false;
+        std::vector<node_ptr> stack;
+        std::function<void(const node_ptr &)> go = [&](const node_ptr &n) {
+            if (!n || veto) return;
+            if (n->kind == node_kind::loop) stack.push_back(n);
+            if (n->kind == node_kind::leaf) {
+                std::string it[3];
+                for (auto &l : stack)
+                    if (l->gpu_thread >= 0) it[l->gpu_thread] = l->iterator;
+                auto count = [&](const buffer *b, const std::vector<expr> &index) {
+                    if (!b || index.size() != b->get_dim_sizes().size()) return;
+                    if (b->get_location() != memory_location::global && b->get_location() != memory_location::host &&
+                        b->get_location() != memory_location::shared) return;
+                    const expr lin = lir::simplify(lir::linearize(b, index));
+                    for (int d = 0; d < 3; d++) {
+                        if (it[d].empty() || !lir::mentions(lin, it[d])) continue;
+                        bool ok = true;
+                        const expr c = lir::simplify(lir::coefficient(lin, it[d], ok));
+                        // a strided access to global memory is one transaction per lane, a strided LDS access a few
+                        // conflict cycles: global accesses decide, LDS accesses break ties
+                        if (ok && c.is_integer_literal() && (c.get_int_val() == 1 || c.get_int_val() == -1))
+                            score[d] += b->get_location() == memory_location::shared ? 1 : 16;
+                    }
+                };
+                auto count_loads = [&](const expr &e) {
+                    if (!e.is_defined()) return;
+                    e.visit([&](const expr &x) {
+                        if (x.get_expr_type() != e_op || x.get_op_type() != o_access) return;
+                        auto b = f->get_buffers().find(x.get_name());
+                        if (b != f->get_buffers().end()) count(b->second, x.get_access());
+                    });
+                };
+                if (n->lkind == leaf_kind::assign && n->lhs) {
+                    const memory_location where = n->lhs->get_location();
+                    if (where == memory_location::global || where == memory_location::host || where == memory_location::shared)
+                        for (int d = 0; d < 3; d++) {
+                            if (it[d].empty()) continue;
+                            bool involved = false;
+                            for (auto &e : n->lhs_index) involved = involved || lir::mentions(e, it[d]);
+                            if (!involved) veto = true;
+                        }
+                    count(n->lhs, n->lhs_index);
+                }
+                if (n->lkind == leaf_kind::assign || n->lkind == leaf_kind::let) {
+                    count_loads(n->rhs);
+                    count_loads(n->predicate);
+                    for (auto &l : n->lets) count_loads(l.second);
+                }
+                if (n->lkind == leaf_kind::call) veto = true;
+            }
+            for (auto &c : n->children) go(c);
+            go(n->body);
+            go(n->then_body);
+            go(n->else_body);
+            if (n->kind == node_kind::loop) stack.pop_back();
+        };
+        go(root);
+        if (veto) return;
+        int best = 0;
+        for (int d = 1; d < 3; d++)
+            if (loops_per_dim[1][d] > 0 && score[d] > score[best]) best = d;
+        if (best == 0) return;
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind != node_kind::loop) return;
+            if (n->gpu_thread == 0) n->gpu_thread = best;
+            else if (n->gpu_thread == best) n->gpu_thread = 0;
+        });
+        std::swap(loops_per_dim[1][0], loops_per_dim[1][best]);
+        lanes_renumbered = true;
+    }
+    bool lanes_renumbered = false;
 
     // ---- sums across threads.  A statement  X[e] = X[e] + term  under a loop mapped to threadIdx.x whose
     // iterator the element e does not involve asks every thread of that loop to add into one element:
@@ -428,6 +515,7 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
 
     kernel k;
     k.how = "generic";
+    if (g.lanes_renumbered) k.how += ", threadIdx.x given to the thread loop along which the accesses have unit stride";
     if (g.wave_reductions)
         k.how += ", " + std::to_string(g.wave_reductions) + " sum(s) across the threads of a loop lowered to DPP wavefront reductions" +
                  (g.needs_reduction_scratch ? " (wavefront totals combined through LDS)" : "");
