@@ -199,7 +199,7 @@ def bench_heat2d(steps, warmup, with_cpu):
                      "vector_alu_busy": t_dom["vector_alu_busy"] if t_dom else None,
                      "limiter": "hbm" if fused_steps == 1 else
                                 "vector ALUs (time-fused launch: the stencil arithmetic of all fused steps sets its duration)" +
-                                ("; this launch also moves its bytes at the rate of a plain copy on this GPU (5.1-5.3 TB/s)"
+                                ("; this launch also moves its bytes at the highest streaming rate measured on this GPU (5.1-5.3 TB/s)"
                                  if achieved >= 5000.0 else "")},
         "kernels": {k: {"ms": v[0], "launches_per_step": v[1], "traffic": measured[k]["bytes"] if measured[k] else None} for k, v in prof.items()},
     }

@@ -6,8 +6,8 @@ written for), the three tuned sgemm schedules and chain_mm.  The programs copy t
 themselves; what is timed is their kernels: HIP events around every launch of a call
 (tiramisu_hip_profile_*), median over the calls.  Bytes are the algorithmic ones: every input and
 output element once.  Prints one markdown table.  Run from the repository root on a machine with a
-GPU:
-    python tests/reference_programs/time_reference_programs.py
+GPU, for all programs or for those named:
+    python tests/reference_programs/time_reference_programs.py [program ...]
 """
 import ctypes
 import os
@@ -25,8 +25,11 @@ HBM_PEAK_GBS, FP32_MFMA_PEAK_TFLOPS = 8000.0, 157.3
 CALLS = 7
 
 
+BUILD = os.environ.get("TIRAMISU_REFERENCE_PROGRAMS_BUILD", os.path.join(HERE, "build"))   # where the libraries lie
+
+
 def library(name):
-    return os.path.join(HERE, "build", "lib%s.so" % name)
+    return os.path.join(BUILD, "lib%s.so" % name)
 
 
 def kernel_times(call):
@@ -42,7 +45,7 @@ def kernel_times(call):
     return runs[len(runs) // 2]
 
 
-def image_pipelines():
+def image_pipelines(only):
     M, N = 3520, 2112                       # rows, columns
     rng = np.random.RandomState(1)
     rgb = rng.randint(0, 256, (3, M, N)).astype(np.uint8)
@@ -50,6 +53,8 @@ def image_pipelines():
     out = []
 
     def add(name, function, args, nbytes, note):
+        if only and name not in only:
+            return
         program = runtime.Program(library(name), function)
         program(*args)                      # first call: module load
         total, by = kernel_times(lambda: program(*args))
@@ -80,14 +85,18 @@ def image_pipelines():
     return out
 
 
-def gemm_programs():
+def gemm_programs(only):
     out = []
+    if only and not any(o.startswith("sgemm") for o in only):
+        return out
     ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
     n = 3072
     rng = np.random.RandomState(3072)
     A, B, C = (rng.uniform(-1, 1, (n, n)).astype(np.float32) for _ in range(3))
     consts = np.array([3, 2], np.float32)
     for g in (1, 2, 3):
+        if only and "sgemm_generator%d" % g not in only:
+            continue
         program = runtime.Program(library("sgemm_generator%d" % g), "matmul")
         t0, t1 = np.zeros(1, np.float32), np.zeros(1, np.float32)
         args = (consts, A, B, C.copy(), t0, t1)
@@ -99,14 +108,15 @@ def gemm_programs():
 
 
 def main():
+    only = set(sys.argv[1:])
     runtime.wrappers()
     print("| program | what | kernels of one call | time | algorithmic rate | of the roofline |")
     print("|---|---|---|---|---|---|")
-    for name, note, total, by, nbytes in image_pipelines():
+    for name, note, total, by, nbytes in image_pipelines(only):
         kernels = ", ".join("%s %.1f us%s" % (k, t / n * 1e3, " x %d" % n if n > 1 else "") for k, (t, n) in sorted(by.items()))
         gbs = nbytes / (total * 1e-3) / 1e9
         print("| `%s` | %s | %s | %.3f ms | %.0f GB/s | %.2f of 8 TB/s |" % (name, note, kernels, total, gbs, gbs / HBM_PEAK_GBS), flush=True)
-    for name, note, total, by, flop in gemm_programs():
+    for name, note, total, by, flop in gemm_programs(only):
         kernels = ", ".join("%s %.3f ms" % (k, t / n) for k, (t, n) in sorted(by.items()))
         tf = flop / (total * 1e-3) / 1e12
         print("| %s | %s | %s | %.3f ms | %.1f TFLOP/s | %.2f of %.1f TFLOP/s |" % (name, note, kernels, total, tf, tf / FP32_MFMA_PEAK_TFLOPS, FP32_MFMA_PEAK_TFLOPS), flush=True)

@@ -68,3 +68,13 @@ def test_gpu_column_sums(programs_dir):
     s = on_gpu(programs_dir, "column_sums_keep_lanes", A, s)
     assert np.array_equal(s, A.sum(axis=0))
     assert np.array_equal(s, s_cpu)
+
+
+def test_workgroups_are_renumbered_where_tiles_share_data(programs_dir, product_programs_dir):
+    # LDS staging (the cache_shared GEMM on the generic emitter): every XCD takes an eighth of the tiles;
+    # a streaming kernel with wide tiles (the copy program; 600-byte-wide tiles here) keeps the hardware order
+    shared = kernel_source(programs_dir, "sgemm_shared_regs_generic")
+    assert "workgroups renumbered: an eighth of the tiles per XCD" in shared
+    assert re.search(r"const int32_t c\d+ = \(int32_t\)_tile\.[xy] \+ 0;", shared) and "blockIdx.x + gridDim.x * blockIdx.y" in shared
+    for text in (kernel_source(product_programs_dir, "copy_plane"), kernel_source(programs_dir, "lanes_follow_unit_stride")):
+        assert "workgroups renumbered" not in text and "_tile" not in text

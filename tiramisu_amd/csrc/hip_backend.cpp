@@ -9,6 +9,7 @@
 //   f.o.host.cpp  host glue source
 //   f.o           host object; exports  extern "C" int <function>(halide_buffer_t *...)
 #include "hip_backend.h"
+#include "kernels/target_gfx950.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -78,6 +79,7 @@ struct generic_kernel_gen {
             }
         });
         choose_lane_dimension(root);
+        choose_block_order(root);
         if (!std::getenv("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
             std::vector<node_ptr> stack;
             find_reductions(root, stack);
@@ -169,6 +171,69 @@ struct generic_kernel_gen {
         lanes_renumbered = true;
     }
     bool lanes_renumbered = false;
+
+    // ---- which tile a workgroup takes.  Workgroups are dealt round-robin to the chip's XCDs, each with an L2 of
+    // its own, in the order x fastest: neighbouring tiles of a 2-D grid run on different XCDs, and a cache line
+    // that several tiles touch (16 one-byte pixels of a 128-byte line per tile in the reference's image pipelines;
+    // the halo of a stencil tile) is fetched from memory once per XCD.  Workgroups being unordered, a kernel with
+    // a two-dimensional grid renumbers them: XCD c takes the c-th eighth of the tiles, walked with the block
+    // dimension fastest whose iterator has the smallest stride in the accesses to global memory, so that tiles
+    // that share lines meet in one L2 at about the same time.  Done only where tiles share data -- a tile is at
+    // most 32 bytes wide along that dimension (four tiles or more per line), the kernel stages data in LDS (halos,
+    // operand panels), or some access to global memory does not depend on one of the two block iterators (a panel
+    // that a row of tiles re-reads): for a plain streaming kernel with wide tiles the renumbering only costs its
+    // integer division per workgroup (the 8192 x 8192 copy kernel, one element per thread: 0.152 ms against 0.105).
+    int fast_block_dim = -1;      // 0 or 1 when the workgroups are renumbered
+    void choose_block_order(const node_ptr &root) {
+        if (std::getenv("TIRAMISU_HIP_KEEP_BLOCK_ORDER")) return;
+        if (loops_per_dim[0][0] != 1 || loops_per_dim[0][1] != 1 || loops_per_dim[0][2] != 0) return;
+        std::string it[2];
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind == node_kind::loop && n->gpu_block >= 0 && n->gpu_block < 2) it[n->gpu_block] = n->iterator;
+        });
+        long stride[2] = {0, 0};      // smallest literal |coefficient| x element size of the block iterator over the global accesses
+        bool other[2] = {false, false};   // ... or some access in which it has a non-literal coefficient
+        bool shares = false;              // tiles share data (LDS staging, or an access that ignores a block iterator)
+        auto count = [&](const buffer *b, const std::vector<expr> &index) {
+            if (!b || index.size() != b->get_dim_sizes().size()) return;
+            if (b->get_location() == memory_location::shared) shares = true;
+            if (b->get_location() != memory_location::global && b->get_location() != memory_location::host) return;
+            const expr lin = lir::simplify(lir::linearize(b, index));
+            const long bytes = (long)primitive_size(b->get_elements_type());
+            for (int d = 0; d < 2; d++) {
+                if (!lir::mentions(lin, it[d])) { shares = true; continue; }
+                bool ok = true;
+                const expr c = lir::simplify(lir::coefficient(lin, it[d], ok));
+                if (ok && c.is_integer_literal() && c.get_int_val() != 0) {
+                    const long a = std::labs(c.get_int_val()) * bytes;
+                    stride[d] = stride[d] == 0 ? a : std::min(stride[d], a);
+                } else {
+                    other[d] = true;
+                }
+            }
+        };
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind != node_kind::leaf) return;
+            if (n->lkind == leaf_kind::assign && n->lhs) count(n->lhs, n->lhs_index);
+            auto loads = [&](const expr &e) {
+                if (!e.is_defined()) return;
+                e.visit([&](const expr &x) {
+                    if (x.get_expr_type() != e_op || x.get_op_type() != o_access) return;
+                    auto b = f->get_buffers().find(x.get_name());
+                    if (b != f->get_buffers().end()) count(b->second, x.get_access());
+                });
+            };
+            if (n->lkind == leaf_kind::assign || n->lkind == leaf_kind::let) {
+                loads(n->rhs);
+                loads(n->predicate);
+                for (auto &l : n->lets) loads(l.second);
+            }
+        });
+        // one dimension with a literal stride, smaller than the other's or the other's symbolic (a row pitch)
+        if (stride[0] > 0 && (stride[1] == 0 ? other[1] : stride[0] < stride[1])) fast_block_dim = 0;
+        else if (stride[1] > 0 && (stride[0] == 0 ? other[0] : stride[1] < stride[0])) fast_block_dim = 1;
+        if (fast_block_dim >= 0 && !shares && stride[fast_block_dim] > 32) fast_block_dim = -1;
+    }
 
     // ---- sums across threads.  A statement  X[e] = X[e] + term  under a loop mapped to threadIdx.x whose
     // iterator the element e does not involve asks every thread of that loop to add into one element:
@@ -418,7 +483,7 @@ struct generic_kernel_gen {
             expr ext = host_extent(n, first, guard);
             (is_block ? grid_ext : block_ext)[dim].push_back(ext);
             if (loops_per_dim[is_block ? 0 : 1][dim] > 1) guard = true;
-            const char *idx = is_block ? "blockIdx." : "threadIdx.";
+            const char *idx = is_block ? (fast_block_dim >= 0 ? "_tile." : "blockIdx.") : "threadIdx.";
             body << pad(ind) << "{\n";
             body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)" << idx << "xyz"[dim] << " + "
                  << dev.print(first) << ";\n";
@@ -516,6 +581,7 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
     kernel k;
     k.how = "generic";
     if (g.lanes_renumbered) k.how += ", threadIdx.x given to the thread loop along which the accesses have unit stride";
+    if (g.fast_block_dim >= 0) k.how += std::string(", workgroups renumbered: an eighth of the tiles per XCD, ") + "xy"[g.fast_block_dim] + " fastest";
     if (g.wave_reductions)
         k.how += ", " + std::to_string(g.wave_reductions) + " sum(s) across the threads of a loop lowered to DPP wavefront reductions" +
                  (g.needs_reduction_scratch ? " (wavefront totals combined through LDS)" : "");
@@ -590,6 +656,16 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
     os << ")\n{\n";
     for (auto &d : top_decls) os << "    " << d << "\n";
     if (g.needs_reduction_scratch) os << "    __shared__ float _reduction_scratch[16];\n";
+    if (g.fast_block_dim >= 0) {
+        // hardware order l (x fastest) -> XCD l % XCDS, its (l / XCDS)-th workgroup -> tile t of the XCD's share
+        const char fast = "xy"[g.fast_block_dim], slow = "xy"[1 - g.fast_block_dim];
+        os << "    uint3 _tile;\n    {\n"
+           << "        const unsigned _n = gridDim.x * gridDim.y, _l = blockIdx.x + gridDim.x * blockIdx.y;\n"
+           << "        const unsigned _c = _l % " << ttarget::XCDS << "u, _share = _n / " << ttarget::XCDS << "u, _extra = _n % " << ttarget::XCDS << "u;\n"
+           << "        const unsigned _t = _c * _share + (_c < _extra ? _c : _extra) + _l / " << ttarget::XCDS << "u;\n";
+        os << "        _tile." << fast << " = _t % gridDim." << fast << ";\n        _tile." << slow << " = _t / gridDim." << fast << ";\n"
+           << "        _tile.z = 0;\n    }\n";
+    }
     os << g.body.str() << "}\n";
     k.source = os.str();
     return k;
