@@ -87,7 +87,7 @@ def image_pipelines(only):
 
 def gemm_programs(only):
     out = []
-    if only and not any(o.startswith("sgemm") for o in only):
+    if only and not any(o.startswith("sgemm") or o == "chain_mm" for o in only):
         return out
     ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
     n = 3072
@@ -104,6 +104,14 @@ def gemm_programs(only):
         total, by = kernel_times(lambda: program(*args))
         out.append(("sgemm generator%d" % g, "3072^3, %s" % ("explicit LDS copies, double-buffered" if g == 1 else "explicit LDS copies" if g == 2 else "cache_shared"),
                     total, by, 2.0 * n ** 3))
+    if not only or "chain_mm" in only:
+        rng = np.random.RandomState(1024)
+        A2, B2, C2 = (rng.uniform(-1, 1, shape).astype(np.float32) for shape in ((1024, 512), (512, 128), (128, 256)))
+        O = np.zeros((1024, 256), np.float32)
+        program = runtime.Program(library("chain_mm"), "matmul")
+        program(A2, B2, C2, O)
+        total, by = kernel_times(lambda: program(A2, B2, C2, O))
+        out.append(("chain_mm", "(1024x512 x 512x128) x 128x256, two gpu_tile nests", total, by, 2.0 * 1024 * 128 * (512 + 256)))
     return out
 
 
