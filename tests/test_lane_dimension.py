@@ -1,6 +1,7 @@
-"""Which tagged thread loop runs along the lanes (tests/programs/lane_dimension.cpp): the kernel gives
-threadIdx.x to the loop along which the accesses have unit stride, unless a sum across threads ties the
-numbering down.  The generated text is checked here without a GPU; results on the GPU against numpy and
+"""Which tagged thread loop runs along the lanes, how wide a workgroup is and which tile it takes
+(tests/programs/lane_dimension.cpp): the kernel gives threadIdx.x to the loop along which the accesses have unit
+stride and deals independent points out to workgroups one wavefront wide, unless a sum across threads ties the
+mapping down.  The generated text is checked here without a GPU; results on the GPU against numpy and
 against the CPU-generated code of the same programs, bit for bit (small integers)."""
 import os
 import re
@@ -35,9 +36,13 @@ def cpu_variant(programs_dir, name):
 def test_threadidx_x_follows_the_unit_stride(programs_dir):
     text = kernel_source(programs_dir, "lanes_follow_unit_stride")
     assert "threadIdx.x given to the thread loop along which the accesses have unit stride" in text
-    # the iterator taken from threadIdx.x is the one added to the store index without a factor
-    x_iterator = re.search(r"const int32_t (c\d+) = \(int32_t\)threadIdx\.x", text).group(1)
-    y_iterator = re.search(r"const int32_t (c\d+) = \(int32_t\)threadIdx\.y", text).group(1)
+    # the points are dealt out again to workgroups one wavefront wide; the iterator that follows threadIdx.x is
+    # the one added to the store index without a factor
+    assert "points dealt out again to workgroups of 64 x 4 (the program's tiles: 16 x 16)" in text
+    assert re.search(r"const uint32_t _g0 = blockIdx\.x \* 64u \+ threadIdx\.x;", text)
+    assert re.search(r"const uint32_t _g1 = blockIdx\.y \* 4u \+ threadIdx\.y;", text)
+    x_iterator = re.search(r"const int32_t (c\d+) = \(int32_t\)\(_g0 % 16u\)", text).group(1)
+    y_iterator = re.search(r"const int32_t (c\d+) = \(int32_t\)\(_g1 % 16u\)", text).group(1)
     store = re.search(r"b_out\[(.*?)\] = ", text).group(1)
     assert re.search(r"\+ %s\) \* 150\)" % y_iterator, store) and re.search(r"\+ %s\)\)$" % x_iterator, store), store
 

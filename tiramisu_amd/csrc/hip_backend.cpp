@@ -79,6 +79,7 @@ struct generic_kernel_gen {
             }
         });
         choose_lane_dimension(root);
+        choose_workgroup_shape(root);
         choose_block_order(root);
         if (!std::getenv("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
             std::vector<node_ptr> stack;
@@ -157,6 +158,7 @@ struct generic_kernel_gen {
             if (n->kind == node_kind::loop) stack.pop_back();
         };
         go(root);
+        threads_independent = !veto;
         if (veto) return;
         int best = 0;
         for (int d = 1; d < 3; d++)
@@ -171,6 +173,111 @@ struct generic_kernel_gen {
         lanes_renumbered = true;
     }
     bool lanes_renumbered = false;
+    bool threads_independent = false;   // every store to memory involves every thread loop around it, no calls
+
+    // ---- how wide a workgroup is.  A program tiled gpu_tile(i, j, 16, 16) gives a wavefront a patch of 16 x 4
+    // points: four short row segments per access.  Where the points of a kernel have nothing to do with one
+    // another (no LDS, no barrier, no sum across threads) the grouping of points into workgroups is free as well,
+    // so such a kernel with a two-dimensional grid and block deals its points out again: along x a workgroup is
+    // 64 wide (one wavefront = 64 consecutive points of a row), along y as high as keeps its thread count, and
+    // every thread recovers the block and thread iterators of the point it stands for,
+    //     g = 64 * blockIdx.x + threadIdx.x,  block iterator = g / S,  thread iterator = g % S,
+    // S being the program's tile extent; the program's own guards, written in those iterators, stay as they are.
+    struct retiling {
+        bool on = false;
+        const node *block[2] = {nullptr, nullptr}, *thread[2] = {nullptr, nullptr};
+        long tile[2] = {0, 0}, wide[2] = {0, 0};     // the program's thread extents, the workgroup's
+    } retile;
+    void choose_workgroup_shape(const node_ptr &root) {
+        if (std::getenv("TIRAMISU_HIP_KEEP_TILES") || !threads_independent) return;
+        for (int d = 0; d < 3; d++)
+            if (loops_per_dim[0][d] != (d < 2) || loops_per_dim[1][d] != (d < 2)) return;
+        bool plain = true;
+        node_ptr block[2], thread[2];
+        std::vector<node_ptr> order;      // mapped loops from the outermost inwards
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind == node_kind::leaf) {
+                if (n->lkind == leaf_kind::sync || n->lkind == leaf_kind::call || n->lkind == leaf_kind::copy) plain = false;
+                if ((n->lkind == leaf_kind::allocate || n->lkind == leaf_kind::release) && n->target &&
+                    n->target->get_location() == memory_location::shared) plain = false;
+                auto shared = [&](const expr &e) {
+                    if (!e.is_defined()) return;
+                    e.visit([&](const expr &x) {
+                        if (x.get_expr_type() != e_op || x.get_op_type() != o_access) return;
+                        auto b = f->get_buffers().find(x.get_name());
+                        if (b != f->get_buffers().end() && b->second->get_location() == memory_location::shared) plain = false;
+                    });
+                };
+                if (n->lhs && n->lhs->get_location() == memory_location::shared) plain = false;
+                shared(n->rhs);
+                shared(n->predicate);
+                for (auto &l : n->lets) shared(l.second);
+            }
+            if (n->kind != node_kind::loop) return;
+            if (n->gpu_block >= 0) { block[n->gpu_block] = n; order.push_back(n); }
+            if (n->gpu_thread >= 0) { thread[n->gpu_thread] = n; order.push_back(n); }
+        });
+        if (!plain || order.size() != 4 || order[0]->gpu_block < 0 || order[1]->gpu_block < 0) return;
+        // the four mapped loops sit directly inside one another (a thread may then define all four iterators at once)
+        if (order[0] != root) return;
+        for (int i = 0; i + 1 < 4; i++) {
+            node_ptr inside = order[i]->body;
+            while (inside && inside->kind == node_kind::block && inside->children.size() == 1) inside = inside->children[0];
+            if (inside != order[i + 1]) return;
+        }
+        long S[2];
+        for (int d = 0; d < 2; d++) {
+            bool guard;
+            expr first;
+            const expr ext = lir::simplify(host_extent(thread[d], first, guard));
+            if (!ext.is_integer_literal() || !lir::simplify(thread[d]->init).is_integer_literal() || lir::simplify(thread[d]->init).get_int_val() != 0) return;
+            if (!lir::simplify(block[d]->init).is_integer_literal() || lir::simplify(block[d]->init).get_int_val() != 0) return;
+            if (depends_on(block[d]->upper, inner)) return;
+            S[d] = ext.get_int_val();
+            if (S[d] < 1 || (S[d] & (S[d] - 1)) != 0) return;
+        }
+        const long W = ttarget::WAVEFRONT;
+        if (S[0] >= W || (S[0] * S[1]) % W != 0) return;
+        // the block loop that tiles the same index as the thread loop on x: its coefficient in some access to
+        // global memory is the tile extent times the thread iterator's
+        int partner = -1;
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind != node_kind::leaf || partner >= 0) return;
+            auto look = [&](const buffer *b, const std::vector<expr> &index) {
+                if (partner >= 0 || !b || index.size() != b->get_dim_sizes().size() || b->get_location() != memory_location::global) return;
+                const expr lin = lir::simplify(lir::linearize(b, index));
+                bool ok = true;
+                const expr ct = lir::simplify(lir::coefficient(lin, thread[0]->iterator, ok));
+                if (!ok || !ct.is_integer_literal() || ct.get_int_val() == 0) return;
+                for (int d = 0; d < 2; d++) {
+                    bool okb = true;
+                    const expr cb = lir::simplify(lir::coefficient(lin, block[d]->iterator, okb));
+                    if (okb && cb.is_integer_literal() && cb.get_int_val() == ct.get_int_val() * S[0]) partner = d;
+                }
+            };
+            if (n->lkind == leaf_kind::assign && n->lhs) look(n->lhs, n->lhs_index);
+            if (n->rhs.is_defined())
+                n->rhs.visit([&](const expr &x) {
+                    if (x.get_expr_type() != e_op || x.get_op_type() != o_access) return;
+                    auto b = f->get_buffers().find(x.get_name());
+                    if (b != f->get_buffers().end()) look(b->second, x.get_access());
+                });
+        });
+        if (partner < 0) return;
+        if (partner == 1) {
+            std::swap(block[0], block[1]);
+            block[0]->gpu_block = 0;
+            block[1]->gpu_block = 1;
+        }
+        retile.on = true;
+        for (int d = 0; d < 2; d++) {
+            retile.block[d] = block[d].get();
+            retile.thread[d] = thread[d].get();
+            retile.tile[d] = S[d];
+        }
+        retile.wide[0] = W;
+        retile.wide[1] = S[0] * S[1] / W;
+    }
 
     // ---- which tile a workgroup takes.  Workgroups are dealt round-robin to the chip's XCDs, each with an L2 of
     // its own, in the order x fastest: neighbouring tiles of a 2-D grid run on different XCDs, and a cache line
@@ -476,6 +583,32 @@ struct generic_kernel_gen {
             emit_thread_reduction(n, red->second, ind);
             return;
         }
+        if (retile.on && (is_block || is_thread)) {
+            const int dim = is_block ? n->gpu_block : n->gpu_thread;
+            bool guard;
+            expr first;
+            const expr ext = host_extent(n, first, guard);
+            const long S = retile.tile[dim], wide = retile.wide[dim];
+            body << pad(ind) << "{\n";
+            if (is_block) {
+                grid_ext[dim].push_back(lir::simplify((ext * expr((int32_t)S) + expr((int32_t)(wide - 1))) / expr((int32_t)wide)));
+                body << pad(ind + 1) << "const uint32_t _g" << dim << " = " << (fast_block_dim >= 0 ? "_tile." : "blockIdx.") << "xyz"[dim] << " * " << wide
+                     << "u + threadIdx." << "xyz"[dim] << ";   // the point's index along this dimension\n";
+                body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)(_g" << dim << " / " << S << "u);\n";
+                body << pad(ind + 1) << "if (" << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+                guard = true;
+            } else {
+                block_ext[dim].push_back(expr((int32_t)wide));
+                body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)(_g" << dim << " % " << S << "u);\n";
+                if (guard)
+                    body << pad(ind + 1) << "if (" << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator
+                         << " <= " << dev.print(n->upper) << ") {\n";
+            }
+            emit(n->body, ind + (guard ? 2 : 1));
+            if (guard) body << pad(ind + 1) << "}\n";
+            body << pad(ind) << "}\n";
+            return;
+        }
         if (is_block || is_thread) {
             const int dim = is_block ? n->gpu_block : n->gpu_thread;
             bool guard;
@@ -581,6 +714,9 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
     kernel k;
     k.how = "generic";
     if (g.lanes_renumbered) k.how += ", threadIdx.x given to the thread loop along which the accesses have unit stride";
+    if (g.retile.on)
+        k.how += ", points dealt out again to workgroups of " + std::to_string(g.retile.wide[0]) + " x " + std::to_string(g.retile.wide[1]) +
+                 " (the program's tiles: " + std::to_string(g.retile.tile[0]) + " x " + std::to_string(g.retile.tile[1]) + ")";
     if (g.fast_block_dim >= 0) k.how += std::string(", workgroups renumbered: an eighth of the tiles per XCD, ") + "xy"[g.fast_block_dim] + " fastest";
     if (g.wave_reductions)
         k.how += ", " + std::to_string(g.wave_reductions) + " sum(s) across the threads of a loop lowered to DPP wavefront reductions" +
