@@ -56,15 +56,16 @@ def sgemm_strided(Abuf, Bbuf, Cbuf, M, N, K, alpha, beta, ldA, ldB, ldC, offA, o
         ldC = N
     out = Cbuf.copy().ravel()
     a, b = Abuf.ravel(), Bbuf.ravel()
+    real = Cbuf.dtype.type              # float32, or float64 for tiramisu_cublas_dgemm (:117-162)
     for m in range(M):
         for n in range(N):
-            acc = np.float32(0)
+            acc = real(0)
             for k in range(K):
                 av = a[offA + (k * ldA + m if tA else m * ldA + k)]
                 bv = b[offB + (n * ldB + k if tB else k * ldB + n)]
-                acc = np.float32(acc + np.float32(av * bv))
+                acc = real(acc + real(av * bv))
             idx = offC + m * ldC + n
-            out[idx] = np.float32(alpha) * acc + (np.float32(beta) * out[idx] if beta != 0 else np.float32(0))
+            out[idx] = real(alpha) * acc + (real(beta) * out[idx] if beta != 0 else real(0))
     return out.reshape(Cbuf.shape)
 
 

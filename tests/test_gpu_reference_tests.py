@@ -149,18 +149,19 @@ def test_alloc_in_time_loop(programs_dir):
     (130, 70, 50, -1.0, 0.5, 1, 3),   # MFMA path with ragged edges and unaligned rows
     (256, 256, 64, 1.0, 1.0, 0, 0),   # MFMA path, whole tiles
 ])
-def test_sgemm_library_call(programs_dir, M, N, K, alpha, beta, pad, off):
+@pytest.mark.parametrize("name,real", [("sgemm_library_call", np.float32), ("dgemm_library_call", np.float64)])
+def test_sgemm_library_call(programs_dir, name, real, M, N, K, alpha, beta, pad, off):
     rng = np.random.RandomState(162 + M)
     ldA, ldB, ldC = M + pad, N + pad, N + 2 * pad
     sizes = np.array([M, N, K, ldA, ldB, ldC, off, off + 1, off + 2], np.int32)
-    scal = np.array([alpha, beta], np.float32)
-    A = ints(rng, (K + 1, ldA))     # stored transposed: K rows
-    B = ints(rng, (K + 1, ldB))
-    C = ints(rng, (M + 1, ldC))
+    scal = np.array([alpha, beta], real)
+    A = ints(rng, (K + 1, ldA)).astype(real)     # stored transposed: K rows
+    B = ints(rng, (K + 1, ldB)).astype(real)
+    C = ints(rng, (M + 1, ldC)).astype(real)
     if beta == 0.0:
         C[:] = np.nan               # reading C would poison the result
     expected = ref.sgemm_strided(A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, off, off + 1, off + 2, True, False)
-    runtime.load(programs_dir, "sgemm_library_call")(sizes, scal, A, B, C)
+    runtime.load(programs_dir, name)(sizes, scal, A, B, C)
     assert np.array_equal(C, expected, equal_nan=True)
 
 
