@@ -279,15 +279,15 @@ def conv2d_bias_relu_loops(in_pad, w, bias):
     return out
 
 
-def lstm(weights, biases, x):
-    """Stacked LSTM forward pass in fp32 with numpy matrix products.
+def lstm(weights, biases, x, real=np.float32):
+    """Stacked LSTM forward pass in fp32 (or in `real`) with numpy matrix products.
     weights[L, 2, 4H, H] (slot 0 = input weights W, slot 1 = recurrent weights R), biases[L, 4H],
     x[S, B, H]; gate order i, f, z, o in the 4H rows; zero initial h and c; returns y[S, B, H], the
     hidden state of the last layer.  Restates benchmarks/DNN/blocks/LSTM/cpu/generator.cpp:31-60 with
     the library variant's packing (gpu_lib/generator.cpp:69-70, :78-79, :84-87)."""
     L, _, H4, H = weights.shape
     S, B, _ = x.shape
-    f32 = np.float32
+    f32 = real
     h_prev = np.zeros((L, B, H), f32)
     c_prev = np.zeros((L, B, H), f32)
     y = np.zeros((S, B, H), f32)

@@ -98,6 +98,34 @@ def build_self_driven(rel, stem, obj):
                 "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
+# The library LSTM in double precision: the reference publishes figures for it (gpu_lib/README.md:7-14) and
+# its configuration.h carries the switch ("#if 1  // Flip to use double precision").  The switch is flipped on
+# the way into the compiler -- the header, flipped, and the generator without its include line go through a pipe
+# to g++ -- so nothing of the reference is written anywhere; everything else is as for the float build.
+def build_lstm_gpu_lib_f64():
+    import subprocess
+    rel = "benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp"
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, "lstm_gpu_lib_f64")
+    os.makedirs(work, exist_ok=True)
+    src = os.path.join(REFERENCE, rel)
+    header = open(os.path.join(os.path.dirname(src), "configuration.h")).read()
+    if "#if 1  // Flip to use double precision" not in header:
+        raise RuntimeError("the precision switch of the reference's LSTM configuration moved")
+    text = header.replace("#if 1  // Flip to use double precision", "#if 0") + "\n" + \
+        "".join(line for line in open(src) if '#include "configuration.h"' not in line)
+    gen = os.path.join(work, "gen")
+    cmd = ["g++", "-std=c++17", "-O1", "-x", "c++", "-", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
+           "-I" + os.path.dirname(src), "-o", gen, "-L" + build.PKG, "-ltiramisu", "-Wl,-rpath," + build.PKG]
+    done = subprocess.run(cmd, input=text.encode(), stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    if done.returncode != 0:
+        sys.stderr.write(done.stdout.decode())
+        raise RuntimeError("build step failed: the reference's library LSTM in double precision")
+    build._run([gen], cwd=work)
+    build._run(["g++", "-shared", "-o", library("lstm_gpu_lib_f64"), os.path.join(work, "lstm.o"), "-L" + build.PKG,
+                "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
+
+
 # The reference's naive restatement of its LSTM (a CPU program: codegen without the GPU flag), compiled
 # unchanged through the oracle's CPU emitter: the pin of the numpy LSTM oracle's packing and gate order
 # for the reference's GPU generator (slot 0 = R, rows i, z, o, f).
@@ -205,6 +233,9 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", rel, flush=True)
         build_self_driven(rel, stem, obj)
+    if verbose:
+        print("[reference programs] benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp (double precision)", flush=True)
+    build_lstm_gpu_lib_f64()
     if verbose:
         print("[reference programs]", LSTM_NAIVE, "(CPU)", flush=True)
     build_lstm_naive()

@@ -261,7 +261,7 @@ def lstm_inputs(L, B, H, S, seed):
     return weights, biases, x
 
 
-@pytest.mark.parametrize("name", ["lstm_gpu", "lstm_gpu_lib"])
+@pytest.mark.parametrize("name", ["lstm_gpu", "lstm_gpu_lib", "lstm_gpu_lib_f64"])
 def test_reference_lstm_library_exports_its_function(name):
     """Both GPU LSTM generators compile and generate code unchanged.  Only gpu_lib's function is
     run: gpu/generator.cpp maps its reads of the previous hidden state to rows {m - 1, l} of the
@@ -300,6 +300,35 @@ def test_reference_lstm_gpu_lib_generator():
         best = ms if best is None else min(best, ms)
         whole = call_ms if whole is None else min(whole, call_ms)
     print("gpu_lib LSTM generator: %.3f ms between its timers, %.3f ms for the whole call with allocation and copies"
+          % (best, whole), flush=True)
+
+
+@pytest.mark.gpu
+def test_reference_lstm_gpu_lib_generator_in_double_precision():
+    """The same generator with its configuration switched to double precision (the switch of the reference's
+    gpu_lib/configuration.h, flipped while the program is compiled): the products go through
+    tiramisu_hip_dgemm (fp64 matrix instructions), the rest through the generic emitter on doubles.  The
+    reference publishes 106.7 ms for this on a K80 (gpu_lib/README.md:7-14)."""
+    if not os.path.exists(library("lstm_gpu_lib_f64")):
+        pytest.skip("reference tree was absent when the libraries were built")
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    L, B, H, S = 4, 64, 512, 100
+    weights, biases, x = (a.astype(np.float64) for a in lstm_inputs(L, B, H, S, 512))
+    program = runtime.Program(library("lstm_gpu_lib_f64"), "lstm")
+    expected = ref.lstm(weights, biases, x, real=np.float64)
+    import time
+    best = whole = None
+    for _ in range(3):
+        y = np.zeros((S, B, H), np.float64)
+        t0, t1 = np.zeros(1, np.float32), np.zeros(1, np.float32)
+        start = time.perf_counter()
+        program(weights, biases, x, y, t0, t1)
+        call_ms = (time.perf_counter() - start) * 1e3
+        assert np.max(np.abs(y - expected)) <= 1e-9 * np.max(np.abs(expected))
+        ms = float(t1[0] - t0[0])
+        best = ms if best is None else min(best, ms)
+        whole = call_ms if whole is None else min(whole, call_ms)
+    print("gpu_lib LSTM generator in double precision: %.3f ms between its timers, %.3f ms for the whole call with allocation and copies"
           % (best, whole), flush=True)
 
 

@@ -573,10 +573,13 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
     // element (m, k) of op(A) and (k, n) of op(B) through two strides each
     const long sam = transposeA ? 1L : (long)ldA, sak = transposeA ? (long)ldA : 1L;
     const long sbk = transposeB ? 1L : (long)ldB, sbn = transposeB ? (long)ldB : 1L;
-    // 128 x 128 tiles when they give every compute unit work, else 64 x 64
-    const long big = (long)((M + 127) / 128) * (long)((N + 127) / 128);
+    // 128 x 128 tiles when they give every compute unit work, else 64 x 64, and 32 x 32 for problems that would
+    // leave half of the chip idle with those (the 64 x 2048 x 512 products of a recurrent cell: 128 workgroups
+    // instead of 32)
+    const long big = (long)((M + 127) / 128) * (long)((N + 127) / 128), medium = (long)((M + 63) / 64) * (long)((N + 63) / 64);
     if (big >= ttarget::COMPUTE_UNITS / 2) launch_dgemm<tgemm64::shape<4, 2, 2, 4>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
-    else launch_dgemm<tgemm64::shape<2, 2, 2, 2>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
+    else if (medium >= ttarget::COMPUTE_UNITS / 2) launch_dgemm<tgemm64::shape<2, 2, 2, 2>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
+    else launch_dgemm<tgemm64::shape<1, 1, 2, 2>>(transposeA, transposeB, a, b, c, (int)M, (int)N, (int)K, sam, sak, sbk, sbn, (long)ldC, alpha, beta);
     return 0;
 }
 
