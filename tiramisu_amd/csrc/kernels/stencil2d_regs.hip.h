@@ -33,6 +33,8 @@
 //      of that step's parity and those after ST_R steps to the other one.  Neither plane is read except for its
 //      fixed cells, so ST_R may be even and the time loop can end with a fused launch that leaves both planes
 //      exactly as the un-tiled loop does.
+//   3  a single step out of place (ST_R = 1): read the first buffer, write another one that comes in the place of
+//      `temp`; the fixed cells are the source's and nothing of them is stored.
 // The host code composes the time loop from such launches.
 //
 // Macros supplied by the emitter before this file is included:
@@ -73,9 +75,9 @@
 #define ST_PLANE(p) (planes + (size_t)(p) * ST_NY * ST_NX)
 #define ST_PLANES                                                                                              \
     const float *__restrict__ src = ST_MODE == 2 ? temp : ST_PLANE(src_plane);                                 \
-    float *__restrict__ dst = ST_MODE == 1 ? temp : ST_PLANE((src_plane + ST_R) & 1);                          \
+    float *__restrict__ dst = (ST_MODE == 1 || ST_MODE == 3) ? temp : ST_PLANE((src_plane + ST_R) & 1);        \
     float *__restrict__ dst_prev = ST_MODE == 2 ? ST_PLANE((src_plane + ST_R - 1) & 1) : nullptr;              \
-    const float *fixed_other = ST_PLANE(1 - src_plane);
+    const float *fixed_other = ST_PLANE(ST_MODE == 3 ? src_plane : 1 - src_plane);
 
 #ifndef TIRAMISU_AMD_STENCIL2D_REGS_COMMON
 #define TIRAMISU_AMD_STENCIL2D_REGS_COMMON
@@ -265,7 +267,7 @@ __attribute__((amdgpu_waves_per_eu(ST_OCC)))
 ST_NAME(float *planes, const int src_plane, float *temp)
 {
     static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
-    static_assert(ST_MODE == 2 ? ST_R >= 2 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
+    static_assert(ST_MODE == 2 ? ST_R >= 2 : ST_MODE == 3 ? ST_R == 1 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
     __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
     ST_PLANES
     const int b = blockIdx.x;

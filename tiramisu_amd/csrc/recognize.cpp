@@ -122,27 +122,37 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
 
     computation *S = leaf->comp;
     const auto &its = S->get_iteration_domain_dimension_names();
-    if (its.size() != 3 || S->get_data_type() != p_float32) return false;
-    auto t_it = leaf->iterators.find(its[0]);
-    if (t_it == leaf->iterators.end()) return false;
-    if (time_loop) {
-        if (t_it->second.get_expr_type() != e_var || t_it->second.get_name() != time_loop->iterator) return false;
-    } else if (!lir::simplify(t_it->second).is_integer_literal()) {
-        return false;
+    // two forms: S(t, y, x) from S(t-1, ...) on a ping-pong pair of planes, and -- a single step out of place --
+    // S(y, x) from another computation I(y+dy, x+dx) that lives in a buffer of its own
+    const bool planar = its.size() == 2 && !time_loop;
+    if ((its.size() != 3 && !planar) || S->get_data_type() != p_float32) return false;
+    if (planar && std::getenv("TIRAMISU_NO_SINGLE_STEP_STENCIL")) return false;
+    if (!planar) {
+        auto t_it = leaf->iterators.find(its[0]);
+        if (t_it == leaf->iterators.end()) return false;
+        if (time_loop) {
+            if (t_it->second.get_expr_type() != e_var || t_it->second.get_name() != time_loop->iterator) return false;
+        } else if (!lir::simplify(t_it->second).is_integer_literal()) {
+            return false;
+        }
     }
+    const std::string &yi = its[planar ? 0 : 1], &xi = its[planar ? 1 : 2];
 
-    // expression: reads of S at (t-1, y+dy, x+dx) and float literals only
+    // expression: reads of S at (t-1, y+dy, x+dx) -- of one other computation at (y+dy, x+dx) -- and float literals only
     int radius = 0;
     bool ok = true;
+    std::string source_name = planar ? std::string() : S->get_name();
     std::function<expr(const expr &)> rewrite = [&](const expr &e) -> expr {
         if (!e.is_defined()) { ok = false; return e; }
         switch (e.get_expr_type()) {
         case e_val: return e;
         case e_op: {
             if (e.get_op_type() == o_access) {
-                long dt, dy, dx;
-                if (e.get_name() != S->get_name() || e.get_access().size() != 3 || !var_plus_const(e.get_access()[0], its[0], dt) ||
-                    !var_plus_const(e.get_access()[1], its[1], dy) || !var_plus_const(e.get_access()[2], its[2], dx) || dt != -1) {
+                long dt = -1, dy, dx;
+                if (planar && source_name.empty() && e.get_name() != S->get_name()) source_name = e.get_name();
+                const size_t first = planar ? 0 : 1;
+                if (e.get_name() != source_name || e.get_access().size() != its.size() || (!planar && !var_plus_const(e.get_access()[0], its[0], dt)) ||
+                    !var_plus_const(e.get_access()[first], yi, dy) || !var_plus_const(e.get_access()[first + 1], xi, dx) || dt != -1) {
                     ok = false;
                     return e;
                 }
@@ -166,15 +176,32 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     if (!ok || radius < 1 || radius > 4) return false;
 
     // store relation and buffer
-    buffer *B = leaf->lhs;
-    if (!B || B->get_location() != memory_location::global || B->get_n_dims() != 3 || !B->has_constant_extents()) return false;
-    if (lir::simplify(B->get_dim_sizes()[0]).get_int_val() != 2) return false;
-    const long NY = lir::simplify(B->get_dim_sizes()[1]).get_int_val(), NX = lir::simplify(B->get_dim_sizes()[2]).get_int_val();
-    if (!access_equals(S, "{ " + S->get_name() + "[t,y,x] -> " + B->get_name() + "[t mod 2, y, x] }")) return false;
+    buffer *B = leaf->lhs, *BI = nullptr;
+    if (!B || B->get_location() != memory_location::global || B->get_n_dims() != (planar ? 2 : 3) || !B->has_constant_extents()) return false;
+    if (!planar && lir::simplify(B->get_dim_sizes()[0]).get_int_val() != 2) return false;
+    const long NY = lir::simplify(B->get_dim_sizes()[planar ? 0 : 1]).get_int_val(), NX = lir::simplify(B->get_dim_sizes()[planar ? 1 : 2]).get_int_val();
+    if (planar) {
+        // both computations stored as they are indexed, in two float buffers of the same shape
+        if (source_name.empty()) return false;
+        auto sources = f->get_computation_by_name(source_name);
+        if (sources.size() != 1 || sources[0]->get_data_type() != p_float32) return false;
+        BI = sources[0]->get_buffer();
+        if (!BI || BI == B || BI->get_location() != memory_location::global || BI->get_n_dims() != 2 || !BI->has_constant_extents() ||
+            BI->get_elements_type() != p_float32 || B->get_elements_type() != p_float32) return false;
+        if (lir::simplify(BI->get_dim_sizes()[0]).get_int_val() != NY || lir::simplify(BI->get_dim_sizes()[1]).get_int_val() != NX) return false;
+        if (!access_equals(S, "{ " + S->get_name() + "[y,x] -> " + B->get_name() + "[y, x] }") ||
+            !access_equals(sources[0], "{ " + source_name + "[y,x] -> " + BI->get_name() + "[y, x] }")) return false;
+    } else if (!access_equals(S, "{ " + S->get_name() + "[t,y,x] -> " + B->get_name() + "[t mod 2, y, x] }")) {
+        return false;
+    }
 
     // iteration domain: a box that keeps the stencil inside the plane
     std::vector<long> lo, hi;
     if (!literal_box(S, lo, hi)) return false;
+    if (planar) {                      // as one time step
+        lo.insert(lo.begin(), 1);
+        hi.insert(hi.begin(), 1);
+    }
     if (lo[1] - radius < 0 || hi[1] + radius > NY - 1 || lo[2] - radius < 0 || hi[2] + radius > NX - 1) return false;
 
     // ---- plan.  On return both planes must hold exactly what the un-tiled loop leaves there: the last step in
@@ -211,8 +238,10 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
         return out;
     };
     std::vector<chunk> chunks;
-    const bool temp_plane = steps >= 3 && env_int("TIRAMISU_STENCIL_TEMP_PLANE", 1) != 0;
-    if (temp_plane) {
+    const bool temp_plane = !planar && steps >= 3 && env_int("TIRAMISU_STENCIL_TEMP_PLANE", 1) != 0;
+    if (planar) {
+        chunks.push_back({T0, 1, 3});
+    } else if (temp_plane) {
         // the final launch's length: the one that needs the fewest launches (the longest of those)
         int best = 2;
         size_t best_n = 0;
@@ -238,12 +267,12 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     auto floor_div = [](long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); };
     // one launch per chunk: the boundary slices ride behind the interior tiles (TIRAMISU_STENCIL_MERGE=0: two launches)
     const bool merge = env_int("TIRAMISU_STENCIL_MERGE", 1) != 0;
-    static const char *const mode_text[] = {"", ", into a third plane", ", from a third plane into both planes"};
+    static const char *const mode_text[] = {"", ", into a third plane", ", from a third plane into both planes", ", out of place"};
     host << "    {\n";
     if (temp_plane)
         host << "        static thread_local float *_st_temp = nullptr;   // third plane: allocated at the first call, kept\n"
              << "        if (!_st_temp) _st_temp = (float *)tiramisu_hip_malloc((uint64_t)" << NY << " * " << NX << " * sizeof(float));\n";
-    else
+    else if (!planar)
         host << "        float *_st_temp = nullptr;\n";
     for (auto &ch : chunks) {
         const std::pair<int, int> key(ch.steps, ch.mode);
@@ -283,14 +312,17 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
             k.source = s.str();            // both kernels come from the one inclusion
             ke.source = "";
             for (kernel *q : {&k, &ke}) {
-                q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}, {true, "_st_temp", p_float32}};
+                // the kernel reads plane _st_src of its first buffer; out of place the source is that buffer and the
+                // destination comes in the place of the third plane
+                if (planar) q->params = {{true, BI->get_name(), p_float32}, {false, "_st_src", p_int32}, {true, B->get_name(), p_float32}};
+                else q->params = {{true, B->get_name(), B->get_elements_type()}, {false, "_st_src", p_int32}, {true, "_st_temp", p_float32}};
                 q->block[0] = std::to_string(64 * WAVES);
             }
             k.grid[0] = std::to_string(merge ? interior + edge_tiles * edge_sub : interior);
             ke.grid[0] = std::to_string(merge ? 0 : edge_tiles * edge_sub);
             by_steps[key] = {k, ke};
         }
-        const long src = (((ch.first - 1) % 2) + 2) % 2;
+        const long src = planar ? 0 : (((ch.first - 1) % 2) + 2) % 2;
         auto &pr = by_steps[key];
         host << "        {\n            const int32_t _st_src = " << src << ";  // steps " << ch.first << ".." << ch.first + ch.steps - 1 << "\n";
         if (pr.first.grid[0] != "0") host << launch_text(pr.first, "            ");
