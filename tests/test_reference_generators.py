@@ -75,7 +75,7 @@ def load(name):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N", [(48, 64), (37, 53)])
+@pytest.mark.parametrize("M,N", [(48, 64), (37, 53), (1, 70), (70, 1), (129, 257)])   # whole tiles, ragged, a single row / column
 def test_reference_cvtcolorgpu(M, N):
     rgb = np.random.RandomState(M).randint(0, 256, (3, M, N)).astype(np.uint8)
     out = np.zeros((M, N), np.uint8)
@@ -120,7 +120,7 @@ def test_reference_convolutiongpu(M, N):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("M,N", [(48, 64), (37, 53)])
+@pytest.mark.parametrize("M,N", [(48, 64), (37, 53), (1, 70), (70, 1)])
 def test_reference_fusiongpu(M, N):
     img = np.random.RandomState(M * N).randint(0, 256, (3, M, N)).astype(np.uint8)
     outs = [np.zeros((3, M, N), np.uint8) for _ in range(4)]
