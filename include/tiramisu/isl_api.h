@@ -167,6 +167,17 @@ char *isl_union_map_to_str(isl_union_map *umap);
 isl_map *isl_map_from_union_map(isl_union_map *umap);
 isl_union_map *isl_union_map_intersect_domain(isl_union_map *umap, isl_union_set *uset);
 isl_union_set *isl_union_set_from_set(isl_set *set);
+isl_bool isl_union_map_is_equal(isl_union_map *a, isl_union_map *b);
+
+/* dataflow analysis: the last write (must source) that every read (sink) sees under a schedule */
+typedef struct isl_union_access_info isl_union_access_info;
+typedef struct isl_union_flow isl_union_flow;
+isl_union_access_info *isl_union_access_info_from_sink(isl_union_map *sink);
+isl_union_access_info *isl_union_access_info_set_must_source(isl_union_access_info *access, isl_union_map *must_source);
+isl_union_access_info *isl_union_access_info_set_schedule_map(isl_union_access_info *access, isl_union_map *schedule_map);
+isl_union_flow *isl_union_access_info_compute_flow(isl_union_access_info *access);
+isl_union_map *isl_union_flow_get_must_dependence(isl_union_flow *flow);
+isl_union_flow *isl_union_flow_free(isl_union_flow *flow);
 isl_union_set *isl_union_set_free(isl_union_set *uset);
 isl_union_map *isl_union_map_reverse(isl_union_map *umap);
 

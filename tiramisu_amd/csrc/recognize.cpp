@@ -87,6 +87,54 @@ bool access_equals(computation *C, const std::string &expected) {
     return eq;
 }
 
+// Dataflow check of the time-iterated stencil, on the program as scheduled: with S stored at B[t mod 2, y, x] and
+// reading B[(t-1) mod 2, y+dy, x+dx], the last write that each read sees (isl's flow analysis over S's
+// schedule) must be exactly the previous step's instance at the offset cell, wherever that cell is in the
+// iteration domain -- i.e. the flow dependences are { S[t-1, y+dy, x+dx] -> S[t, y, x] } and nothing else.
+// Cells outside the domain have no source: they hold what the buffer held on entry.
+bool flow_is_previous_step(computation *S, buffer *B, const std::vector<std::pair<long, long>> &taps) {
+    isl_ctx *ctx = S->get_ctx();
+    const std::string s = S->get_name(), b = B->get_name();
+    auto restricted = [&](const std::string &text) {
+        isl_union_map *m = isl_union_map_read_from_str(ctx, text.c_str());
+        return m ? isl_union_map_intersect_domain(m, isl_union_set_from_set(isl_set_copy(S->get_iteration_domain()))) : nullptr;
+    };
+    isl_union_map *writes = restricted("{ " + s + "[t,y,x] -> " + b + "[t mod 2, y, x] }");
+    isl_union_map *reads = nullptr, *expected = nullptr;
+    for (auto &tap : taps) {
+        const std::string dy = std::to_string(tap.first), dx = std::to_string(tap.second);
+        isl_union_map *r = restricted("{ " + s + "[t,y,x] -> " + b + "[(t - 1) mod 2, y + (" + dy + "), x + (" + dx + ")] }");
+        // source instance -> sink instance, both inside the domain
+        isl_union_map *e = restricted("{ " + s + "[t,y,x] -> " + s + "[t + 1, y - (" + dy + "), x - (" + dx + ")] }");
+        if (e) e = isl_union_map_intersect_domain(isl_union_map_reverse(e), isl_union_set_from_set(isl_set_copy(S->get_iteration_domain())));
+        if (e) e = isl_union_map_reverse(e);
+        reads = reads ? isl_union_map_union(reads, r) : r;
+        expected = expected ? isl_union_map_union(expected, e) : e;
+    }
+    isl_map *sched = isl_map_project_out(isl_map_copy(S->get_schedule()), isl_dim_out, 0, 1);   // the duplicate dimension
+    sched = isl_map_intersect_domain(sched, isl_set_copy(S->get_iteration_domain()));
+    bool ok = false;
+    if (writes && reads && expected && sched) {
+        isl_union_access_info *info = isl_union_access_info_from_sink(reads);
+        info = isl_union_access_info_set_must_source(info, writes);
+        info = isl_union_access_info_set_schedule_map(info, isl_union_map_from_map(sched));
+        reads = writes = nullptr;
+        sched = nullptr;
+        isl_union_flow *flow = isl_union_access_info_compute_flow(info);
+        if (flow) {
+            isl_union_map *dep = isl_union_flow_get_must_dependence(flow);
+            ok = dep && isl_union_map_is_equal(dep, expected) == isl_bool_true;
+            if (dep) isl_union_map_free(dep);
+            isl_union_flow_free(flow);
+        }
+    }
+    if (writes) isl_union_map_free(writes);
+    if (reads) isl_union_map_free(reads);
+    if (expected) isl_union_map_free(expected);
+    if (sched) isl_map_free(sched);
+    return ok;
+}
+
 void leaves_under(const node_ptr &n, std::vector<node_ptr> &out, bool &has_cond) {
     lir::walk(n, [&](const node_ptr &x) {
         if (x->kind == node_kind::leaf) out.push_back(x);
@@ -142,6 +190,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     int radius = 0;
     bool ok = true;
     std::string source_name = planar ? std::string() : S->get_name();
+    std::vector<std::pair<long, long>> taps;
     std::function<expr(const expr &)> rewrite = [&](const expr &e) -> expr {
         if (!e.is_defined()) { ok = false; return e; }
         switch (e.get_expr_type()) {
@@ -157,6 +206,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
                     return e;
                 }
                 radius = std::max<long>(radius, std::max(std::labs(dy), std::labs(dx)));
+                if (std::find(taps.begin(), taps.end(), std::make_pair(dy, dx)) == taps.end()) taps.push_back({dy, dx});
                 return expr(o_call, "ST_AT", {expr((int32_t)dy), expr((int32_t)dx)}, p_float32);
             }
             if (e.get_op_type() == o_call) { ok = false; return e; }
@@ -192,6 +242,8 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
         if (!access_equals(S, "{ " + S->get_name() + "[y,x] -> " + B->get_name() + "[y, x] }") ||
             !access_equals(sources[0], "{ " + source_name + "[y,x] -> " + BI->get_name() + "[y, x] }")) return false;
     } else if (!access_equals(S, "{ " + S->get_name() + "[t,y,x] -> " + B->get_name() + "[t mod 2, y, x] }")) {
+        return false;
+    } else if (!std::getenv("TIRAMISU_STENCIL_NO_FLOW_CHECK") && !flow_is_previous_step(S, B, taps)) {
         return false;
     }
 
