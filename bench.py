@@ -6,7 +6,7 @@
 Prints ONE JSON line.  The headline is benchmark configuration 2 (heat2d 8192x8192, 32 time steps,
 the configuration the HBM-roofline target is quoted on).  A "step" is one call of the compiled
 Tiramisu function (32 stencil time steps) with its buffers already resident in HBM.  The compiled
-function fuses up to 11 time steps per launch, so it moves far fewer bytes than the un-fused
+function fuses up to 12 time steps per launch, so it moves far fewer bytes than the un-fused
 program's 8 bytes per cell and time step: `value` is the HBM traffic the function really causes
 (hardware counters, per kernel, from profiles/hbm_traffic_by_kernel.md) per second, and
 `algorithmic_gbs` -- the un-fused program's bytes per second of this run, the figure that time
@@ -18,7 +18,10 @@ HIP events around every launch (the runtime ABI's tiramisu_hip_profile_*) on the
 generated code launches on: flops per launch over duration against the MFMA peak for the
 contractions; counter-measured HBM bytes per launch over duration against the HBM peak for the
 stencil (`frac` <= 1 by construction; `algorithmic_gbs` and `vector_alu_busy` say why a fused
-launch sits below the HBM peak).  `traffic` is looked up by the emitter's own description of the
+launch sits below the HBM peak).  A kernel launched many times per call in a dependent chain (the
+LSTM's cell kernel) takes its launch duration from the timed region instead -- the call minus the other
+kernels, over its launches -- because events between dependent launches cost a launch themselves; the
+per-event figure stays in `kernel_ms_between_events`.  `traffic` is looked up by the emitter's own description of the
 kernel, so a kernel the table does not know reports null instead of a stale figure.
 `cpu_baseline` times the CPU-generated code of the same Tiramisu program (the oracle's CPU
 back-end restatement: parallelize + vectorize schedule, OpenMP) on the host cores of this machine.
