@@ -148,8 +148,10 @@ void leaves_under(const node_ptr &n, std::vector<node_ptr> &out, bool &has_cond)
 // Stencil over a ping-pong pair of planes inside a host time loop:
 //     S(t, y, x) = f( S(t-1, y+dy, x+dx) ... ),   S stored at B[t mod 2, y, x].
 // Every read at step t is of step t-1 within a constant radius, so all flow dependences have
-// distance (1, dy, dx) and overlapped time tiles are legal; the time loop is replaced by
-// launches that each advance an odd number of steps (see kernels/stencil2d_regs.hip.h).
+// distance (1, dy, dx) (flow_is_previous_step checks that on the scheduled program with isl's dataflow
+// analysis) and overlapped time tiles are legal; the time loop is replaced by
+// launches that each advance several steps (see kernels/stencil2d_regs.hip.h).  The second form is a single
+// step out of place:  S(y, x) = f( I(y+dy, x+dx) ... )  with I and S in buffers of their own.
 bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop, launch_plan &plan) {
     // either a host time loop around a mapped nest, or a mapped nest whose time step is fixed
     // (a one-step time loop has no loop node in the AST)
