@@ -272,6 +272,28 @@ def bench_copy(steps, warmup, with_cpu):
     return out
 
 
+def bench_sweep5(steps, warmup, with_cpu):
+    """One 5-point sweep out of place on 8192 x 8192 floats (programs/stencil_sweep.cpp): the stencil back-end's
+    single-step form.  Bytes: the plane read once and written once."""
+    from tiramisu_amd import runtime
+    n = 8192
+    rng = np.random.RandomState(3)
+    dS, dD = device_array(rng.uniform(0, 1, (n, n)).astype(np.float32)), device_array(np.zeros((n, n), np.float32))
+    prog = runtime.load(PROGRAMS, "sweep5_8192x8192")
+    args = (dS.buffer(), dD.buffer())
+    ms = time_steps(lambda: prog(*args), steps, warmup)
+    prof = kernel_profile(lambda: prog(*args), steps)
+    dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
+    nbytes = 2.0 * n * n * 4
+    out = {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
+           "roofline": {"bound": "hbm", "achieved": nbytes / (dom[1][0] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / (dom[1][0] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": (kernel_traffic("sweep5_8192x8192", dom[0]) or {}).get("bytes"),
+                        "kernel": dom[0], "kernel_ms": dom[1][0]}}
+    dS.free()
+    dD.free()
+    return out
+
+
 def _generic_bench(name, host_arrays, flop, peak_tflops, steps, warmup, with_cpu, cpu_sample, dominant_flop_share=1.0):
     """A compiled function whose arguments are all GPU-resident (except leading host scalars)."""
     from tiramisu_amd import runtime
@@ -394,8 +416,9 @@ def main():
     if runtime.wrappers().tiramisu_hip_device_count() < 1:
         sys.exit("no HIP device visible")
     WORKLOADS["copy"] = bench_copy   # calibration only, not part of "all"
+    WORKLOADS["sweep5"] = bench_sweep5   # the single-step form of the stencil back-end, not part of "all"
     WORKLOADS["sgemm_cache_shared"] = bench_sgemm_cache_shared   # profiling of the schedule-faithful emitter only
-    names = [n for n in WORKLOADS if n not in ("copy", "sgemm_cache_shared")] if a.workload == "all" else [a.workload]
+    names = [n for n in WORKLOADS if n not in ("copy", "sweep5", "sgemm_cache_shared")] if a.workload == "all" else [a.workload]
     results = {}
     for n in names:
         with_cpu = not a.no_cpu

@@ -56,6 +56,5 @@ int main()
     sweep5(45, 39);       // rows not a multiple of 4 elements: element loads
     wide9(200, 520);
     wide9(70, 50);
-    sweep5(8192, 8192);   // the size of the benchmark plane, for timing
     return 0;
 }
