@@ -83,3 +83,18 @@ def test_workgroups_are_renumbered_where_tiles_share_data(programs_dir, product_
     assert re.search(r"const int32_t c\d+ = \(int32_t\)_tile\.[xy] \+ 0;", shared) and "blockIdx.x + gridDim.x * blockIdx.y" in shared
     for text in (kernel_source(product_programs_dir, "copy_plane"), kernel_source(programs_dir, "lanes_follow_unit_stride")):
         assert "workgroups renumbered" not in text and "_tile" not in text
+
+
+def test_the_mapping_passes_can_be_switched_off(programs_dir, tmp_path, monkeypatch):
+    # the reference's own mapping: thread dimensions from the innermost tagged level outwards, the program's
+    # tiles as workgroups, workgroups in hardware order
+    from tiramisu_amd import build
+    for knob in ("TIRAMISU_HIP_KEEP_THREAD_DIMENSIONS", "TIRAMISU_HIP_KEEP_TILES", "TIRAMISU_HIP_KEEP_BLOCK_ORDER"):
+        monkeypatch.setenv(knob, "1")
+    build.build_program(os.path.join(programs_dir, "lane_dimension.cpp"), directory=str(tmp_path))
+    text = open(os.path.join(str(tmp_path), "build", "lanes_follow_unit_stride.o.hip")).read()
+    assert "// _kernel_0: generic\n" in text
+    # the innermost tagged loop (over y, the strided index) sits on threadIdx.x again
+    x_iterator = re.search(r"const int32_t (c\d+) = \(int32_t\)threadIdx\.x \+ 0;", text).group(1)
+    store = re.search(r"b_out\[(.*?)\] = ", text).group(1)
+    assert re.search(r"\+ %s\) \* 150\)" % x_iterator, store), store
