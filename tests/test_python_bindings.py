@@ -84,3 +84,27 @@ def test_heat2d_written_in_python():
     d = DeviceArray(planes)
     runtime.load(PROGRAMS, "heat2d_py")(d.buffer())
     assert np.array_equal(d.download(), ref.heat2d(grid, STEPS))
+
+
+def test_every_name_of_the_reference_stub_exists(tm):
+    """Classes, their methods and the module's functions of the reference's python_bindings/tiramisu.pyi (read
+    where it lies; skipped where the tree is absent) exist in this module under the same names."""
+    stub = "/root/reference/python_bindings/tiramisu.pyi"
+    if not os.path.exists(stub):
+        pytest.skip("reference tree absent")
+    t = tm
+    missing, current = [], None
+    for line in open(stub):
+        m = re.match(r"^class ([A-Za-z_0-9]+)", line)
+        if m:
+            current = m.group(1)
+            if not hasattr(t, current):
+                missing.append(current)
+            continue
+        m = re.match(r"^    def ([a-zA-Z_][a-zA-Z_0-9]*)", line)
+        if m and current and hasattr(t, current) and not m.group(1).startswith("__") and not hasattr(getattr(t, current), m.group(1)):
+            missing.append(current + "." + m.group(1))
+        m = re.match(r"^def ([a-zA-Z_][a-zA-Z_0-9]*)", line)
+        if m and not hasattr(t, m.group(1)):
+            missing.append(m.group(1))
+    assert not missing, sorted(set(missing))

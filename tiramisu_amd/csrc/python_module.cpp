@@ -25,6 +25,7 @@ void define_types(py::module &m) {
         .value("p_float32", p_float32).value("p_float64", p_float64).value("p_boolean", p_boolean)
         .value("p_bfloat16", p_bfloat16).value("p_none", p_none)
         .export_values();
+    py::enum_<rank_t>(m, "rank_t").value("r_sender", rank_t::r_sender).value("r_receiver", rank_t::r_receiver).export_values();
     py::enum_<argument_t>(m, "argument_t")
         .value("a_input", a_input).value("a_output", a_output).value("a_temporary", a_temporary).export_values();
     py::enum_<expr_t>(m, "expr_t")
@@ -63,6 +64,7 @@ void define_expr(py::module &m) {
         .def(py::init<op_t, std::string, std::vector<expr>, primitive_t>())
         .def("cast", [](const expr &x, primitive_t t) { return cast(t, x); })
         .def("is_equal", &expr::is_equal)
+        .def("set_name", &expr::set_name)
         .def("get_name", [](const expr &x) { return x.get_name(); })
         .def("get_data_type", &expr::get_data_type)
         .def("get_int_val", &expr::get_int_val)

@@ -23,14 +23,16 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _PKG = os.path.dirname(os.path.dirname(_HERE))      # tiramisu_amd/
 
 
-def pycodegen(arguments, obj_filename, gen_gpu=True, *unused):
+def pycodegen(arguments, obj_filename, gen_gpu=True, *unused, _function=None):
     """Generate ``obj_filename`` for the implicit function, link it into ``lib<function>.so`` next
     to it and register a module ``<function>`` whose attribute ``<function>`` runs the code."""
-    if isinstance(gen_gpu, _ext.hardware_architecture_t):
+    if _function is not None:
+        _function.codegen(arguments, obj_filename, bool(gen_gpu), False)
+    elif isinstance(gen_gpu, _ext.hardware_architecture_t):
         _ext.codegen(arguments, obj_filename, gen_gpu)
     else:
         _ext.codegen(arguments, obj_filename, bool(gen_gpu))
-    name = _ext.get_implicit_function().get_name()
+    name = (_function or _ext.get_implicit_function()).get_name()
     directory = os.path.dirname(os.path.abspath(obj_filename))
     library = os.path.join(directory, "lib%s.so" % name)
     subprocess.run(["g++", "-shared", "-o", library, os.path.abspath(obj_filename), "-L" + _PKG, "-ltiramisu_hip_wrappers",
@@ -45,3 +47,12 @@ def pycodegen(arguments, obj_filename, gen_gpu=True, *unused):
     setattr(module, name, runtime.Program(library, name))
     sys.modules[name] = module
     return module
+
+
+def _function_pycodegen(self, arguments, obj_filename, gen_gpu=True):
+    """``function.pycodegen`` of the reference's bindings (python_bindings/tiramisu.pyi:309): pycodegen for a
+    function object instead of the implicit one."""
+    return pycodegen(arguments, obj_filename, gen_gpu, _function=self)
+
+
+_ext.function.pycodegen = _function_pycodegen
