@@ -23,6 +23,7 @@ struct isl_ctx;
 struct isl_set;
 struct isl_map;
 struct isl_ast_node;
+struct isl_union_map;
 
 namespace tiramisu {
 
@@ -47,6 +48,14 @@ void codegen(const std::vector<buffer *> &arguments, const std::string obj_filen
              const bool gen_gpu = false);
 void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
              const hardware_architecture_t gen_architecture_flag);
+
+/** The same calls on the implicit function (reference: core.h:139-181). */
+void perform_full_dependency_analysis();
+bool check_legality_of_function();
+void prepare_schedules_for_legality_checks(bool reset_static_dimesion = false);
+bool loop_parallelization_is_legal(var i, std::vector<computation *> fused_computations);
+bool loop_unrolling_is_legal(var i, std::vector<computation *> fused_computations);
+bool loop_vectorization_is_legal(var i, std::vector<computation *> fused_computations);
 
 /** GPU memory spaces of a buffer (reference: cuda_ast.h:180-188). */
 enum class memory_location { host, global, shared, local, constant, reg };
@@ -180,6 +189,52 @@ public:
     void dump_time_processor_domain() const;
     void dump_trimmed_time_processor_domain() const { dump_time_processor_domain(); }
     constant *get_invariant_by_name(std::string str) const;
+
+    // ---- dependence analysis and legality of schedules
+    //      (reference: tiramisu_function.cpp:165-357, :2618-3047, :3091-3660; core.h:1236-1330)
+    /** Results of perform_full_dependency_analysis(), each { source instance -> [sink instance -> buffer cell] }
+      * over the iteration domains: the last write before every read, the reads before every write that no write
+      * between them hides, the last write before every write; then { instance -> cell } for the reads that see no
+      * write of this function and for the writes that nothing overwrites. */
+    isl_union_map *dep_read_after_write = nullptr;
+    isl_union_map *dep_write_after_read = nullptr;
+    isl_union_map *dep_write_after_write = nullptr;
+    isl_union_map *live_in_access = nullptr;
+    isl_union_map *live_out_access = nullptr;
+    /** Dataflow analysis of the program as scheduled at the time of the call: call it once every computation has
+      * its buffer (store_in) and before the schedule commands whose legality is in question. */
+    void perform_full_dependency_analysis();
+    void calculate_dep_flow(bool global_memory_only = false);
+    /** Aligns and orders the schedules (after/then/between) so that they can be compared; \p reset_static_dimesion
+      * first clears the ordering an earlier call left in the static dimensions. */
+    void prepare_schedules_for_legality_checks(bool reset_static_dimesion = false);
+    void reset_all_static_dims_to_zero();
+    /** True when, under the present schedules, the source of every dependence is executed strictly before its
+      * sink; the second form looks only at dependences between the computations given. */
+    bool check_legality_for_function();
+    bool check_partial_legality_in_function(std::vector<computation *> involved_computations);
+    /** True when no dependence between the computations given (fused in that loop) is carried by loop \p i. */
+    bool loop_parallelization_is_legal(var i, std::vector<computation *> fused_computations);
+    bool loop_parallelization_is_legal(int parallel_dim, std::vector<computation *> fused_computations);
+    /** True when the bounds of loop \p i are one affine expression of the outer loops each (no min/max). */
+    bool loop_unrolling_is_legal(var i, std::vector<computation *> fused_computations);
+    bool loop_vectorization_is_legal(var i, std::vector<computation *> fused_computations);
+    /** The smallest non-negative shifts of \p current along \p vars_subjected_to_shifting (lexicographically,
+      * outer loop first) that make every dependence between it and \p previous_computations -- the computations
+      * fused before it -- legal; one (var, shift) per variable, or nothing when no shift does or a dependence
+      * distance is not constant up to the innermost of the variables. */
+    std::vector<std::tuple<var, int>> correcting_loop_fusion_with_shifting(std::vector<computation *> previous_computations,
+                                                                          computation &current,
+                                                                          std::vector<var> vars_subjected_to_shifting);
+    /** The race check of the GPU mapping: one line for every loop tagged as a block or thread dimension that, in
+      * the program as scheduled now, carries a dependence through global memory (what goes through LDS is ordered
+      * by the program's barriers and is left out).  codegen() for the GPU calls it and stops on a finding when
+      * the environment variable TIRAMISU_HIP_CHECK_MAPPED_LOOPS is set. */
+    std::vector<std::string> gpu_mapped_loops_that_carry_dependences();
+    /** The five results of the analysis, one "name: relation" line each. */
+    std::string dependences_as_text() const;
+    /** Every dependence as { source instance -> sink instance }. */
+    isl_union_map *get_statement_dependences() const;
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
                  const hardware_architecture_t arch);
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
@@ -469,6 +524,12 @@ public:
     virtual void skew(var i, var j, var k, int factor);
     virtual void skew(var i, var j, var k, var l, int factor);
     virtual void skew(int i, int j, int k, int l, int factor);
+    /** Legality of the present schedules for the dependences from this computation to \p second
+      * (reference: tiramisu_core.cpp:4695-4904); after function::perform_full_dependency_analysis(). */
+    virtual bool involved_subset_of_dependencies_is_legal(computation *second);
+    /** True when the bounds of loop \p l are single affine expressions of the loops around it
+      * (reference: tiramisu_core.cpp:4906-5011). */
+    virtual bool unrolling_is_legal(var l);
     virtual void loop_reversal(var old_var, var new_var);
     virtual void loop_reversal(int i);
     virtual void parallelize(var L);

@@ -177,8 +177,31 @@ isl_union_access_info *isl_union_access_info_set_must_source(isl_union_access_in
 isl_union_access_info *isl_union_access_info_set_schedule_map(isl_union_access_info *access, isl_union_map *schedule_map);
 isl_union_flow *isl_union_access_info_compute_flow(isl_union_access_info *access);
 isl_union_map *isl_union_flow_get_must_dependence(isl_union_flow *flow);
+isl_union_access_info *isl_union_access_info_set_may_source(isl_union_access_info *access, isl_union_map *may_source);
+isl_union_access_info *isl_union_access_info_set_kill(isl_union_access_info *access, isl_union_map *kill);
+/* { source -> [sink -> memory cell] }: the dependence together with the cell it goes through */
+isl_union_map *isl_union_flow_get_full_must_dependence(isl_union_flow *flow);
+isl_union_map *isl_union_flow_get_full_may_dependence(isl_union_flow *flow);
+/* the sink accesses that no source writes before them */
+isl_union_map *isl_union_flow_get_must_no_source(isl_union_flow *flow);
+isl_union_map *isl_union_map_range_factor_domain(isl_union_map *umap);
+isl_union_map *isl_union_map_range_factor_range(isl_union_map *umap);
+isl_union_map *isl_union_map_subtract(isl_union_map *a, isl_union_map *b);
+isl_union_map *isl_union_map_apply_range(isl_union_map *a, isl_union_map *b);
+isl_union_map *isl_union_map_apply_domain(isl_union_map *a, isl_union_map *b);
+isl_union_map *isl_union_map_intersect_range(isl_union_map *umap, isl_union_set *uset);
+isl_union_map *isl_union_map_coalesce(isl_union_map *umap);
+isl_bool isl_union_map_is_empty(isl_union_map *umap);
+isl_stat isl_union_map_foreach_map(isl_union_map *umap, isl_stat (*fn)(isl_map *map, void *user), void *user);
+isl_stat isl_map_foreach_basic_map(isl_map *map, isl_stat (*fn)(isl_basic_map *bmap, void *user), void *user);
+isl_map *isl_map_from_basic_map(isl_basic_map *bmap);
+isl_map *isl_map_lex_ge(isl_space *set_space);
+isl_space *isl_space_range(isl_space *space);
+isl_set *isl_map_params(isl_map *map);
+isl_map *isl_map_subtract(isl_map *a, isl_map *b);
 isl_union_flow *isl_union_flow_free(isl_union_flow *flow);
 isl_union_set *isl_union_set_free(isl_union_set *uset);
+isl_union_set *isl_union_set_copy(isl_union_set *uset);
 isl_union_map *isl_union_map_reverse(isl_union_map *umap);
 
 // piecewise affine functions

@@ -22,4 +22,5 @@ def test_reference_test_passes(n):
     assert os.path.exists(program), "not built: run tests/reference_programs/build_reference_programs.py where the reference tree is"
     r = subprocess.run([program], cwd=os.path.dirname(program), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert r.returncode == 0, r.stdout[-2000:]
-    assert "succeeded" in r.stdout and "failed" not in r.stdout.lower(), r.stdout[-2000:]
+    assert "failed" not in r.stdout.lower(), r.stdout[-2000:]
+    assert "succeeded" in r.stdout or n in brp.SUITE_SILENT, r.stdout[-2000:]

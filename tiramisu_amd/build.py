@@ -26,7 +26,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 COMPILER_SOURCES = ["expr.cpp", "core.cpp", "astgen.cpp", "c_print.cpp", "hip_backend.cpp",
-                    "recognize.cpp"]
+                    "recognize.cpp", "dependences.cpp"]
 
 PROGRAM_DIRS = [os.path.join(PKG, "programs"), os.path.join(ROOT, "tests", "programs")]
 

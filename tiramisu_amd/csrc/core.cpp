@@ -351,6 +351,15 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
     }
     set_arguments(arguments);
     gen_time_space_domain();
+    if (arch == hardware_architecture_t::arch_amd_gpu && std::getenv("TIRAMISU_HIP_CHECK_MAPPED_LOOPS")) {
+        const std::vector<std::string> races = gpu_mapped_loops_that_carry_dependences();
+        bool refuse = false;
+        for (auto &r : races) {
+            std::cerr << "GPU mapping: " << r << std::endl;
+            refuse |= r.find("carries a dependence") != std::string::npos;      // a reduction is only reported
+        }
+        if (refuse) ERROR("loops mapped to the GPU carry dependences", true);
+    }
     gen_isl_ast();
     b->generate(*this, get_lowered_program(), obj_filename);
 }
@@ -1643,7 +1652,7 @@ computation *computation::select(int duplicate_id) {
 }
 
 // { consumer[iterators] -> producer[indices] } for every read of `producer` in the consumer's expression and predicate
-static isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain = true) {
+isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain) {
     function *f = consumer.get_function();
     const std::string wanted = producer.get_first_definition()->get_name();
     std::vector<std::string> pieces;

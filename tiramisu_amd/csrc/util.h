@@ -25,5 +25,10 @@ class expr;
 /** isl syntax for an integer (quasi-)affine expression; sets \p ok to false otherwise. */
 std::string expr_to_isl_str(const expr &e, bool &ok);
 
+class computation;
+/** { consumer[iterators] -> producer[indices] } for every read of \p producer in the consumer's expression and
+  * predicate, over the consumer's iteration domain (and, on request, inside the producer's); null if none. */
+struct isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain = true);
+
 }  // namespace tiramisu
 #endif
