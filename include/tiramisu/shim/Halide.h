@@ -41,7 +41,8 @@ template <> struct type_code<bool> { static constexpr uint8_t value = 1; };
 template <class T>
 class Buffer {
     struct storage {
-        std::unique_ptr<T[]> data;           // a plain array: Buffer<bool> must hand out bool *
+        std::unique_ptr<T[]> owned;          // a plain array: Buffer<bool> must hand out bool *
+        T *data = nullptr;                   // the array above, or memory of the caller's
         size_t count = 0;
         std::vector<halide_dimension_t> dims;
         halide_buffer_t raw;
@@ -49,7 +50,7 @@ class Buffer {
     };
     std::shared_ptr<storage> s;   // copies share the array, as Halide's do
 
-    void build(const std::vector<int> &extents) {
+    void build(const std::vector<int> &extents, T *existing = nullptr) {
         s = std::make_shared<storage>();
         size_t count = 1;
         s->dims.resize(extents.empty() ? 1 : extents.size());
@@ -58,32 +59,47 @@ class Buffer {
             count *= (size_t)extents[d];
         }
         s->count = count;
-        s->data.reset(new T[count > 0 ? count : 1]());
+        if (!existing) s->owned.reset(new T[count > 0 ? count : 1]());
+        s->data = existing ? existing : s->owned.get();
         std::memset(&s->raw, 0, sizeof(s->raw));
-        s->raw.host = reinterpret_cast<uint8_t *>(s->data.get());
+        s->raw.host = reinterpret_cast<uint8_t *>(s->data);
         s->raw.type = halide_type_t{shim::type_code<T>::value, (uint8_t)(8 * sizeof(T)), 1};
         s->raw.dimensions = (int32_t)extents.size();
         s->raw.dim = s->dims.data();
     }
-    size_t offset(std::initializer_list<int> idx) const {
-        size_t o = 0, d = 0;
-        for (int i : idx) o += (size_t)i * (size_t)s->dims[d++].stride;
+    // indices beyond the buffer's dimensions are ignored, missing ones are 0
+    template <class... I>
+    size_t offset(I... idx) const {
+        const int list[] = {(int)idx...};
+        size_t o = 0;
+        for (int d = 0; d < (int)sizeof...(I) && d < s->raw.dimensions; d++) o += (size_t)list[d] * (size_t)s->dims[d].stride;
         return o;
+    }
+    // extents followed, optionally, by a name (a label: print_buffer shows it)
+    static void gather(std::vector<int> &, std::string &) {}
+    static void gather(std::vector<int> &, std::string &name, const std::string &nm) { name = nm; }
+    static void gather(std::vector<int> &, std::string &name, const char *nm) { name = nm; }
+    template <class... R>
+    static void gather(std::vector<int> &extents, std::string &name, int e, R... rest) {
+        extents.push_back(e);
+        gather(extents, name, rest...);
     }
 
 public:
     Buffer() { build({}); }
-    explicit Buffer(int e0) { build({e0}); }
-    Buffer(int e0, int e1) { build({e0, e1}); }
-    Buffer(int e0, int e1, int e2) { build({e0, e1, e2}); }
-    Buffer(int e0, int e1, int e2, int e3) { build({e0, e1, e2, e3}); }
+    template <class... R>
+    explicit Buffer(int e0, R... rest) {
+        std::vector<int> extents;
+        std::string nm;
+        gather(extents, nm, e0, rest...);
+        build(extents);
+        s->name = nm;
+    }
     explicit Buffer(const std::vector<int> &extents) { build(extents); }
-    // the same with a trailing name (a label: print_buffer shows it)
-    Buffer(int e0, const std::string &nm) { build({e0}); s->name = nm; }
-    Buffer(int e0, int e1, const std::string &nm) { build({e0, e1}); s->name = nm; }
-    Buffer(int e0, int e1, int e2, const std::string &nm) { build({e0, e1, e2}); s->name = nm; }
-    Buffer(int e0, int e1, int e2, int e3, const std::string &nm) { build({e0, e1, e2, e3}); s->name = nm; }
     Buffer(const std::vector<int> &extents, const std::string &nm) { build(extents); s->name = nm; }
+    // over memory that the caller owns
+    Buffer(T *existing, const std::vector<int> &extents) { build(extents, existing); }
+    Buffer(T *existing, const std::vector<int> &extents, const std::string &nm) { build(extents, existing); s->name = nm; }
 
     const std::string &name() const { return s->name; }
     halide_buffer_t *raw_buffer() { return &s->raw; }
@@ -94,8 +110,8 @@ public:
     int device_sync(void * = nullptr) { return 0; }
     void set_host_dirty(bool = true) {}
     void set_device_dirty(bool = true) {}
-    T *data() { return s->data.get(); }
-    const T *data() const { return s->data.get(); }
+    T *data() { return s->data; }
+    const T *data() const { return s->data; }
     T *begin() { return data(); }
     T *end() { return data() + s->count; }
     int dimensions() const { return s->raw.dimensions; }
@@ -109,22 +125,10 @@ public:
     void copy_from(const Buffer<T> &o) { for (size_t i = 0; i < s->count && i < o.s->count; i++) s->data[i] = o.s->data[i]; }
 
     // missing trailing indices are 0, so a 2-D buffer can be read as b(x, y, 0)
-    T &operator()(int i0) { return s->data[offset({i0})]; }
-    T &operator()(int i0, int i1) { return s->data[offset({i0, i1})]; }
-    T &operator()(int i0, int i1, int i2) { return s->data[offset3(i0, i1, i2)]; }
-    T &operator()(int i0, int i1, int i2, int i3) { return s->data[offset({i0, i1, i2, i3})]; }
-    const T &operator()(int i0) const { return s->data[offset({i0})]; }
-    const T &operator()(int i0, int i1) const { return s->data[offset({i0, i1})]; }
-    const T &operator()(int i0, int i1, int i2) const { return s->data[offset3(i0, i1, i2)]; }
-    const T &operator()(int i0, int i1, int i2, int i3) const { return s->data[offset({i0, i1, i2, i3})]; }
-
-private:
-    size_t offset3(int i0, int i1, int i2) const {
-        size_t o = 0;
-        const int idx[3] = {i0, i1, i2};
-        for (int d = 0; d < 3 && d < dimensions(); d++) o += (size_t)idx[d] * (size_t)s->dims[d].stride;
-        return o;
-    }
+    template <class... I>
+    T &operator()(int i0, I... rest) { return s->data[offset(i0, rest...)]; }
+    template <class... I>
+    const T &operator()(int i0, I... rest) const { return s->data[offset(i0, rest...)]; }
 };
 
 }  // namespace Halide

@@ -65,6 +65,36 @@ def build_test(generator_rel, wrapper_rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
+# The lattice-QCD correlator benchmarks for the GPU whose code this build generates in seconds (complex fp64
+# arithmetic through utils/complex_util.h, six kernels each; the four dibaryon programs take from ten minutes
+# upwards to generate and are left out).  Each wrapper fills random propagators and wave functions, calls the
+# generated function and the plain C++ restatement its authors wrote next to it (<...>_ref.cpp, which the wrapper
+# includes), and compares the correlators to a relative 1e-12.  Built like the tests above: generator unchanged,
+# wrapper unchanged, its main() renamed so that a test can call it in-process.
+BARYON = ["benchmarks/tensors/baryon/gpu_tiramisu_make_fused_baryon_blocks_correlator",
+          "benchmarks/tensors/baryon/gpu_tiramisu_make_fused_identical_baryon_blocks_correlator",
+          "benchmarks/tensors/baryon/gpu_single_tiramisu_make_fused_identical_baryon_blocks_correlator"]
+
+
+def build_baryon(rel):
+    name = os.path.basename(rel)
+    source = os.path.join(REFERENCE, rel)
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, name)                  # the generator writes generated_<name>.o where it runs
+    os.makedirs(work, exist_ok=True)
+    generator = [f for f in os.listdir(source) if f.endswith("_generator.cpp")][0]
+    wrapper = [f for f in os.listdir(source) if f.endswith("_wrapper.cpp")][0]
+    build.build_program(os.path.join(source, generator), directory=work, shim_headers=True)
+    objects = [os.path.join(work, f) for f in os.listdir(work) if f.endswith(".o")]
+    entry = os.path.join(bdir, "entry.h")
+    with open(entry, "w") as f:
+        f.write('extern "C" int tiramisu_wrapper_main(int, char **);\n')
+    build._run(["g++", "-std=c++17", "-O2", "-w", "-fPIC", "-shared", "-I" + build.INCLUDE,
+                "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"), "-I" + source,
+                "-include", entry, "-Dmain=tiramisu_wrapper_main", "-o", library(name), os.path.join(source, wrapper)] + objects +
+               ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
+
+
 # Benchmark generators whose wrapper needs CUDA, cuBLAS or cuDNN headers: the tests drive the
 # generated function themselves.  Each program writes its object into its working directory and
 # (all but the first LSTM) times its kernels through an external get_time(): timer_hook.c.
@@ -239,6 +269,10 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", rel, flush=True)
         build_self_driven(rel, stem, obj)
+    for rel in BARYON:
+        if verbose:
+            print("[reference programs]", rel, flush=True)
+        build_baryon(rel)
     if verbose:
         print("[reference programs] benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp (double precision)", flush=True)
     build_lstm_gpu_lib_f64()

@@ -200,6 +200,35 @@ def test_reference_gpu_test_passes(name):
     assert lib.tiramisu_wrapper_main(0, None) == 0
 
 
+BARYON = ["gpu_tiramisu_make_fused_baryon_blocks_correlator", "gpu_tiramisu_make_fused_identical_baryon_blocks_correlator",
+          "gpu_single_tiramisu_make_fused_identical_baryon_blocks_correlator"]
+
+
+@pytest.mark.parametrize("name", BARYON)
+def test_reference_baryon_library_exports_its_entry_point(name):
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    assert hasattr(ctypes.CDLL(library(name)), "tiramisu_wrapper_main")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", BARYON)
+def test_reference_baryon_correlator_passes_its_own_check(name):
+    """benchmarks/tensors/baryon/gpu_*: generator and wrapper of the reference, both unchanged.  The wrapper fills
+    random propagators, wave functions and weights, runs the generated function (six kernels in complex fp64) and
+    the C++ restatement that the reference keeps next to it, and compares every correlator entry to a relative
+    1e-12; on a difference it ends the process with status 1."""
+    if not os.path.exists(library(name)):
+        pytest.skip("reference tree was absent when the libraries were built")
+    runtime.wrappers()
+    lib = ctypes.CDLL(library(name))
+    lib.tiramisu_wrapper_main.restype = ctypes.c_int
+    lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    print("running", name, flush=True)
+    assert lib.tiramisu_wrapper_main(0, None) == 0
+
+
 TUNED_SGEMM = {"sgemm_generator1": "generic", "sgemm_generator2": "generic", "sgemm_generator3": "mfma-contraction"}
 
 
