@@ -233,6 +233,19 @@ public:
     std::vector<std::string> gpu_mapped_loops_that_carry_dependences();
     /** The five results of the analysis, one "name: relation" line each. */
     std::string dependences_as_text() const;
+    /** Skewings of two consecutive loops, from the distances of the dependences among \p fused_computations at
+      * those loops (reference: core.h:1325-1384): pairs (a, b) for computation::skew(i, j, a, b) after which the outer
+      * loop is parallel (first vector, at most one), the inner loop is parallel (second: the \p nb_parallel smallest
+      * with b > 0, then with b < 0), or some dependence stays inside one iteration of the outer loop (third: one
+      * with b > 0, one with b < 0; the inner loop may then have to be reversed).  Empty vectors when there is no
+      * dependence at these loops or no skewing with coefficients up to 8 does it. */
+    std::tuple<std::vector<std::pair<int, int>>, std::vector<std::pair<int, int>>, std::vector<std::pair<int, int>>>
+    skewing_local_solver(std::vector<computation *> fused_computations, var outer_variable, var inner_variable, int nb_parallel);
+    /** The same with all four coefficients (alpha, beta, gamma, sigma) of computation::skew, chosen so that every
+      * distance has non-negative components afterwards (both loops can then be tiled); the third vector holds
+      * the skewing of the inner loop alone, (1, 0, gamma, 1). */
+    std::tuple<std::vector<std::tuple<int, int, int, int>>, std::vector<std::tuple<int, int, int, int>>, std::vector<std::tuple<int, int, int, int>>>
+    skewing_local_solver_positive(std::vector<computation *> fused_computations, var outer_variable, var inner_variable, int nb_parallel);
     /** Every dependence as { source instance -> sink instance }. */
     isl_union_map *get_statement_dependences() const;
     void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,

@@ -107,6 +107,7 @@ isl_bool isl_set_is_subset(isl_set *a, isl_set *b);
 isl_space *isl_set_get_space(isl_set *set);
 isl_set *isl_set_project_out(isl_set *set, enum isl_dim_type type, unsigned first, unsigned n);
 isl_set *isl_set_params(isl_set *set);
+isl_ctx *isl_set_get_ctx(isl_set *set);
 isl_val *isl_set_dim_max_val(isl_set *set, int pos);
 isl_val *isl_set_dim_min_val(isl_set *set, int pos);
 isl_set *isl_set_align_params(isl_set *set, isl_space *model);

@@ -39,6 +39,60 @@ static void wavefront()
     say("wavefront.skewed.inner_vectorizable", loop_vectorization_is_legal(j1, {&S}));
 }
 
+// skewings found from the distances: (1,0),(0,1) need a > 0 and b > 0 to be carried by the outer loop; a diagonal
+// recurrence with distance (1,1) only leaves the outer loop free after i - j
+static void list(const std::string &what, const std::vector<std::pair<int, int>> &v)
+{
+    report << what << "=" << v.size();
+    for (auto &p : v) report << " (" << p.first << "," << p.second << ")";
+    report << "\n";
+}
+
+static void skewing()
+{
+    {
+        tiramisu::init("skewing_wavefront");
+        var i("i", 1, 40), j("j", 1, 30);
+        input A("A", {var("y", 0, 40), var("x", 0, 30)}, p_float32);
+        computation S("S", {i, j}, A(i - 1, j) + A(i, j - 1));
+        S.store_in(A.get_buffer());
+        perform_full_dependency_analysis();
+        auto found = global::get_implicit_function()->skewing_local_solver({&S}, i, j, 2);
+        list("skewing.wavefront.outer_parallel", std::get<0>(found));
+        list("skewing.wavefront.inner_parallel", std::get<1>(found));
+        list("skewing.wavefront.locality", std::get<2>(found));
+        auto positive = global::get_implicit_function()->skewing_local_solver_positive({&S}, i, j, 1);
+        report << "skewing.wavefront.positive.inner_parallel=" << std::get<1>(positive).size();
+        for (auto &t : std::get<1>(positive)) report << " (" << std::get<0>(t) << "," << std::get<1>(t) << "," << std::get<2>(t) << "," << std::get<3>(t) << ")";
+        report << "\n";
+    }
+    {
+        tiramisu::init("skewing_diagonal");
+        var i("i", 1, 40), j("j", 1, 30), i1("i1"), j1("j1");
+        input A("A", {var("y", 0, 40), var("x", 0, 30)}, p_float32);
+        computation S("S", {i, j}, A(i - 1, j - 1) * 2.0f);
+        S.store_in(A.get_buffer());
+        perform_full_dependency_analysis();
+        auto found = global::get_implicit_function()->skewing_local_solver({&S}, i, j, 1);
+        list("skewing.diagonal.outer_parallel", std::get<0>(found));
+        if (!std::get<0>(found).empty()) {
+            S.skew(i, j, std::get<0>(found)[0].first, std::get<0>(found)[0].second, i1, j1);
+            prepare_schedules_for_legality_checks();
+            say("skewing.diagonal.skewed.legal", check_legality_of_function());
+            say("skewing.diagonal.skewed.outer_parallel", loop_parallelization_is_legal(i1, {&S}));
+        }
+    }
+    {
+        tiramisu::init("skewing_nothing_to_do");
+        var i("i", 1, 40), j("j", 1, 30);
+        input A("A", {var("y", 0, 41), var("x", 0, 31)}, p_float32);
+        computation B("B", {i, j}, A(i - 1, j) + A(i + 1, j + 1));
+        perform_full_dependency_analysis();
+        auto found = global::get_implicit_function()->skewing_local_solver({&B}, i, j, 2);
+        report << "skewing.out_of_place.total=" << std::get<0>(found).size() + std::get<1>(found).size() + std::get<2>(found).size() << "\n";
+    }
+}
+
 // the same recurrence with the inner loop run backwards: (0,1) becomes (0,-1)
 static void reversed()
 {
@@ -152,6 +206,7 @@ int main(int argc, char **argv)
     reversed();
     out_of_place();
     fusion();
+    skewing();
     mapped_loops();
     report.close();
     return 0;

@@ -180,10 +180,9 @@ def build_lstm_naive():
 # The reference's own test-suite (tests/test_N.cpp + wrapper_test_N.cpp, both unchanged) through this
 # front-end and the oracle's CPU emitter (GPU tests among them with TIRAMISU_FORCE_ARCH=cpu): each wrapper
 # fills its inputs, calls the generated function and compares with the expectation its authors wrote.
-# Listed: the tests that pass; 179-191 are the tests of the dependence analysis, the legality checks and the shifts
-# that repair a fusion (the generator itself asserts what each check must answer, so building them runs the
-# checks; the wrappers of SUITE_SILENT print nothing).  Not listed, by cause: the skewing solver of the
-# auto-scheduler (192-195, 198, 199),
+# Listed: the tests that pass; 179-195, 198, 199 are the tests of the dependence analysis, the legality checks, the
+# shifts that repair a fusion and the skewing solvers (the generator itself asserts what each check must answer,
+# so building them runs the checks; the wrappers of SUITE_SILENT print nothing).  Not listed, by cause:
 # distributed tags, Halide image I/O (not provided by this front-end; test 14, compute_at on a loaded image, among
 # them); 27, 130 (compute_bounds: the wrapper hands a 1-element buffer to a 10x10 program), 82, 83, 90 (store_at /
 # compute_at programs that the reference's own test list leaves out as well: 83 expects values where its
@@ -194,7 +193,7 @@ def build_lstm_naive():
 SUITE = """01 02 03 04 06 07 08 09 10 11 12 13 16 17 18 19 20 22 23 24 25 26 29 30 31 32 33 34 35 36 37 38 39 40 41 42 43 44 45 46 47 48 51 52 53 54 55 56 57 58 59 60 61 62 63 64
 65 66 67 68 69 70 71 72 73 74 75 76 77 78 80 81 84 86 87 88 89 91 97 103 104 105 106 107 108 109 110 111 112 113 114 115 116 117 118 119 120 121 122 123
 124 125 126 127 128 129 131 141 142 143 144 145 146 147 148 149 150 151 152 153 154 155 156 157 158 159 161 163 167 168 169 170 171 175
-176 177 178 179 180 181 182 183 184 185 186 187 188 189 190 191 197""".split()
+176 177 178 179 180 181 182 183 184 185 186 187 188 189 190 191 192 193 194 195 197 198 199""".split()
 
 # wrappers that call the generated function and print nothing: the test is the generator's own assertions
 SUITE_SILENT = ["183", "184", "191"]

@@ -3,7 +3,7 @@ reference's core.h:139-181 and :1236-1330).  tests/programs/dependence_checks.cp
 answers can be read off the code -- a wavefront recurrence in place with distances (1,0) and (0,1), the same with
 the inner loop reversed, an out-of-place stencil, a producer and a consumer fused into one loop -- and about loops
 mapped to GPU threads; its answers are compared here.  The reference's own tests of these calls (tests/test_179 -
-test_191) run in test_reference_suite.py."""
+test_195, test_198, test_199) run in test_reference_suite.py."""
 import os
 import subprocess
 
@@ -52,6 +52,16 @@ def answer(text, what):
     ("fusion.shifts", "1 i:2"),
     ("fusion.shifted.legal", "yes"),
     ("mapped.scale.findings", "0"),
+    # skewings from the distances.  (1,0),(0,1): the outer loop carries both when a > 0 and b > 0; no skewing
+    # leaves the outer loop free, none keeps a dependence inside it.  (1,1) alone: i - j is constant along it
+    ("skewing.wavefront.outer_parallel", "0"),
+    ("skewing.wavefront.inner_parallel", "2 (1,1) (1,2)"),
+    ("skewing.wavefront.locality", "0"),
+    ("skewing.wavefront.positive.inner_parallel", "1 (1,1,0,1)"),
+    ("skewing.diagonal.outer_parallel", "1 (1,-1)"),
+    ("skewing.diagonal.skewed.legal", "yes"),
+    ("skewing.diagonal.skewed.outer_parallel", "yes"),
+    ("skewing.out_of_place.total", "0"),
 ])
 def test_answer(answers, what, expected):
     assert answer(answers, what) == expected

@@ -972,15 +972,16 @@ void computation::skew(int i, int j, int alpha, int beta, int gamma, int sigma) 
     out[dynamic_pos(j)] = std::to_string(gamma) + "*" + vi + " + " + std::to_string(sigma) + "*" + vj;
     apply_on_range("{ [" + join(in, ",") + "] -> [" + join(out, ",") + "] }");
 }
-void computation::skew(int i, int j, int a, int b) {
+bool skewing_second_row(int &a, int &b, int &gamma, int &sigma) {
     // the second row of the unimodular matrix, chosen as the reference chooses it (tiramisu_core.cpp:4445-4497)
-    if (b == 0 || a < 0) ERROR("skew: needs a >= 0 and b != 0", true);
+    if (b == 0 || a < 0) return false;
     int n1 = std::abs(a), n2 = std::abs(b);
     if (n1 == 0) n1 = n2;
     while (n1 != n2) { if (n1 > n2) n1 -= n2; else n2 -= n1; }
     a /= n1;
     b /= n1;
-    int gamma = 0, sigma = 1;
+    gamma = 0;
+    sigma = 1;
     if (b == 1 || a == 1) gamma = a - 1;
     else if (b == -1 && a > 1) { gamma = 1; sigma = 0; }
     else {
@@ -989,9 +990,16 @@ void computation::skew(int i, int j, int a, int b) {
             if ((sigma * a) % std::abs(b) == 1) found = true;
             else sigma++;
         }
-        if (!found) ERROR("skew: no integer solution of a * sigma - b * gamma = 1", true);
+        if (!found) return false;
         gamma = (sigma * a - 1) / b;
     }
+    return true;
+}
+
+void computation::skew(int i, int j, int a, int b) {
+    int gamma, sigma;
+    if (b == 0 || a < 0) ERROR("skew: needs a >= 0 and b != 0", true);
+    if (!skewing_second_row(a, b, gamma, sigma)) ERROR("skew: no integer solution of a * sigma - b * gamma = 1", true);
     skew(i, j, a, b, gamma, sigma);
 }
 void computation::skew(var i, var j, int a, int b, var ni, var nj) {

@@ -403,6 +403,142 @@ std::vector<std::tuple<var, int>> function::correcting_loop_fusion_with_shifting
     return result;
 }
 
+// ------------------------------------------------------------------ skewing two loops
+
+namespace {
+
+// the distances { [di, dj] } of the dependences at two loop levels, between instances inside one iteration of the
+// loops around them, without (0, 0); null when there is none
+isl_set *distances_at(function *f, const std::vector<computation *> &fused, int outer, int inner) {
+    isl_union_map *s = schedules_of(f->get_isl_ctx(), fused);
+    isl_map *t = in_time(f->get_statement_dependences(), isl_union_map_copy(s), s);
+    if (!t) return nullptr;
+    for (int d = 0; d < outer; d++) t = isl_map_equate(t, isl_dim_in, d, isl_dim_out, d);
+    isl_set *delta = isl_map_deltas(t);
+    const int n = (int)isl_set_dim(delta, isl_dim_set);
+    delta = isl_set_project_out(delta, isl_dim_set, inner + 1, n - inner - 1);
+    delta = isl_set_project_out(delta, isl_dim_set, outer + 1, inner - outer - 1);
+    delta = isl_set_project_out(delta, isl_dim_set, 0, outer);
+    delta = isl_set_project_out(delta, isl_dim_param, 0, isl_set_dim(delta, isl_dim_param));
+    delta = isl_set_subtract(delta, isl_set_read_from_str(f->get_isl_ctx(), "{ [0, 0] }"));
+    if (isl_set_is_empty(delta) == isl_bool_true) {
+        isl_set_free(delta);
+        return nullptr;
+    }
+    return delta;
+}
+
+// no distance satisfies the condition (text over di, dj)
+bool none(isl_set *delta, const std::string &condition) {
+    isl_set *c = isl_set_read_from_str(isl_set_get_ctx(delta), ("{ [di, dj] : " + condition + " }").c_str());
+    c = isl_set_intersect(c, isl_set_copy(delta));
+    const bool yes = isl_set_is_empty(c) == isl_bool_true;
+    isl_set_free(c);
+    return yes;
+}
+
+std::string row(int a, int b) { return std::to_string(a) + "*di " + (b < 0 ? "- " : "+ ") + std::to_string(std::abs(b)) + "*dj"; }
+
+int common_divisor(int a, int b) {
+    a = std::abs(a);
+    b = std::abs(b);
+    while (b) { const int r = a % b; a = b; b = r; }
+    return a;
+}
+
+const int LARGEST_COEFFICIENT = 8;
+
+// (a, b), a >= 1, b of the sign given, smallest first
+std::vector<std::pair<int, int>> candidates(int sign) {
+    std::vector<std::pair<int, int>> v;
+    for (int a = 1; a <= LARGEST_COEFFICIENT; a++)
+        for (int b = 1; b <= LARGEST_COEFFICIENT; b++)
+            if (common_divisor(a, b) == 1) v.push_back({a, sign * b});
+    return v;
+}
+
+}  // namespace
+
+std::tuple<std::vector<std::pair<int, int>>, std::vector<std::pair<int, int>>, std::vector<std::pair<int, int>>>
+function::skewing_local_solver(std::vector<computation *> fused_computations, var outer_variable, var inner_variable, int nb_parallel) {
+    std::vector<std::pair<int, int>> outermost, innermost, locality;
+    if (fused_computations.empty()) ERROR("skewing_local_solver: no computation given", true);
+    computation *c = fused_computations[0];
+    const int outer = c->dynamic_pos(c->get_loop_level_number_from_dimension_name(outer_variable.get_name()));
+    const int inner = c->dynamic_pos(c->get_loop_level_number_from_dimension_name(inner_variable.get_name()));
+    align_schedules();
+    isl_set *delta = distances_at(this, fused_computations, outer, inner);
+    if (!delta) return std::make_tuple(outermost, innermost, locality);
+    for (int sign : {1, -1}) {
+        int found = 0;
+        bool local = false;
+        for (auto &ab : candidates(sign)) {
+            const std::string across = row(ab.first, ab.second);
+            if (!none(delta, across + " < 0")) continue;                 // some dependence would run backwards in the outer loop
+            const bool strongly = none(delta, across + " = 0"), all_inside = none(delta, across + " > 0");
+            if (strongly && found < nb_parallel) {                       // the outer loop carries everything: the inner one is free
+                innermost.push_back(ab);
+                found++;
+            }
+            int a = ab.first, b = ab.second, gamma, sigma;
+            if (all_inside && outermost.empty() && skewing_second_row(a, b, gamma, sigma) && none(delta, row(gamma, sigma) + " <= 0"))
+                outermost.push_back(ab);                                  // nothing crosses iterations of the outer loop
+            if (!strongly && !all_inside && !local) {
+                locality.push_back(ab);
+                local = true;
+            }
+        }
+    }
+    isl_set_free(delta);
+    return std::make_tuple(outermost, innermost, locality);
+}
+
+std::tuple<std::vector<std::tuple<int, int, int, int>>, std::vector<std::tuple<int, int, int, int>>, std::vector<std::tuple<int, int, int, int>>>
+function::skewing_local_solver_positive(std::vector<computation *> fused_computations, var outer_variable, var inner_variable, int nb_parallel) {
+    std::vector<std::tuple<int, int, int, int>> outermost, innermost, identity;
+    if (fused_computations.empty()) ERROR("skewing_local_solver_positive: no computation given", true);
+    computation *c = fused_computations[0];
+    const int outer = c->dynamic_pos(c->get_loop_level_number_from_dimension_name(outer_variable.get_name()));
+    const int inner = c->dynamic_pos(c->get_loop_level_number_from_dimension_name(inner_variable.get_name()));
+    align_schedules();
+    isl_set *delta = distances_at(this, fused_computations, outer, inner);
+    if (!delta) return std::make_tuple(outermost, innermost, identity);
+    // a second row of determinant 1 under which no distance turns negative (strictly positive where asked)
+    auto second_row = [&](int a, int b, bool strictly, int &gamma, int &sigma) {
+        for (int size = 0; size <= 2 * LARGEST_COEFFICIENT; size++)
+            for (int g = -size; g <= size; g++)
+                for (int sg : {size - std::abs(g), -(size - std::abs(g))}) {
+                    if (a * sg - b * g != 1 || !none(delta, row(g, sg) + (strictly ? " <= 0" : " < 0"))) continue;
+                    gamma = g;
+                    sigma = sg;
+                    return true;
+                }
+        return false;
+    };
+    for (int sign : {1, -1}) {
+        int found = 0;
+        for (auto &ab : candidates(sign)) {
+            const std::string across = row(ab.first, ab.second);
+            if (!none(delta, across + " < 0")) continue;
+            int gamma, sigma;
+            if (none(delta, across + " = 0") && found < nb_parallel && second_row(ab.first, ab.second, false, gamma, sigma)) {
+                innermost.push_back(std::make_tuple(ab.first, ab.second, gamma, sigma));
+                found++;
+            }
+            if (none(delta, across + " > 0") && outermost.empty() && second_row(ab.first, ab.second, true, gamma, sigma))
+                outermost.push_back(std::make_tuple(ab.first, ab.second, gamma, sigma));
+        }
+    }
+    if (none(delta, "di < 0"))
+        for (int gamma = 0; gamma <= LARGEST_COEFFICIENT; gamma++)
+            if (none(delta, row(gamma, 1) + " < 0")) {
+                identity.push_back(std::make_tuple(1, 0, gamma, 1));
+                break;
+            }
+    isl_set_free(delta);
+    return std::make_tuple(outermost, innermost, identity);
+}
+
 // ------------------------------------------------------------------ the implicit function
 
 void perform_full_dependency_analysis() { global::get_implicit_function()->perform_full_dependency_analysis(); }

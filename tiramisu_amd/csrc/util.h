@@ -25,6 +25,10 @@ class expr;
 /** isl syntax for an integer (quasi-)affine expression; sets \p ok to false otherwise. */
 std::string expr_to_isl_str(const expr &e, bool &ok);
 
+/** skew(i, j, a, b): divides a and b by their common divisor and completes (a, b) to a matrix of determinant 1
+  * with the second row (gamma, sigma) that computation::skew uses; false when a < 0, b == 0 or none is found. */
+bool skewing_second_row(int &a, int &b, int &gamma, int &sigma);
+
 class computation;
 /** { consumer[iterators] -> producer[indices] } for every read of \p producer in the consumer's expression and
   * predicate, over the consumer's iteration domain (and, on request, inside the producer's); null if none. */
