@@ -93,6 +93,23 @@ static void skewing()
     }
 }
 
+// the schedule of the reference's tests/test_133.cpp (134-140 vary it): the recurrence above, skew(i, j, 1) -- which
+// keeps i outermost, (1,0),(0,1) -> (1,1),(0,1) -- and the outer loop tagged parallel although it carries (1,1)
+static void skewed_outer_loop_tagged_parallel()
+{
+    tiramisu::init("skewed_outer_parallel");
+    var i("i", 1, 40), j("j", 1, 40), ni("ni"), nj("nj");
+    input A("A", {var("y", 0, 40), var("x", 0, 40)}, p_uint8);
+    computation S("S", {i, j}, A(i - 1, j) + A(i, j - 1));
+    S.store_in(A.get_buffer());
+    perform_full_dependency_analysis();
+    S.skew(i, j, 1, ni, nj);
+    prepare_schedules_for_legality_checks();
+    say("test_133.order_legal", check_legality_of_function());
+    say("test_133.ni_parallel", loop_parallelization_is_legal(ni, {&S}));
+    say("test_133.nj_parallel", loop_parallelization_is_legal(nj, {&S}));
+}
+
 // the same recurrence with the inner loop run backwards: (0,1) becomes (0,-1)
 static void reversed()
 {
@@ -206,6 +223,7 @@ int main(int argc, char **argv)
     reversed();
     out_of_place();
     fusion();
+    skewed_outer_loop_tagged_parallel();
     skewing();
     mapped_loops();
     report.close();

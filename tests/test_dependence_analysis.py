@@ -52,6 +52,10 @@ def answer(text, what):
     ("fusion.shifts", "1 i:2"),
     ("fusion.shifted.legal", "yes"),
     ("mapped.scale.findings", "0"),
+    # the schedule of the reference's tests 133-140: sequentially fine, but the loop they tag parallel carries (1,1)
+    ("test_133.order_legal", "yes"),
+    ("test_133.ni_parallel", "no"),
+    ("test_133.nj_parallel", "no"),
     # skewings from the distances.  (1,0),(0,1): the outer loop carries both when a > 0 and b > 0; no skewing
     # leaves the outer loop free, none keeps a dependence inside it.  (1,1) alone: i - j is constant along it
     ("skewing.wavefront.outer_parallel", "0"),
