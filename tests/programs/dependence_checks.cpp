@@ -203,6 +203,19 @@ static void mapped_loops()
     f->gen_ordering_schedules();
     for (auto &line : f->gpu_mapped_loops_that_carry_dependences()) report << "mapped.row_sums: " << line << "\n";
 
+    // a permutation in place through an index table: the element an iteration reads may be one that another writes
+    tiramisu::init("gather_in_place");
+    var k("k", 0, 64), k0("k0"), k1("k1");
+    input T("T", {k}, p_int32);
+    input V("V", {k}, p_float32);
+    computation G("G", {k}, V(T(k)) + 1.0f);
+    G.store_in(V.get_buffer());
+    G.split(k, 16, k0, k1);
+    G.tag_gpu_level(k0, k1);
+    f = global::get_implicit_function();
+    f->gen_ordering_schedules();
+    for (auto &line : f->gpu_mapped_loops_that_carry_dependences()) report << "mapped.gather: " << line << "\n";
+
     tiramisu::init("scale_mapped");
     input C("C", {i, j}, p_float32);
     computation D("D", {i, j}, C(i, j) * 3.0f);

@@ -89,6 +89,9 @@ def test_loops_mapped_to_threads(answers):
     wavefront reduction); independent points are not reported."""
     assert "mapped.scan_rows: S: loop j (level 1, mapped to threadIdx) carries a dependence through global memory" in answers
     assert "mapped.row_sums: s: loop j (level 1, mapped to threadIdx) carries a reduction through global memory" in answers
+    # an index read from a table may name any element: both loops of the permutation in place are refused
+    assert "mapped.gather: G: loop k0 (level 0, mapped to blockIdx) carries a dependence" in answers
+    assert "mapped.gather: G: loop k1 (level 1, mapped to threadIdx) carries a dependence" in answers
     assert "mapped.scan_rows: S: loop i" not in answers and "mapped.row_sums: s: loop i" not in answers
 
 

@@ -1660,17 +1660,25 @@ computation *computation::select(int duplicate_id) {
 }
 
 // { consumer[iterators] -> producer[indices] } for every read of `producer` in the consumer's expression and predicate
-isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain) {
+isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain, bool any_where_not_affine) {
     function *f = consumer.get_function();
     const std::string wanted = producer.get_first_definition()->get_name();
     std::vector<std::string> pieces;
     bool ok = true;
+    int free_dimensions = 0;
     auto collect = [&](const expr &e) {
         if (!e.is_defined()) return;
         e.visit([&](const expr &x) {
             if (x.get_expr_type() != e_op || x.get_op_type() != o_access || x.get_name() != wanted) return;
             std::vector<std::string> idx;
-            for (auto &i : x.get_access()) idx.push_back(expr_to_isl_str(i, ok));
+            for (auto &i : x.get_access()) {
+                bool affine = true;
+                std::string text = expr_to_isl_str(i, affine);
+                // an index looked up in a table (or otherwise not affine) may be anything: a free dimension
+                if (!affine && any_where_not_affine) text = "_any" + std::to_string(free_dimensions++);
+                else ok = ok && affine;
+                idx.push_back(text);
+            }
             pieces.push_back(consumer.get_name() + "[" + join(consumer.get_iteration_domain_dimension_names(), ",") + "] -> " + producer.get_name() + "[" + join(idx, ",") + "]");
         });
     };

@@ -104,7 +104,7 @@ void function::calculate_dep_flow(bool global_memory_only) {
         // what c reads of p, carried on to the cells p is stored in (an input writes nothing here but is read from its buffer)
         for (auto p : body) {
             if (!counted(p)) continue;
-            isl_map *r = reads_of(*c, *p, false);
+            isl_map *r = reads_of(*c, *p, false, true);
             if (r) unite(reads, isl_map_apply_range(r, isl_map_copy(p->get_access_relation())));
         }
     }

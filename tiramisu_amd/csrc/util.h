@@ -31,8 +31,10 @@ bool skewing_second_row(int &a, int &b, int &gamma, int &sigma);
 
 class computation;
 /** { consumer[iterators] -> producer[indices] } for every read of \p producer in the consumer's expression and
-  * predicate, over the consumer's iteration domain (and, on request, inside the producer's); null if none. */
-struct isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain = true);
+  * predicate, over the consumer's iteration domain (and, on request, inside the producer's); null if none.  An index
+  * that is not affine is an error, or -- with \p any_where_not_affine -- a dimension left free (the read may be of any element). */
+struct isl_map *reads_of(computation &consumer, computation &producer, bool within_producer_domain = true,
+                         bool any_where_not_affine = false);
 
 }  // namespace tiramisu
 #endif
