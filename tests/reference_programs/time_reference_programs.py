@@ -2,7 +2,7 @@
 (build_reference_programs.py) on the GPU of this machine, at the sizes their own wrappers use:
 the eight image pipelines of benchmarks/halide on a 2112 x 3520 image (the size of the tree's
 utils/images; heat2dgpu on its wrapper's 10000 x 10000 grid, edgegpu on the 8192 x 8192 x 3 it is
-written for), the three tuned sgemm schedules and chain_mm.  The programs copy to and from the GPU
+written for), the three tuned sgemm schedules, chain_mm and the three baryon correlators (through their own wrappers).  The programs copy to and from the GPU
 themselves; what is timed is their kernels: HIP events around every launch of a call
 (tiramisu_hip_profile_*), median over the calls.  Bytes are the algorithmic ones: every input and
 output element once.  Prints one markdown table.  Run from the repository root on a machine with a
@@ -115,6 +115,39 @@ def gemm_programs(only):
     return out
 
 
+BARYON = ["gpu_tiramisu_make_fused_baryon_blocks_correlator", "gpu_tiramisu_make_fused_identical_baryon_blocks_correlator",
+          "gpu_single_tiramisu_make_fused_identical_baryon_blocks_correlator"]
+
+
+def correlator_programs(only):
+    """The baryon correlator benchmarks, run by their own wrappers (which also run the reference's C++ restatement
+    and compare): the kernels of the generated function, at the lattice size the reference's parameter header sets."""
+    out = []
+    for name in BARYON:
+        if only and name not in only:
+            continue
+        lib = ctypes.CDLL(library(name))
+        lib.tiramisu_wrapper_main.restype = ctypes.c_int
+        lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
+
+        def call():
+            # the wrapper prints every correlator entry: keep that out of the table
+            sys.stdout.flush()
+            saved, null = os.dup(1), os.open(os.devnull, os.O_WRONLY)
+            os.dup2(null, 1)
+            try:
+                status = lib.tiramisu_wrapper_main(0, None)
+            finally:
+                os.dup2(saved, 1)
+                os.close(saved)
+                os.close(null)
+            assert status == 0
+        call()
+        total, by = kernel_times(call)
+        out.append((name, total, by))
+    return out
+
+
 def main():
     only = set(sys.argv[1:])
     runtime.wrappers()
@@ -124,6 +157,10 @@ def main():
         kernels = ", ".join("%s %.1f us%s" % (k, t / n * 1e3, " x %d" % n if n > 1 else "") for k, (t, n) in sorted(by.items()))
         gbs = nbytes / (total * 1e-3) / 1e9
         print("| `%s` | %s | %s | %.3f ms | %.0f GB/s | %.2f of 8 TB/s |" % (name, note, kernels, total, gbs, gbs / HBM_PEAK_GBS), flush=True)
+    for name, total, by in correlator_programs(only):
+        kernels = ", ".join("%s %.1f us%s" % (k, t / n * 1e3, " x %d" % n if n > 1 else "") for k, (t, n) in sorted(by.items()))
+        print("| `%s` | complex fp64 contractions, the reference's parameter set; checked by the wrapper against the reference's C++ | %s | %.3f ms | - | - |"
+              % (name, kernels, total), flush=True)
     for name, note, total, by, flop in gemm_programs(only):
         kernels = ", ".join("%s %.3f ms" % (k, t / n) for k, (t, n) in sorted(by.items()))
         tf = flop / (total * 1e-3) / 1e12
