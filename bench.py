@@ -42,26 +42,43 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 FP32_VALU_PEAK_TFLOPS = 157.3  # MI355X vector fp32 (256 CUs x 128 lanes x 2 flops x 2.4 GHz): what a kernel without MFMA is priced against
+FP32_VALU_PLAIN_TFLOPS = 39.3  # 256 CUs x 64 lanes x 2.4 GHz x 1 flop: separate adds and multiplies, one per lane and clock (no FMA:
+                               # the stencil's value must round as the un-fused program's; packed fp32 is not used on this pool)
 PROGRAMS = os.path.join(ROOT, "tiramisu_amd", "programs")
 
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_by_kernel.md")
 
 
 def traffic_table():
-    """{(function, kernel description): {"bytes": HBM bytes per launch, "vector_alu_busy": share or None}} from the
-    table of counter measurements in profiles/ (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
-    scaled by what the same counters read for a plain copy of known size)."""
+    """{(function, kernel description): {"bytes": HBM bytes per launch, "vector_alu_busy": share or None, "source": hash}}
+    from the table of counter measurements in profiles/ (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch,
+    scaled by what the same counters read for a plain copy of known size).  "source" is kernel_source_hash() of
+    the function at the time of the measurement."""
     out = {}
     if not os.path.exists(TRAFFIC_TABLE):
         return out
     for line in open(TRAFFIC_TABLE):
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
-        if len(cells) < 6 or not cells[4].replace(".", "", 1).isdigit():
+        if len(cells) < 7 or not cells[4].replace(".", "", 1).isdigit():
             continue
         busy = cells[5].rstrip("%").strip()
         out[(cells[0].strip("`"), cells[1].strip("`"))] = {
-            "bytes": float(cells[4]), "vector_alu_busy": float(busy) / 100.0 if busy.replace(".", "", 1).isdigit() else None}
+            "bytes": float(cells[4]), "vector_alu_busy": float(busy) / 100.0 if busy.replace(".", "", 1).isdigit() else None,
+            "source": cells[6].strip("`")}
     return out
+
+
+def kernel_source_hash(name):
+    """Twelve hex digits over the generated device source of a function and the kernel headers it includes: a
+    counter measurement belongs to exactly this text."""
+    import hashlib
+    import re
+    text = open(os.path.join(PROGRAMS, "build", name + ".o.hip")).read()
+    h = hashlib.sha1(re.sub(r'#include "[^"]*/kernels/', '#include "kernels/', text).encode())
+    for inc in sorted(set(re.findall(r'#include "([^"]*/kernels/[^"]+)"', text))):
+        path = os.path.join(ROOT, "tiramisu_amd", "csrc", "kernels", os.path.basename(inc))
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:12]
 
 
 def kernel_descriptions(name):
@@ -71,7 +88,12 @@ def kernel_descriptions(name):
 
 
 def kernel_traffic(name, kernel):
-    return traffic_table().get((name, kernel_descriptions(name).get(kernel, "")))
+    """The counter record of a kernel, or None when there is none for this description or the kernel's source
+    has changed since it was measured."""
+    row = traffic_table().get((name, kernel_descriptions(name).get(kernel, "")))
+    if row and row["source"] != kernel_source_hash(name):
+        return None
+    return row
 
 
 def device_array(host):
@@ -121,7 +143,9 @@ def launch_duration(prof, dominant, ms_per_call):
     """(milliseconds per launch of the dominant kernel, how it was obtained).  HIP events around every launch
     include what an event costs between two launches; the timed calls (no events inside) bound the kernel
     from above as well: the call minus the other kernels, over this kernel's launches.  The smaller of the two
-    is the one a kernel trace agrees with (a chain of dependent launches, or a kernel of a few microseconds)."""
+    is the one a kernel trace agrees with (a chain of dependent launches, or a kernel of a few microseconds);
+    the other kernels' event times carry the same overhead, so the subtraction leans low: the roofline entry
+    also carries `frac_between_events`, the fraction on the per-event duration, as the conservative figure."""
     per_event, launches = prof[dominant]
     others = sum(v[0] * v[1] for k, v in prof.items() if k != dominant)
     from_calls = (ms_per_call - others) / launches
@@ -170,6 +194,25 @@ def stencil_kernels(kernel_source, domain_cells):
     return out
 
 
+def stencil_arithmetic(kernel_source):
+    """{kernel name: (floating-point operations of the stencil expression per cell and step, cells that a launch
+    stages = computes at every one of its steps, halo and stale cells included)} from the generated kernel source:
+    the operators of ST_EXPR, and the tile geometry in the emitter's descriptions (a workgroup stages wavefronts x
+    rows x 256 cells; a boundary slice stages its rows + 2 x steps x radius)."""
+    import re
+    text = open(kernel_source).read()
+    out = {}
+    for m in re.finditer(r"// (\w+): stencil: (\d+) time step\(s\) per launch, radius (\d+), tile \d+x\d+ in registers, (\d+) wavefronts x (\d+) rows, "
+                         r"(\d+) interior tiles[^\n]*\n(?:#define [^\n]*\n)*?#define ST_EXPR ([^\n]*)", text):
+        name, steps, radius = m.group(1), int(m.group(2)), int(m.group(3))
+        staged = int(m.group(6)) * int(m.group(4)) * int(m.group(5)) * 256
+        e = re.search(r"// \w+: stencil: the (\d+) tiles of %s's launch[^\n]*in (\d+) slice\(s\) of (\d+) rows each[^\n]*carried by" % name, text)
+        if e:
+            staged += int(e.group(1)) * int(e.group(2)) * (int(e.group(3)) + 2 * steps * radius) * 256
+        out[name] = (len(re.findall(r" [-+*/] ", m.group(7))), staged)
+    return out
+
+
 def bench_heat2d(steps, warmup, with_cpu):
     from tiramisu_amd import runtime
     from oracle import build as oracle_build
@@ -198,25 +241,49 @@ def bench_heat2d(steps, warmup, with_cpu):
     # whole function: counter bytes of every launch; the fused minimum stands in for a kernel the table does not know
     call_bytes = sum((measured[k]["bytes"] if measured[k] else minimum[k]) * v[1] for k, v in prof.items())
     dom_bytes = t_dom["bytes"] if t_dom else None
-    achieved = (dom_bytes if dom_bytes else fused_min) / (dom[1][0] * 1e-3) / 1e9
+    hbm_gbs = (dom_bytes if dom_bytes else fused_min) / (dom[1][0] * 1e-3) / 1e9
+    # what the launch computes: every cell of the domain at every fused step (useful), and every cell it stages
+    # at every step (what the vector ALUs really execute: halo and stale cells included)
+    ops, staged_cells = stencil_arithmetic(os.path.join(PROGRAMS, "build", name + ".o.hip"))[dom[0]]
+    useful_tflops = cells * fused_steps * ops / (dom[1][0] * 1e-3) / 1e12
+    staged_tflops = staged_cells * fused_steps * ops / (dom[1][0] * 1e-3) / 1e12
+    dev.free()
+    rates = streaming_rates()
+    hbm = {"achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_gbs / HBM_PEAK_GBS,
+           "traffic": dom_bytes, "traffic_basis": "hardware counters of profiles/hbm_traffic_by_kernel.md (same kernel source)" if dom_bytes
+                      else "none for this kernel source: the read-once-write-once minimum stands in",
+           "fused_minimum_bytes": fused_min, "traffic_over_fused_minimum": dom_bytes / fused_min if dom_bytes else None,
+           "streaming_ceiling_gbs": rates["ceiling"], "frac_of_streaming_ceiling": hbm_gbs / rates["ceiling"],
+           "algorithmic_gbs": per_launch_alg / (dom[1][0] * 1e-3) / 1e9}
+    if fused_steps == 1:
+        roofline = dict(hbm, bound="hbm")
+        roofline["limiter"] = "hbm: %.0f GB/s against %.0f GB/s for the fastest plain pass over the same planes in this run" % (hbm_gbs, rates["ceiling"])
+    else:
+        roofline = {"bound": "valu", "achieved": useful_tflops, "peak": FP32_VALU_PLAIN_TFLOPS, "unit": "TFLOP/s",
+                    "frac": useful_tflops / FP32_VALU_PLAIN_TFLOPS, "traffic": dom_bytes,
+                    "useful_valu_frac": useful_tflops / FP32_VALU_PLAIN_TFLOPS, "staged_valu_frac": staged_tflops / FP32_VALU_PLAIN_TFLOPS,
+                    "flops_per_cell_step": ops, "staged_cells_per_launch": staged_cells,
+                    "peak_basis": "256 compute units x 64 lanes x 2.4 GHz, one add or multiply per lane and clock (no FMA: results must round as "
+                                  "the un-fused program's; no packed fp32 on this pool)",
+                    "vector_alu_busy": t_dom["vector_alu_busy"] if t_dom else None,
+                    "hbm": hbm,
+                    "limiter": "vector ALUs: a time-fused launch advances %d steps per byte it moves, so its stencil arithmetic sets its duration "
+                               "(%.2f of the plain VALU rate on the cells of the domain, %.2f with the halo and stale cells it also computes); "
+                               "its HBM traffic runs at %.0f GB/s against %.0f GB/s for the fastest plain pass over the same planes in this run "
+                               "(vendor device-to-device copy: %.0f GB/s)"
+                               % (fused_steps, useful_tflops / FP32_VALU_PLAIN_TFLOPS, staged_tflops / FP32_VALU_PLAIN_TFLOPS, hbm_gbs, rates["ceiling"], rates["vendor_d2d"])}
+    roofline.update({"kernel": dom[0], "kernel_ms": dom[1][0], "launches_per_step": dom[1][1],
+                     "time_steps_per_launch": fused_steps, "cells_per_launch": cells})
     out = {
         "value": call_bytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
         "value_basis": "HBM bytes moved per call (hardware counters per kernel x launches%s) / time per call"
-                       % ("" if all(measured.values()) else "; read-once-write-once minimum for kernels without a counter record"),
+                       % ("" if all(measured.values()) else "; read-once-write-once minimum for kernels without a counter record of their present source"),
+        "value_lower_bound_gbs": sum(minimum[k] * v[1] for k, v in prof.items()) / (ms * 1e-3) / 1e9,
+        "value_lower_bound_basis": "needs no counters: every launch reads one plane and writes each plane it leaves once",
         "algorithmic_gbs": alg_bytes / (ms * 1e-3) / 1e9,
         "algorithmic_basis": "8 bytes per cell and time step of the un-fused program (32 x 2 x 8192^2 x 4 B = 17.18 GB per call)",
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": dom_bytes,
-                     "kernel": dom[0], "kernel_ms": dom[1][0], "launches_per_step": dom[1][1],
-                     "time_steps_per_launch": fused_steps, "cells_per_launch": cells,
-                     "algorithmic_gbs": per_launch_alg / (dom[1][0] * 1e-3) / 1e9,
-                     "fused_minimum_bytes": fused_min,
-                     "traffic_over_fused_minimum": dom_bytes / fused_min if dom_bytes else None,
-                     "vector_alu_busy": t_dom["vector_alu_busy"] if t_dom else None,
-                     "limiter": "hbm" if fused_steps == 1 else
-                                "vector ALUs (time-fused launch: the stencil arithmetic of all fused steps sets its duration)" +
-                                ("; this launch also moves its bytes at the highest streaming rate measured on this GPU (5.1-5.3 TB/s)"
-                                 if achieved >= 5000.0 else "")},
+        "roofline": roofline,
+        "streaming_rates_gbs": rates,
         "kernels": {k: {"ms": v[0], "launches_per_step": v[1], "traffic": measured[k]["bytes"] if measured[k] else None} for k, v in prof.items()},
     }
     if with_cpu:
@@ -227,7 +294,6 @@ def bench_heat2d(steps, warmup, with_cpu):
                                "sample": "whole workload (8192x8192, 32 steps), median of %d runs of the CPU-generated "
                                          "code (parallelize y, vectorize x by 8; g++ -O2 -mavx, OpenMP); bytes = 8 per cell and "
                                          "time step, which is what the un-fused CPU code moves" % runs}
-    dev.free()
     return out
 
 
@@ -254,7 +320,8 @@ def bench_sgemm(M, steps, warmup, with_cpu):
         "value": flop / (ms * 1e-3) / 1e9, "unit": "GFLOP/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": (kernel_traffic(name, dom[0]) or {}).get("bytes"),
-                     "kernel": dom[0], "kernel_ms": kernel_ms, "kernel_ms_basis": basis, "kernel_ms_between_events": dom[1][0]},
+                     "kernel": dom[0], "kernel_ms": kernel_ms, "kernel_ms_basis": basis, "kernel_ms_between_events": dom[1][0],
+                     "frac_between_events": flop / (dom[1][0] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS},
     }
     if with_cpu:
         cpu = runtime.Program(oracle_build.cpu_program_library(PROGRAMS, name), name, needs_gpu_runtime=False)
@@ -268,21 +335,80 @@ def bench_sgemm(M, steps, warmup, with_cpu):
     return out
 
 
+def streaming_rates(reps=30, with_torch=False):
+    """Read-once-write-once rates on the benchmark's plane size (256 MiB read + 256 MiB written per pass, GB/s of both
+    directions together), measured here: the ceiling that the HBM-bound stencil launches are stated against.
+      vendor_d2d          hipMemcpyAsync device to device (through the runtime ABI's tiramisu_hip_memcpy_device_to_device)
+      copy_plane          the copy program on the schedule-faithful emitter (4 bytes per lane)
+      copy_plane_quads    the same program taken by the stencil emitter (16 bytes per lane, non-temporal stores)
+      torch_copy / torch_add   torch.Tensor.copy_ and an element-wise add (second opinions; only with `with_torch`)"""
+    from tiramisu_amd import runtime
+    w = runtime.wrappers()
+    n = 8192
+    nbytes = 2.0 * n * n * 4
+    a = np.ones((n, n), np.float32)
+    dS, dD = device_array(a), device_array(a)
+    out = {}
+
+    def rate(call):
+        for _ in range(reps):
+            call()
+        w.tiramisu_hip_stream_synchronize(0)
+        best = None
+        for _ in range(3):
+            with runtime.DeviceTimer() as t:
+                for _ in range(reps):
+                    call()
+            best = t.ms if best is None else min(best, t.ms)
+        return nbytes / (best / reps * 1e-3) / 1e9
+    out["vendor_d2d"] = rate(lambda: w.tiramisu_hip_memcpy_device_to_device(dD.ptr, dS.ptr, n * n * 4))
+    for prog_name in ("copy_plane", "copy_plane_quads"):
+        prog = runtime.load(PROGRAMS, prog_name)
+        args = (dS.buffer(), dD.buffer())
+        out[prog_name] = rate(lambda: prog(*args))
+    dS.free()
+    dD.free()
+    if with_torch:
+        try:
+            import torch
+            ta = torch.ones(n, n, device="cuda")
+            tb = torch.empty_like(ta)
+            for key, call in (("torch_copy", lambda: tb.copy_(ta)), ("torch_add", lambda: torch.add(ta, 1.0, out=tb))):
+                for _ in range(reps):
+                    call()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(reps):
+                    call()
+                e1.record()
+                torch.cuda.synchronize()
+                out[key] = nbytes / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9
+        except ImportError:
+            pass
+    out["ceiling"] = max(out.values())
+    out["ceiling_basis"] = "the fastest of these passes over 256 MiB in + 256 MiB out, timed in this run: " + ", ".join(k for k in out if k != "ceiling")
+    return out
+
+
 def bench_copy(steps, warmup, with_cpu):
-    """Plain 256 MiB -> 256 MiB copy (schedule-faithful kernel): counter calibration."""
+    """Streaming calibration: 256 MiB -> 256 MiB by the vendor's device-to-device copy, by torch, and by the copy
+    program on both emitters.  `value` is the copy program as the back-end compiles it when left alone."""
     from tiramisu_amd import runtime
     n = 8192
     a = np.ones((n, n), np.float32)
     dS, dD = device_array(a), device_array(a)
-    prog = runtime.load(PROGRAMS, "copy_plane")
+    prog = runtime.load(PROGRAMS, "copy_plane_quads")
     args = (dS.buffer(), dD.buffer())
     ms = time_steps(lambda: prog(*args), steps, warmup)
     nbytes = 2.0 * n * n * 4
-    out = {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
-           "roofline": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": nbytes}}
     dS.free()
     dD.free()
+    rates = streaming_rates(max(steps, 20), with_torch=True)
+    out = {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
+           "roofline": {"bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": nbytes, "kernel": "copy_plane_quads"},
+           "streaming_rates_gbs": rates}
     return out
 
 
@@ -299,12 +425,18 @@ def bench_sweep5(steps, warmup, with_cpu):
     prof = kernel_profile(lambda: prog(*args), steps)
     dom = max(prof.items(), key=lambda kv: kv[1][0] * kv[1][1])
     nbytes = 2.0 * n * n * 4
-    out = {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
-           "roofline": {"bound": "hbm", "achieved": nbytes / (dom[1][0] * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                        "frac": nbytes / (dom[1][0] * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": (kernel_traffic("sweep5_8192x8192", dom[0]) or {}).get("bytes"),
-                        "kernel": dom[0], "kernel_ms": dom[1][0]}}
     dS.free()
     dD.free()
+    rates = streaming_rates()
+    achieved = nbytes / (dom[1][0] * 1e-3) / 1e9
+    out = {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": ms, "warmup_extra_steps": EXTRA_WARMUP.get("last", 0),
+           "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                        "frac": achieved / HBM_PEAK_GBS, "traffic": (kernel_traffic("sweep5_8192x8192", dom[0]) or {}).get("bytes"),
+                        "kernel": dom[0], "kernel_ms": dom[1][0],
+                        "streaming_ceiling_gbs": rates["ceiling"], "frac_of_streaming_ceiling": achieved / rates["ceiling"],
+                        "limiter": "hbm: %.0f GB/s against %.0f GB/s for the fastest plain pass over the same planes in this run (vendor "
+                                   "device-to-device copy %.0f GB/s)" % (achieved, rates["ceiling"], rates["vendor_d2d"])},
+           "streaming_rates_gbs": rates}
     return out
 
 
@@ -331,6 +463,7 @@ def _generic_bench(name, host_arrays, flop, peak_tflops, steps, warmup, with_cpu
            "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak_tflops, "unit": "TFLOP/s",
                         "frac": achieved / peak_tflops, "traffic": (kernel_traffic(name, dom[0]) or {}).get("bytes"),
                         "kernel": dom[0], "kernel_ms": kernel_ms, "kernel_ms_basis": basis, "kernel_ms_between_events": dom[1][0],
+                        "frac_between_events": dom_flop / (dom[1][0] * 1e-3) / 1e12 / peak_tflops,
                         "launches_per_step": dom[1][1]},
            "kernels": {k: {"ms": v[0], "launches_per_step": v[1]} for k, v in prof.items()}}
     if with_cpu:
@@ -378,8 +511,8 @@ def bench_lstm(steps, warmup, with_cpu):
     x = rng.uniform(-1, 1, (S, B, H)).astype(np.float32)
     y = np.zeros((S, B, H), np.float32)
     flop = L * S * 2 * (2.0 * B * 4 * H * H)
-    return _generic_bench("lstm_4x64x512x100", [w, b, x, y], flop, FP32_MFMA_PEAK_TFLOPS, max(2, steps // 4), max(1, warmup // 2),
-                          with_cpu, "unscheduled program, batch loop parallelized")   # one kernel does all the flops: the fused cell
+    return _generic_bench("lstm_4x64x512x100", [w, b, x, y], flop, FP32_MFMA_PEAK_TFLOPS, steps, warmup,
+                          with_cpu, "naive ordered nest, no tiling, parallelize(k): the reference's cpu/generator.cpp order")   # one kernel does all the flops: the fused cell
 
 
 def bench_sgemm_cache_shared(steps, warmup, with_cpu):
@@ -445,7 +578,7 @@ def main():
                                 "lstm": "4-layer LSTM B64 H512 S100 (benchmark configs[4])"}.get(head_name, head_name)},
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
-        **{k: head[k] for k in ("value_basis", "algorithmic_gbs", "algorithmic_basis") if k in head},
+        **{k: head[k] for k in ("value_basis", "value_lower_bound_gbs", "value_lower_bound_basis", "algorithmic_gbs", "algorithmic_basis", "streaming_rates_gbs") if k in head},
         "workloads": {k: v for k, v in results.items() if k != head_name},
     }
     print(json.dumps(line))

@@ -7,6 +7,7 @@
 #define TIRAMISU_AMD_CORE_H
 #include <cassert>
 #include <cmath>
+#include <array>
 #include <map>
 #include <memory>
 #include <set>
@@ -48,6 +49,13 @@ void codegen(const std::vector<buffer *> &arguments, const std::string obj_filen
              const bool gen_gpu = false);
 void codegen(const std::vector<buffer *> &arguments, const std::string obj_filename,
              const hardware_architecture_t gen_architecture_flag);
+
+/** function::set_backend_option on the implicit function. */
+void set_backend_option(const std::string &name, const std::string &value);
+void set_backend_option(const std::string &name, long value);
+/** The option of the function whose code is being generated (of the implicit function outside code
+  * generation); plain getenv when there is no function at all.  For the back-end's own sources. */
+const char *backend_option(const char *env_name);
 
 /** The same calls on the implicit function (reference: core.h:139-181). */
 void perform_full_dependency_analysis();
@@ -103,6 +111,9 @@ public:
     std::unordered_map<computation *, std::unordered_map<computation *, int>> sched_graph_reversed;
     std::set<computation *> starting_computations;
     bool use_low_level_scheduling_commands = false;
+
+    std::map<std::string, std::string> backend_options;                          // set_backend_option
+    mutable std::vector<std::array<std::string, 3>> consulted_options;          // backend_option
 
     explicit function(std::string name);
     ~function();
@@ -256,6 +267,25 @@ public:
     std::string generate_new_name(const std::string &prefix);
     const std::vector<std::string> &get_codegen_log() const { return codegen_log; }
     void log(const std::string &s) { codegen_log.push_back(s); }
+
+    // ---- options of the code-generation back-end (no counterpart in the reference, whose CUDA back-end has none)
+    /** Sets an option of the back-end for this function: tile shapes, steps fused per stencil launch, which
+      * emitters may take a nest, and so on.  An option is named after its environment variable without the
+      * TIRAMISU_ prefix, in lower case: "stencil_rows", "mfma_tile", "no_single_step_stencil"; switches take
+      * "1".  The environment variable, when set, overrides the program's value (so a run can still be
+      * steered from outside); the manifest written beside the object lists every option that code generation
+      * found set, with its value and where it came from.  An empty value removes the option. */
+    void set_backend_option(const std::string &name, const std::string &value);
+    void set_backend_option(const std::string &name, long value) { set_backend_option(name, std::to_string(value)); }
+    void clear_backend_options() { backend_options.clear(); }
+    const std::map<std::string, std::string> &get_backend_options() const { return backend_options; }
+    /** The value of the option whose environment variable is \p env_name ("TIRAMISU_STENCIL_ROWS"): the
+      * environment's, else the program's, else null.  Remembers what it found for the manifest. */
+    const char *backend_option(const char *env_name) const;
+    /** (option, value, "environment" | "program") of every option looked up and found set since the last
+      * clear_consulted_backend_options(). */
+    const std::vector<std::array<std::string, 3>> &consulted_backend_options() const { return consulted_options; }
+    void clear_consulted_backend_options() const { consulted_options.clear(); }
 
     /** True when GPU-mapped loops are generated without gen_cuda_stmt() -- the route that, in the
       * reference, hands the loops to Halide's own GPU target, which moves buffers between host and

@@ -81,6 +81,58 @@ void codegen(const std::vector<buffer *> &arguments, const std::string obj_filen
     global::get_implicit_function()->codegen(arguments, obj_filename, arch);
 }
 
+// ---- options of the back-end.  While a function's code is generated it is the scope of every lookup.
+static const function *option_scope = nullptr;
+namespace {
+struct option_scope_guard {
+    const function *saved;
+    explicit option_scope_guard(const function *f) : saved(option_scope) { option_scope = f; }
+    ~option_scope_guard() { option_scope = saved; }
+};
+std::string option_name_of(const char *env_name) {
+    std::string n = env_name;
+    if (n.rfind("TIRAMISU_", 0) == 0) n = n.substr(9);
+    for (char &c : n) c = (char)std::tolower((unsigned char)c);
+    return n;
+}
+}  // namespace
+
+void function::set_backend_option(const std::string &name_in, const std::string &value) {
+    std::string n = name_in;
+    for (char &c : n) c = (char)std::tolower((unsigned char)c);
+    if (n.rfind("tiramisu_", 0) == 0) n = n.substr(9);
+    if (n.empty()) ERROR("set_backend_option: empty option name", true);
+    if (value.empty()) backend_options.erase(n);
+    else backend_options[n] = value;
+}
+
+const char *function::backend_option(const char *env_name) const {
+    const std::string n = option_name_of(env_name);
+    const char *v = std::getenv(env_name);
+    const char *from = "environment";
+    if (!v) {
+        auto it = backend_options.find(n);
+        if (it == backend_options.end()) return nullptr;
+        v = it->second.c_str();
+        from = "program";
+    }
+    for (auto &c : consulted_options)
+        if (c[0] == n) return v;
+    consulted_options.push_back({n, v, from});
+    return v;
+}
+
+void set_backend_option(const std::string &name, const std::string &value) {
+    if (!global::get_implicit_function()) ERROR("declare a function (tiramisu::init) before setting back-end options", true);
+    global::get_implicit_function()->set_backend_option(name, value);
+}
+void set_backend_option(const std::string &name, long value) { set_backend_option(name, std::to_string(value)); }
+
+const char *backend_option(const char *env_name) {
+    const function *f = option_scope ? option_scope : global::get_implicit_function();
+    return f ? f->backend_option(env_name) : std::getenv(env_name);
+}
+
 static std::map<hardware_architecture_t, backend *> &backend_table() {
     static std::map<hardware_architecture_t, backend *> t;
     return t;
@@ -326,6 +378,8 @@ void function::Automatic_communication(computation *c1, computation *c2) {
 
 void function::codegen(const std::vector<buffer *> &arguments, const std::string obj_filename_in,
                        hardware_architecture_t arch) {
+    option_scope_guard scope(this);
+    clear_consulted_backend_options();
     if (arch == hardware_architecture_t::arch_nvidia_gpu) arch = hardware_architecture_t::arch_amd_gpu;
     // mapped buffers get their copies inserted for a GPU target (reference: tiramisu_function.cpp:2542-2549)
     if (arch == hardware_architecture_t::arch_amd_gpu && !mapping.empty())
@@ -351,7 +405,7 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
     }
     set_arguments(arguments);
     gen_time_space_domain();
-    if (arch == hardware_architecture_t::arch_amd_gpu && std::getenv("TIRAMISU_HIP_CHECK_MAPPED_LOOPS")) {
+    if (arch == hardware_architecture_t::arch_amd_gpu && backend_option("TIRAMISU_HIP_CHECK_MAPPED_LOOPS")) {
         const std::vector<std::string> races = gpu_mapped_loops_that_carry_dependences();
         bool refuse = false;
         for (auto &r : races) {
@@ -365,6 +419,7 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
 }
 
 void function::gen_halide_obj(const std::string &obj_file_name) {
+    option_scope_guard scope(this);
     hardware_architecture_t arch =
         hand_driven_gpu ? hardware_architecture_t::arch_amd_gpu : hardware_architecture_t::arch_cpu;
     // GPU-mapped loops without gen_cuda_stmt(): the reference leaves them to Halide's GPU target
@@ -1083,7 +1138,7 @@ void computation::separate_and_split(int level, int factor, const std::string &o
     isl_set *level_values = isl_set_project_out(isl_set_copy(ts), isl_dim_set, p + 1, 2 * n + 2 - (p + 1));
     level_values = isl_set_project_out(level_values, isl_dim_set, 0, p);
     const bool separable = !single_piece_text(isl_set_dim_max(isl_set_copy(level_values), 0)).empty() &&
-                           !single_piece_text(isl_set_dim_min(level_values, 0)).empty() && !std::getenv("TIRAMISU_NO_SEPARATION");
+                           !single_piece_text(isl_set_dim_min(level_values, 0)).empty() && !fct->backend_option("TIRAMISU_NO_SEPARATION");
     isl_val *mx = isl_set_dim_max_val(isl_set_copy(ts), p);
     isl_val *mn = isl_set_dim_min_val(ts, p);
     long extent = -1;

@@ -81,7 +81,7 @@ struct generic_kernel_gen {
         choose_lane_dimension(root);
         choose_workgroup_shape(root);
         choose_block_order(root);
-        if (!std::getenv("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
+        if (!backend_option("TIRAMISU_HIP_NO_WAVE_REDUCTION")) {
             std::vector<node_ptr> stack;
             find_reductions(root, stack);
         }
@@ -96,7 +96,7 @@ struct generic_kernel_gen {
     // unit stride becomes x.  Not done when some statement stores to memory at an element that does not involve
     // every thread loop around it (a sum or a broadcast across threads: the lowering of those is tied to x).
     void choose_lane_dimension(const node_ptr &root) {
-        if (std::getenv("TIRAMISU_HIP_KEEP_THREAD_DIMENSIONS")) return;
+        if (backend_option("TIRAMISU_HIP_KEEP_THREAD_DIMENSIONS")) return;
         int used = 0;
         for (int d = 0; d < 3; d++) used += loops_per_dim[1][d] > 0;
         if (used < 2) return;
@@ -189,7 +189,7 @@ struct generic_kernel_gen {
         long tile[2] = {0, 0}, wide[2] = {0, 0};     // the program's thread extents, the workgroup's
     } retile;
     void choose_workgroup_shape(const node_ptr &root) {
-        if (std::getenv("TIRAMISU_HIP_KEEP_TILES") || !threads_independent) return;
+        if (backend_option("TIRAMISU_HIP_KEEP_TILES") || !threads_independent) return;
         for (int d = 0; d < 3; d++)
             if (loops_per_dim[0][d] != (d < 2) || loops_per_dim[1][d] != (d < 2)) return;
         bool plain = true;
@@ -292,7 +292,7 @@ struct generic_kernel_gen {
     // integer division per workgroup (the 8192 x 8192 copy kernel, one element per thread: 0.152 ms against 0.105).
     int fast_block_dim = -1;      // 0 or 1 when the workgroups are renumbered
     void choose_block_order(const node_ptr &root) {
-        if (std::getenv("TIRAMISU_HIP_KEEP_BLOCK_ORDER")) return;
+        if (backend_option("TIRAMISU_HIP_KEEP_BLOCK_ORDER")) return;
         if (loops_per_dim[0][0] != 1 || loops_per_dim[0][1] != 1 || loops_per_dim[0][2] != 0) return;
         std::string it[2];
         lir::walk(root, [&](const node_ptr &n) {
@@ -529,7 +529,7 @@ struct generic_kernel_gen {
     }
 
     std::vector<node_ptr> without_redundant_barriers(const std::vector<node_ptr> &in) const {
-        if (std::getenv("TIRAMISU_HIP_KEEP_BARRIERS")) return in;
+        if (backend_option("TIRAMISU_HIP_KEEP_BARRIERS")) return in;
         std::vector<node_ptr> flat, v;
         std::function<void(const node_ptr &)> flatten = [&](const node_ptr &n) {
             if (n && n->kind == node_kind::block) for (auto &c : n->children) flatten(c);
@@ -865,7 +865,7 @@ struct host_gen {
     bool in_parallel_loop = false;
     int parallel_loops = 0;
     bool runs_in_parallel(const node_ptr &n) const {
-        if (!n->parallel || in_parallel_loop || std::getenv("TIRAMISU_HIP_SERIAL_HOST_LOOPS")) return false;
+        if (!n->parallel || in_parallel_loop || backend_option("TIRAMISU_HIP_SERIAL_HOST_LOOPS")) return false;
         const expr inc = lir::simplify(n->increment);
         if (!inc.is_integer_literal() || inc.get_int_val() != 1) return false;
         bool ok = true;
@@ -985,7 +985,7 @@ struct host_gen {
     // the body still run one after the other, each over all iterations, which keeps every dependence
     // that the serial loop body had within an iteration.)
     bool emit_batched(const node_ptr &n, int ind) {
-        if (std::getenv("TIRAMISU_HIP_NO_BATCHED_LAUNCH")) return false;
+        if (backend_option("TIRAMISU_HIP_NO_BATCHED_LAUNCH")) return false;
         std::vector<node_ptr> nests;
         if (n->body && n->body->kind == node_kind::block) nests = n->body->children;
         else if (n->body) nests.push_back(n->body);
@@ -1258,8 +1258,8 @@ public:
         }
         if (device_code) {
             const char *hipcc = std::getenv("HIPCC_PATH");
-            const char *arch = std::getenv("TIRAMISU_HIP_ARCH");
-            const char *flags = std::getenv("TIRAMISU_HIP_FLAGS");
+            const char *arch = backend_option("TIRAMISU_HIP_ARCH");
+            const char *flags = backend_option("TIRAMISU_HIP_FLAGS");
             std::vector<std::string> cmd = {hipcc ? hipcc : TIRAMISU_DEFAULT_HIPCC, "--genco",
                                             std::string("--offload-arch=") + (arch ? arch : TIRAMISU_DEFAULT_HIP_ARCH), "-std=c++17"};
             for (auto &w : words(flags ? flags : "-O3")) cmd.push_back(w);
@@ -1329,6 +1329,10 @@ public:
             m << "\n  ],\n  \"kernels\": [";
             for (size_t i = 0; i < ctx.kernels.size(); i++)
                 m << (i ? "," : "") << "\n    {\"name\": " << quoted(ctx.kernels[i].name) << ", \"how\": " << quoted(ctx.kernels[i].how) << "}";
+            m << "\n  ],\n  \"options\": [";
+            const auto &opts = f.consulted_backend_options();
+            for (size_t i = 0; i < opts.size(); i++)
+                m << (i ? "," : "") << "\n    {\"name\": " << quoted(opts[i][0]) << ", \"value\": " << quoted(opts[i][1]) << ", \"from\": " << quoted(opts[i][2]) << "}";
             m << "\n  ]\n}\n";
         }
         for (auto &k : ctx.kernels) f.log(k.name + ": " + k.how);

@@ -43,7 +43,7 @@
 //   ST_Y0, ST_Y1, ST_X0, ST_X1   inclusive bounds of the iteration domain
 //   ST_R               time steps fused in one launch
 //   ST_MODE            0, 1 or 2: see above
-//   ST_RAD             stencil radius (<= 4, <= ST_RPT)
+//   ST_RAD             stencil radius (<= 4, <= ST_RPT); 0 for a point-wise map (mode 3): nothing is exchanged
 //   ST_W               wavefronts per workgroup
 //   ST_RPT             rows per thread
 //   ST_RPT_EDGE        rows per thread in the kernel for boundary tiles (a divisor-sized slice
@@ -51,6 +51,7 @@
 //                      workgroups per boundary tile)
 //   ST_EXPR            expression of the new value in terms of ST_AT(dy, dx)
 //   ST_NAME_EDGE       name of the kernel for the tiles that touch the fixed boundary
+//   ST_STREAM          bit 0: staging loads carry the non-temporal hint, bit 1: the stores of the tile centre do
 //   ST_GX, ST_GY       number of tiles along x and y
 //   ST_IBX0, ST_IBX1, ST_IBY0, ST_IBY1   inclusive ranges of interior tiles (ST_IBY0 = ST_GY and
 //                      ST_IBY1 = ST_GY - 1 when there is none); launch ST_NAME with one workgroup
@@ -100,11 +101,16 @@ __device__ __forceinline__ float st_from_right(float v) {
 // cells outside the plane read as 0.  With CHECK false the quad is known to be inside.
 // Element loads always use a clamped (valid) address and select afterwards.  `plane` carries no
 // restrict qualifier: the boundary path reads the plane that the same kernel later writes.
-template <bool CHECK, int NY, int NX>
+// STREAM: the quad is asked for with the non-temporal hint (read once by this launch: it should not displace the
+// halo rows and columns that neighbouring tiles share in the L2).
+template <bool CHECK, int NY, int NX, bool STREAM = false>
 __device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx) {
     st_f4 v = {0.f, 0.f, 0.f, 0.f};
     if (NX % 4 == 0) {
-        if (!CHECK) return *reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx);
+        if (!CHECK) {
+            const st_f4 *q = reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx);
+            return STREAM ? __builtin_nontemporal_load(q) : *q;
+        }
         const bool in = gy >= 0 && gy < NY && gx >= 0 && gx < NX;
         const st_f4 a = *reinterpret_cast<const st_f4 *>(plane + (in ? (size_t)gy * NX + gx : (size_t)0));
         return in ? a : v;
@@ -142,7 +148,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     st_f4 cur[RPT], other[EDGE ? RPT : 1];   // other: the other plane's values (fixed cells only)
 #pragma unroll
     for (int r = 0; r < RPT; r++) {
-        cur[r] = st_load_quad<EDGE, ST_NY, ST_NX>(src, gy0 + r, gx);
+        cur[r] = st_load_quad<EDGE, ST_NY, ST_NX, (ST_STREAM & 1) != 0>(src, gy0 + r, gx);
         if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(fixed_other, gy0 + r, gx);
     }
 
@@ -163,7 +169,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
                 if (row < ST_HY || row >= ST_HY + CENTRE_ROWS || gy >= row_end) continue;
                 if (EDGE && (gy < WY0 || gy > WY1)) continue;
                 if ((ST_NX % 4 == 0) && (!EDGE || (gx >= WX0 && gx + 3 <= WX1))) {
-                    *reinterpret_cast<st_f4 *>(to + (size_t)gy * ST_NX + gx) = cur[r];
+                    st_f4 *q = reinterpret_cast<st_f4 *>(to + (size_t)gy * ST_NX + gx);
+                    if ((ST_STREAM & 2) != 0) __builtin_nontemporal_store(cur[r], q); else *q = cur[r];
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
@@ -182,7 +189,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
             *slot(parity, wave, 0, i) = cur[i];
             *slot(parity, wave, 1, i) = cur[RPT - ST_RAD + i];
         }
-        __syncthreads();
+        if (ST_RAD > 0) __syncthreads();
         // my rows with ST_RAD rows of the neighbouring wavefronts above and below
         st_f4 ext[RPT + 2 * ST_RAD];
 #pragma unroll
@@ -268,7 +275,7 @@ ST_NAME(float *planes, const int src_plane, float *temp)
 {
     static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
     static_assert(ST_MODE == 2 ? ST_R >= 2 : ST_MODE == 3 ? ST_R == 1 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
-    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    __shared__ st_f4 xch[2 * ST_W * 2 * (ST_RAD > 0 ? ST_RAD : 1) * 64];
     ST_PLANES
     const int b = blockIdx.x;
 #if ST_MERGE
@@ -295,7 +302,7 @@ ST_NAME(float *planes, const int src_plane, float *temp)
 extern "C" __global__ void __launch_bounds__(64 * ST_W)
 ST_NAME_EDGE(float *planes, const int src_plane, float *temp)
 {
-    __shared__ st_f4 xch[2 * ST_W * 2 * ST_RAD * 64];
+    __shared__ st_f4 xch[2 * ST_W * 2 * (ST_RAD > 0 ? ST_RAD : 1) * 64];
     ST_PLANES
     ST_CAT(ST_NAME, _edge_slice)(src, dst, dst_prev, fixed_other, xch, blockIdx.x);
 }

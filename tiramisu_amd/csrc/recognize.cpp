@@ -37,7 +37,7 @@ namespace {
 
 
 int env_int(const char *name, int dflt) {
-    const char *e = std::getenv(name);
+    const char *e = backend_option(name);
     return e ? std::atoi(e) : dflt;
 }
 
@@ -156,7 +156,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     // either a host time loop around a mapped nest, or a mapped nest whose time step is fixed
     // (a one-step time loop has no loop node in the AST)
     if ((!time_loop && !root) || (time_loop && root)) return false;
-    if (std::getenv("TIRAMISU_NO_STENCIL")) return false;
+    if (backend_option("TIRAMISU_NO_STENCIL")) return false;
     function *f = ctx.f;
     const node_ptr scope = time_loop ? time_loop->body : root;
     std::vector<node_ptr> leaves;
@@ -176,7 +176,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     // S(y, x) from another computation I(y+dy, x+dx) that lives in a buffer of its own
     const bool planar = its.size() == 2 && !time_loop;
     if ((its.size() != 3 && !planar) || S->get_data_type() != p_float32) return false;
-    if (planar && std::getenv("TIRAMISU_NO_SINGLE_STEP_STENCIL")) return false;
+    if (planar && backend_option("TIRAMISU_NO_SINGLE_STEP_STENCIL")) return false;
     if (!planar) {
         auto t_it = leaf->iterators.find(its[0]);
         if (t_it == leaf->iterators.end()) return false;
@@ -225,7 +225,8 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
         }
     };
     expr point = rewrite(S->get_expr());
-    if (!ok || radius < 1 || radius > 4) return false;
+    // radius 0 (a point-wise map of one buffer into another) is taken as a single step out of place only
+    if (!ok || radius > 4 || (radius < 1 && !planar)) return false;
 
     // store relation and buffer
     buffer *B = leaf->lhs, *BI = nullptr;
@@ -245,7 +246,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
             !access_equals(sources[0], "{ " + source_name + "[y,x] -> " + BI->get_name() + "[y, x] }")) return false;
     } else if (!access_equals(S, "{ " + S->get_name() + "[t,y,x] -> " + B->get_name() + "[t mod 2, y, x] }")) {
         return false;
-    } else if (!std::getenv("TIRAMISU_STENCIL_NO_FLOW_CHECK") && !flow_is_previous_step(S, B, taps)) {
+    } else if (!backend_option("TIRAMISU_STENCIL_NO_FLOW_CHECK") && !flow_is_previous_step(S, B, taps)) {
         return false;
     }
 
@@ -268,7 +269,9 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     const long T0 = lo[0], T1 = hi[0];
     const long steps = T1 - T0 + 1;
     // region staged by one workgroup: WAVES*ROWS rows by 256 columns (kernels/stencil2d_regs.hip.h)
-    const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", 11);
+    // fused launches: 8 wavefronts x 11 rows (a sweep over both put the optimum there); a single step out of place
+    // streams, and 4 rows per thread keep more workgroups and loads in flight
+    const int WAVES = env_int("TIRAMISU_STENCIL_WAVES", 8), ROWS = env_int("TIRAMISU_STENCIL_ROWS", planar ? 4 : 11);
     if (WAVES < 1 || WAVES > 16 || ROWS < radius || ROWS > 32) return false;
     const int LH = WAVES * ROWS, LW = 256;
     // most steps of one launch; a launch between the two planes takes the largest odd number below.  12: the final
@@ -357,11 +360,11 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
               << "\n#define ST_Y0 " << lo[1] << "\n#define ST_Y1 " << hi[1] << "\n#define ST_X0 " << lo[2] << "\n#define ST_X1 " << hi[2]
               << "\n#define ST_GX " << GX << "\n#define ST_GY " << GY << "\n#define ST_IBX0 " << bx0 << "\n#define ST_IBX1 " << bx1
               << "\n#define ST_IBY0 " << by0 << "\n#define ST_IBY1 " << by1 << "\n#define ST_W " << WAVES
-              << "\n#define ST_MERGE " << (merge ? 1 : 0) << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0)
+              << "\n#define ST_MERGE " << (merge ? 1 : 0) << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0) << "\n#define ST_STREAM " << env_int("TIRAMISU_STENCIL_STREAM", 2)
               << "\n#define ST_RPT " << ROWS << "\n#define ST_RPT_EDGE " << rows_edge << "\n#define ST_R " << ch.steps << "\n#define ST_MODE " << ch.mode << "\n#define ST_RAD " << radius
               << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
               << "#undef ST_NAME\n#undef ST_NAME_EDGE\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n"
-              << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n"
+              << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n#undef ST_STREAM\n"
               << "#undef ST_MERGE\n#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_MODE\n#undef ST_RAD\n#undef ST_EXPR\n";
             k.source = s.str();            // both kernels come from the one inclusion
             ke.source = "";
@@ -701,8 +704,8 @@ bool reject(int where) {
 }  // namespace
 
 bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, const fusion_request *fuse) {
-    if (std::getenv("TIRAMISU_NO_MFMA")) return false;
-    const bool with_consumer = fuse && fuse->consumer && !std::getenv("TIRAMISU_MFMA_NO_CONSUMER");
+    if (backend_option("TIRAMISU_NO_MFMA")) return false;
+    const bool with_consumer = fuse && fuse->consumer && !backend_option("TIRAMISU_MFMA_NO_CONSUMER");
     const bool batched = fuse && !fuse->batch_iterator.empty();
     if (fuse && fuse->consumer && !with_consumer) return false;
     function *f = ctx.f;
@@ -1165,7 +1168,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     // few C tiles but a long reduction (a batch-sized M against wide weights, as in recurrent cells):
     // 64x32 tiles, and 8 groups of wavefronts share the K range of each tile
     if (lit && !bf16 && BM == 64 && BN == 64 && Ml <= 64 && ((Nl + 63) / 64) <= ttarget::COMPUTE_UNITS / 4 && Nl % 32 == 0 && Kl % 128 == 0 && Kl >= 256 &&
-        !std::getenv("TIRAMISU_MFMA_NO_SPLITK")) {
+        !backend_option("TIRAMISU_MFMA_NO_SPLITK")) {
         BN = 32; BK = 128; WGM = 2; WGN = 1; WGK = 8; PADX = 0;
         DEPTH = (int)std::min<long>(4, std::max<long>(1, Kl / BK - 1));   // latency-bound: ask for (up to) all slices at once
         // a reduction of 1024 or more (several terms run as one loop): the loop is long enough to hide its own
@@ -1179,15 +1182,15 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         (Ml / 64) * (Nl / 64) <= ttarget::COMPUTE_UNITS) {
         WGK = 2; BK = 64;
     }
-    if (const char *e = std::getenv("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
-    if (const char *e = std::getenv("TIRAMISU_MFMA_BM")) BM = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_BN")) BN = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_WGM")) WGM = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_WGN")) WGN = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
-    if (const char *e = std::getenv("TIRAMISU_MFMA_WGK")) WGK = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
+    if (const char *e = backend_option("TIRAMISU_MFMA_BM")) BM = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_BN")) BN = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_WGM")) WGM = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_WGN")) WGN = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_BK")) BK = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_DEPTH")) DEPTH = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_PAD")) PADX = std::atoi(e);
+    if (const char *e = backend_option("TIRAMISU_MFMA_WGK")) WGK = std::atoi(e);
     bool bf16_edge = false;
     if (bf16) {
         // 256x256 when that fills the chip, else 128x128 (both load their slices straight into LDS and want whole
@@ -1248,7 +1251,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     std::string window_call_head;
     if (!bf16 && !with_consumer && lit && operands.size() == 1 && operands[0].first.linear && operands[0].first.kmajor &&
         !operands[0].second.linear && GK.dims.size() >= 2 && GK.literal && GN.literal && Ml % BM == 0 && Nl % BN == 0 && WGK == 1 &&
-        !std::getenv("TIRAMISU_MFMA_NO_WINDOW")) {
+        !backend_option("TIRAMISU_MFMA_NO_WINDOW")) {
         const operand_info &xo = operands[0].second;
         std::vector<long> ck, cn;
         bool ok = true;
@@ -1303,7 +1306,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
                 win_resident = 2 * (2 * stage_bytes + 64) <= ttarget::LDS_BYTES_PER_CU ? env_int("TIRAMISU_MFMA_WINDOW_RESIDENT", 2) : 1;
                 win_grid = std::min<long>(tiles, (long)ttarget::COMPUTE_UNITS * win_resident);
                 const long rest = tiles % win_grid;
-                if (rest > 0 && tiles > win_grid && !std::getenv("TIRAMISU_MFMA_NO_TAIL_SPLIT")) win_splits = (int)std::min<long>(std::min<long>(blocks, 2 * win_grid / rest), 16);
+                if (rest > 0 && tiles > win_grid && !backend_option("TIRAMISU_MFMA_NO_TAIL_SPLIT")) win_splits = (int)std::min<long>(std::min<long>(blocks, 2 * win_grid / rest), 16);
                 if (win_splits < 2) win_splits = 1;
                 // partial tiles of the pieces, a counter per remaining tile, the work queues' counters (pieces,
                 // finished workgroups, one per XCD)
@@ -1507,7 +1510,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     const std::string kname = "_kernel_" + std::to_string(ctx.next_kernel_id());
     // several product terms over plain operands: one pipelined loop over the concatenated reduction ranges
     // (a call per term would drain and refill the pipeline between the terms)
-    bool merge_terms = !bf16 && operands.size() > 1 && lit && Kl % 4 == 0 && !std::getenv("TIRAMISU_MFMA_SEPARATE_TERMS");
+    bool merge_terms = !bf16 && operands.size() > 1 && lit && Kl % 4 == 0 && !backend_option("TIRAMISU_MFMA_SEPARATE_TERMS");
     for (auto &o : operands) merge_terms = merge_terms && o.first.linear && o.second.linear;
     for (auto &o : operands) {
         if (!merge_terms || term == 0) body << "    {\n";
@@ -1565,7 +1568,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
                 // the k part of the offset (divisions by the extents of the reduction dimensions) is
                 // tabulated in LDS once per workgroup when the table is small: one LDS read per load
                 // instead of the digit arithmetic
-                const bool tabulate = small && lit && Kl * 4 <= 32768 && ktab_words == 0 && !std::getenv("TIRAMISU_MFMA_NO_KTAB");
+                const bool tabulate = small && lit && Kl * 4 <= 32768 && ktab_words == 0 && !backend_option("TIRAMISU_MFMA_NO_KTAB");
                 pre << "struct " << sname << " {\n    const float *__restrict__ base;\n    int XE, KE;\n    const int32_t *ktab;\n";
                 pre << "    static __device__ __forceinline__ " << OT << " koff(int _k) {\n" << digits(GK, "_k", "        ", false) << "        return 0";
                 for (int p : GK.dims) pre << " + (" << OT << ")" << U.dims[p].kvar << " * " << dev.print(g->coef.at(p));
@@ -1656,7 +1659,7 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         epi_store_text = dev.store(E.leaf->lhs, ix, "_v", val.get_data_type());
         epi_one_pass_text = dev.store(E.leaf->lhs, ix, epi_value_text, val.get_data_type());
     }
-    const bool two_pass = !(acc_stored && has_epi) && epi_is_float && !std::getenv("TIRAMISU_MFMA_ONE_PASS_EPILOGUE");
+    const bool two_pass = !(acc_stored && has_epi) && epi_is_float && !backend_option("TIRAMISU_MFMA_ONE_PASS_EPILOGUE");
     if (two_pass) {
         body << "    auto _epi_value = [&](int _r, int _c, float _sum) -> float {\n" << digit_text << accv_text;
         body << "        return " << (has_epi ? epi_value_text : std::string("_accv")) << ";\n    };\n";
