@@ -335,6 +335,9 @@ def bench_sgemm(M, steps, warmup, with_cpu):
     return out
 
 
+SKIP_STREAMING_RATES = False   # --no-streaming-rates: counter runs want the workload's own kernels only
+
+
 def streaming_rates(reps=30, with_torch=False):
     """Read-once-write-once rates on the benchmark's plane size (256 MiB read + 256 MiB written per pass, GB/s of both
     directions together), measured here: the ceiling that the HBM-bound stencil launches are stated against.
@@ -343,6 +346,8 @@ def streaming_rates(reps=30, with_torch=False):
       copy_plane_quads    the same program taken by the stencil emitter (16 bytes per lane, non-temporal stores)
       torch_copy / torch_add   torch.Tensor.copy_ and an element-wise add (second opinions; only with `with_torch`)"""
     from tiramisu_amd import runtime
+    if SKIP_STREAMING_RATES:
+        return {"ceiling": float("nan"), "vendor_d2d": float("nan"), "ceiling_basis": "not measured (--no-streaming-rates)"}
     w = runtime.wrappers()
     n = 8192
     nbytes = 2.0 * n * n * 4
@@ -547,7 +552,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-streaming-rates", action="store_true", help="skip the copy passes that calibrate the streaming ceiling")
     a = ap.parse_args()
+    global SKIP_STREAMING_RATES
+    SKIP_STREAMING_RATES = a.no_streaming_rates
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this back-end compiles single-GPU Tiramisu programs and nothing here "
                  "uses a second device (run with --gpus 1)")

@@ -69,6 +69,10 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
 int tiramisu_hip_sgemm_static_scratch(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
                                       float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
                                       uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
+/* The scratch block that deep reductions of tiramisu_hip_sgemm use on the calling thread's current stream (partial
+ * tiles and per-tile counters), or NULL before the first such call: one block per (host thread, stream), so that
+ * calls of one thread on two streams may overlap.  No counterpart in the reference; for tests and diagnostics. */
+void *tiramisu_hip_sgemm_workspace(void);
 
 /* ---- code objects and launches.  The reference links nvcc-compiled kernel wrappers
  *      (_kernel_N_wrapper, tiramisu_codegen_cuda.cpp:1288-1318) into the program; here
@@ -112,6 +116,11 @@ void tiramisu_hip_parallel_for(int32_t first, int32_t last, void (*body)(int32_t
  * block out again while that work still runs. */
 int tiramisu_hip_set_stream(void *stream);
 void *tiramisu_hip_get_stream(void);
+/* A new stream that does not synchronise with the default stream (default priority), for callers that overlap
+ * calls; destroy waits for the stream's work and, if it is the calling thread's current stream, restores the
+ * per-thread default stream.  Scratch blocks that the runtime keeps per (thread, stream) stay allocated. */
+void *tiramisu_hip_stream_create(void);
+int tiramisu_hip_stream_destroy(void *stream);
 void *tiramisu_hip_event_create(void);
 int tiramisu_hip_event_record(void *event);              /* on the current stream */
 float tiramisu_hip_event_elapsed_ms(void *start, void *stop); /* waits for `stop` */

@@ -138,3 +138,37 @@ def test_freed_device_blocks_are_reused():
     assert d == a and c not in (a, b)
     for p in (b, c, d):
         w.tiramisu_hip_free(p)
+
+
+def test_deep_reductions_on_two_streams_of_one_thread_use_separate_scratch():
+    """One host thread issues deep reductions alternately on two streams without waiting in between: each
+    stream has a scratch block of its own (partial tiles and counters would otherwise be shared by launches that
+    run at the same time), and every result is the exact integer product."""
+    from gpu_util import DeviceArray
+    w = runtime.wrappers()
+    M, N, K = 128, 192, 8192
+    rng = np.random.RandomState(44)
+    streams = [w.tiramisu_hip_stream_create(), w.tiramisu_hip_stream_create()]
+    jobs = []
+    for i in range(6):
+        A = rng.randint(-3, 4, (M, K)).astype(np.float32)
+        B = rng.randint(-3, 4, (K, N)).astype(np.float32)
+        jobs.append((A, B, DeviceArray(A), DeviceArray(B), DeviceArray(np.zeros((M, N), np.float32))))
+    blocks = set()
+    try:
+        for i, (A, B, dA, dB, dC) in enumerate(jobs):
+            w.tiramisu_hip_set_stream(streams[i % 2])
+            assert w.tiramisu_hip_sgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 1.0, 0.0, 0, 0, 0, 0, 0, 0, False, False) == 0
+            blocks.add((i % 2, w.tiramisu_hip_sgemm_workspace()))
+        for s in streams:
+            w.tiramisu_hip_set_stream(s)
+            w.tiramisu_hip_stream_synchronize(0)
+    finally:
+        w.tiramisu_hip_set_stream(None)
+    assert len(blocks) == 2 and len({b for _, b in blocks}) == 2 and all(b for _, b in blocks)
+    for A, B, dA, dB, dC in jobs:
+        assert np.array_equal(dC.download(), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+        for d in (dA, dB, dC):
+            d.free()
+    for s in streams:
+        w.tiramisu_hip_stream_destroy(s)

@@ -54,6 +54,30 @@ def test_two_calls_in_a_row_the_second_smaller():
     check_pair(192, 64, 4096, seed=4, tA=True, tB=True)
 
 
+def test_the_static_scratch_call_takes_no_workspace_block():
+    """In a thread of its own (the allocating entry point keeps its scratch per thread and stream, so a new thread
+    starts without any): a deep reduction through the static-scratch entry point leaves the thread without a
+    workspace block, the same shape through tiramisu_hip_sgemm creates one -- the static path did not fall through
+    to the allocating one."""
+    import threading
+    w = runtime.wrappers()
+    seen = {}
+
+    def body():
+        M, N, K = 128, 128, 4096
+        A, B, C = operands(M, N, K, 7, True)
+        rc, got = call(w.tiramisu_hip_sgemm_static_scratch, A, B, C, M, N, K, 1.0, 0.0)
+        seen["static"] = (rc, w.tiramisu_hip_sgemm_workspace(), got)
+        rc, expected = call(w.tiramisu_hip_sgemm, A, B, C, M, N, K, 1.0, 0.0)
+        seen["allocating"] = (rc, w.tiramisu_hip_sgemm_workspace(), expected)
+    t = threading.Thread(target=body)
+    t.start()
+    t.join()
+    assert seen["static"][0] == 0 and not seen["static"][1]
+    assert seen["allocating"][0] == 0 and seen["allocating"][1]
+    assert np.array_equal(seen["static"][2], seen["allocating"][2])
+
+
 def test_shape_that_does_not_split_runs_the_ordinary_kernels():
     check_pair(512, 512, 256, seed=5)
 

@@ -1278,7 +1278,7 @@ public:
             if (!h) ERROR("cannot write " + host_file, true);
             std::string sym = "_tiramisu_hsaco_" + sanitize(f.get_name());
             h << "// Generated by the Tiramisu HIP back-end: host glue of function " << f.get_name() << "\n";
-            h << "#include <stdint.h>\n#include <stdlib.h>\n#include <string.h>\n#include <math.h>\n";
+            h << "#include <stdint.h>\n#include <stdlib.h>\n#include <string.h>\n#include <math.h>\n#include <map>\n";
             h << "#include <tiramisu_hip_wrappers.h>\n";
             h << halide_buffer_definition() << c_prelude(false) << "\n";
             for (auto &d : hg.extern_decls) h << d << "\n";

@@ -318,10 +318,11 @@ void dispatch_splitk(const splitk_plan &p, bool tA, bool tB, bool edge, const fl
 #undef SPLITK_CASE
 }
 
-// Scratch of the allocating entry point: one block per host thread (calls work on the thread's
-// current stream), grown on demand, kept until the process ends.
-thread_local void *splitk_workspace = nullptr;
-thread_local uint64_t splitk_workspace_bytes = 0;
+// Scratch of the allocating entry point: one block per host thread and stream (a call works on the thread's
+// current stream, and two calls of one thread on two streams may run at the same time: they must not share partial
+// tiles and counters), grown on demand, kept until the process ends.
+struct splitk_block { void *ptr = nullptr; uint64_t bytes = 0; };
+thread_local std::map<hipStream_t, splitk_block> splitk_workspaces;
 constexpr uint64_t SPLITK_WORKSPACE_LIMIT = (uint64_t)256 << 20;
 
 // Scratch of the entry point that allocates nothing: lives in the code object, one copy per device.
@@ -520,15 +521,16 @@ static int sgemm_impl(const char *fn, bool static_scratch, float *A, float *B, f
             }
             ws = static_scratch_here();
         } else {
-            if (splitk_workspace_bytes < plan.scratch_bytes) {
-                if (splitk_workspace) {
+            splitk_block &block = splitk_workspaces[current_stream];
+            if (block.bytes < plan.scratch_bytes) {
+                if (block.ptr) {
                     check(hipStreamSynchronize(current_stream), fn);
-                    check(hipFree(splitk_workspace), fn);
+                    check(hipFree(block.ptr), fn);
                 }
-                check(hipMalloc(&splitk_workspace, plan.scratch_bytes), fn);
-                splitk_workspace_bytes = plan.scratch_bytes;
+                check(hipMalloc(&block.ptr, plan.scratch_bytes), fn);
+                block.bytes = plan.scratch_bytes;
             }
-            ws = splitk_workspace;
+            ws = block.ptr;
         }
         const bool edge = !(vec_ok && m % SPLITK_TILE == 0 && n % SPLITK_TILE == 0 && plan.chunk % 32 == 0 && k % plan.chunk == 0);
         dispatch_splitk(plan, transposeA, transposeB, edge, a, b, c, m, n, k, ldA, ldB, ldC, alpha, beta, vec_ok, ws);
@@ -554,6 +556,11 @@ int tiramisu_hip_sgemm_static_scratch(float *A, float *B, float *C, uint64_t M, 
                                       uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA, uint64_t offsetB, uint64_t offsetC,
                                       bool transposeA, bool transposeB) {
     return sgemm_impl(__FUNCTION__, true, A, B, C, M, N, K, alpha, beta, ldA, ldB, ldC, offsetA, offsetB, offsetC, transposeA, transposeB);
+}
+
+void *tiramisu_hip_sgemm_workspace(void) {
+    auto it = splitk_workspaces.find(current_stream);
+    return it == splitk_workspaces.end() ? nullptr : it->second.ptr;
 }
 
 int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha, double beta,
@@ -656,6 +663,20 @@ int tiramisu_hip_set_stream(void *stream) {
 }
 
 void *tiramisu_hip_get_stream(void) { return (void *)current_stream; }
+
+void *tiramisu_hip_stream_create(void) {
+    hipStream_t s;
+    check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), __FUNCTION__);   // default priority
+    return (void *)s;
+}
+
+int tiramisu_hip_stream_destroy(void *stream) {
+    if (!stream) return 0;
+    check(hipStreamSynchronize((hipStream_t)stream), __FUNCTION__);
+    if (current_stream == (hipStream_t)stream) current_stream = hipStreamPerThread;
+    check(hipStreamDestroy((hipStream_t)stream), __FUNCTION__);
+    return 0;
+}
 
 void *tiramisu_hip_event_create(void) {
     hipEvent_t e;

@@ -57,10 +57,29 @@
 //                      ST_IBY1 = ST_GY - 1 when there is none); launch ST_NAME with one workgroup
 //                      per interior tile and ST_NAME_EDGE with one per remaining tile
 // The tile extents follow: ST_TH = ST_W*ST_RPT - 2*ST_R*ST_RAD, ST_TW = 256 - 2*roundup4(ST_R*ST_RAD).
+//
+// The same text also compiles as plain host C++ (ST_HOST_MODEL defined by the includer, which then supplies
+// threadIdx / blockIdx and the few device keywords as stand-ins): every access to global memory goes through the
+// ST_GLOBAL_* macros below, the plane geometry may then be run-time values (ST_CONSTEXPR, ST_STATIC_ASSERT), and with
+// ST_SKIP_ARITHMETIC the steps are walked without computing -- which leaves exactly the kernel's own loads, stores
+// and the conditions they sit under, for a host program to enumerate.
+#ifndef ST_HOST_MODEL
 #include <hip/hip_runtime.h>
+#endif
 #include <stdint.h>
 
 #include "target_gfx950.h"
+
+#ifndef ST_CONSTEXPR
+#define ST_CONSTEXPR constexpr
+#define ST_STATIC_ASSERT(cond, text) static_assert(cond, text)
+#define ST_SKIP_ARITHMETIC 0
+// p: pointer to a quad (16 bytes) or to one cell; stream: ask with the non-temporal hint
+#define ST_GLOBAL_LOAD4(p, stream) ((stream) ? __builtin_nontemporal_load(p) : *(p))
+#define ST_GLOBAL_LOAD1(p) (*(p))
+#define ST_GLOBAL_STORE4(p, v, stream) do { if (stream) __builtin_nontemporal_store((v), (p)); else *(p) = (v); } while (0)
+#define ST_GLOBAL_STORE1(p, v) (*(p) = (v))
+#endif
 
 #define ST_HY (ST_R * ST_RAD)                       /* halo rows */
 #define ST_HX ((ST_R * ST_RAD + 3) / 4 * 4)         /* halo columns, multiple of 4 */
@@ -82,7 +101,11 @@
 
 #ifndef TIRAMISU_AMD_STENCIL2D_REGS_COMMON
 #define TIRAMISU_AMD_STENCIL2D_REGS_COMMON
+#ifdef ST_HOST_MODEL
+typedef float st_f4 __attribute__((vector_size(16)));
+#else
 typedef float st_f4 __attribute__((ext_vector_type(4)));
+#endif
 
 // lane i receives lane i-1's value; lane 0, which has no such neighbour, reads 0 (its cells next to the region's
 // edge are stale from the first step on and never written).  With nothing to keep for the lanes out of range, the
@@ -102,17 +125,14 @@ __device__ __forceinline__ float st_from_right(float v) {
 // Element loads always use a clamped (valid) address and select afterwards.  `plane` carries no
 // restrict qualifier: the boundary path reads the plane that the same kernel later writes.
 // STREAM: the quad is asked for with the non-temporal hint (read once by this launch: it should not displace the
-// halo rows and columns that neighbouring tiles share in the L2).
-template <bool CHECK, int NY, int NX, bool STREAM = false>
-__device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx) {
+// halo rows and columns that neighbouring tiles share in the L2).  NY, NX are compile-time constants in a kernel.
+template <bool CHECK, bool STREAM = false>
+__device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx, const int NY, const int NX) {
     st_f4 v = {0.f, 0.f, 0.f, 0.f};
     if (NX % 4 == 0) {
-        if (!CHECK) {
-            const st_f4 *q = reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx);
-            return STREAM ? __builtin_nontemporal_load(q) : *q;
-        }
+        if (!CHECK) return ST_GLOBAL_LOAD4(reinterpret_cast<const st_f4 *>(plane + (size_t)gy * NX + gx), STREAM);
         const bool in = gy >= 0 && gy < NY && gx >= 0 && gx < NX;
-        const st_f4 a = *reinterpret_cast<const st_f4 *>(plane + (in ? (size_t)gy * NX + gx : (size_t)0));
+        const st_f4 a = ST_GLOBAL_LOAD4(reinterpret_cast<const st_f4 *>(plane + (in ? (size_t)gy * NX + gx : (size_t)0)), false);
         return in ? a : v;
     }
     const bool row_in = !CHECK || (gy >= 0 && gy < NY);
@@ -120,7 +140,7 @@ __device__ __forceinline__ st_f4 st_load_quad(const float *plane, int gy, int gx
     for (int e = 0; e < 4; e++) {
         const int xx = gx + e;
         const bool in = row_in && (!CHECK || (xx >= 0 && xx < NX));
-        const float a = plane[in ? (size_t)gy * NX + xx : (size_t)0];
+        const float a = ST_GLOBAL_LOAD1(plane + (in ? (size_t)gy * NX + xx : (size_t)0));
         v[e] = in ? a : 0.f;
     }
     return v;
@@ -139,8 +159,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     // un-tiled program's
 #pragma clang fp contract(off)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    constexpr int CENTRE_ROWS = ST_W * RPT - 2 * ST_HY;
-    static_assert(CENTRE_ROWS > 0 && RPT >= ST_RAD, "the halo leaves no rows to write");
+    ST_CONSTEXPR int CENTRE_ROWS = ST_W * RPT - 2 * ST_HY;
+    ST_STATIC_ASSERT(CENTRE_ROWS > 0 && RPT >= ST_RAD, "the halo leaves no rows to write");
     const int gy0 = oy - ST_HY + wave * RPT;              // plane row of my first row
     const int gx = ox - ST_HX + 4 * lane;                 // plane column of my quads
     const int wave_up = wave > 0 ? wave - 1 : 0, wave_dn = wave < ST_W - 1 ? wave + 1 : ST_W - 1;
@@ -148,8 +168,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     st_f4 cur[RPT], other[EDGE ? RPT : 1];   // other: the other plane's values (fixed cells only)
 #pragma unroll
     for (int r = 0; r < RPT; r++) {
-        cur[r] = st_load_quad<EDGE, ST_NY, ST_NX, (ST_STREAM & 1) != 0>(src, gy0 + r, gx);
-        if (EDGE) other[r] = st_load_quad<true, ST_NY, ST_NX>(fixed_other, gy0 + r, gx);
+        cur[r] = st_load_quad<EDGE, (ST_STREAM & 1) != 0>(src, gy0 + r, gx, ST_NY, ST_NX);
+        if (EDGE) other[r] = st_load_quad<true>(fixed_other, gy0 + r, gx, ST_NY, ST_NX);
     }
 
     // xch[parity][wave][top|bottom][row][lane]
@@ -159,8 +179,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
 
     // ---- write the tile centre: the cells of the domain, or in mode 1 all cells of the plane (a fixed cell then
     // holds the value of the plane that `to` stands in for)
-    constexpr int WY0 = ST_MODE == 1 ? 0 : ST_Y0, WY1 = ST_MODE == 1 ? ST_NY - 1 : ST_Y1;
-    constexpr int WX0 = ST_MODE == 1 ? 0 : ST_X0, WX1 = ST_MODE == 1 ? ST_NX - 1 : ST_X1;
+    ST_CONSTEXPR int WY0 = ST_MODE == 1 ? 0 : ST_Y0, WY1 = ST_MODE == 1 ? ST_NY - 1 : ST_Y1;
+    ST_CONSTEXPR int WX0 = ST_MODE == 1 ? 0 : ST_X0, WX1 = ST_MODE == 1 ? ST_NX - 1 : ST_X1;
     auto store_centre = [&](float *__restrict__ to) {
         if (4 * lane >= ST_HX && 4 * lane < ST_HX + ST_TW) {
 #pragma unroll
@@ -169,12 +189,11 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
                 if (row < ST_HY || row >= ST_HY + CENTRE_ROWS || gy >= row_end) continue;
                 if (EDGE && (gy < WY0 || gy > WY1)) continue;
                 if ((ST_NX % 4 == 0) && (!EDGE || (gx >= WX0 && gx + 3 <= WX1))) {
-                    st_f4 *q = reinterpret_cast<st_f4 *>(to + (size_t)gy * ST_NX + gx);
-                    if ((ST_STREAM & 2) != 0) __builtin_nontemporal_store(cur[r], q); else *q = cur[r];
+                    ST_GLOBAL_STORE4(reinterpret_cast<st_f4 *>(to + (size_t)gy * ST_NX + gx), cur[r], (ST_STREAM & 2) != 0);
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (!EDGE || (gx + e >= WX0 && gx + e <= WX1)) to[(size_t)gy * ST_NX + gx + e] = cur[r][e];
+                        if (!EDGE || (gx + e >= WX0 && gx + e <= WX1)) ST_GLOBAL_STORE1(to + (size_t)gy * ST_NX + gx + e, cur[r][e]);
                 }
             }
         }
@@ -184,6 +203,7 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
     for (int s = 1; s <= ST_R; s++) {
         const int parity = s & 1;
         if (ST_MODE == 2 && s == ST_R) store_centre(dst_prev);   // the values after ST_R - 1 steps
+        if (ST_SKIP_ARITHMETIC) continue;
 #pragma unroll
         for (int i = 0; i < ST_RAD; i++) {
             *slot(parity, wave, 0, i) = cur[i];
@@ -241,8 +261,8 @@ __device__ __forceinline__ void ST_CAT(ST_NAME, _sweep)(const float *__restrict_
 static __device__ __forceinline__ void ST_CAT(ST_NAME, _edge_slice)(const float *__restrict__ src, float *__restrict__ dst,
                                                                      float *__restrict__ dst_prev, const float *fixed_other, st_f4 *xch, int eb)
 {
-    constexpr int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
-    constexpr int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
+    ST_CONSTEXPR int TOP = ST_IBY0 * ST_GX, BOTTOM = (ST_GY - 1 - ST_IBY1) * ST_GX;
+    ST_CONSTEXPR int SIDE = ST_IBX0 + (ST_GX - 1 - ST_IBX1);   // edge tiles per row of the interior band
     const int sub = eb % ST_EDGE_SUB;
     int e = eb / ST_EDGE_SUB, bx, by;
     if (e < TOP) {
@@ -273,8 +293,8 @@ __attribute__((amdgpu_waves_per_eu(ST_OCC)))
 #endif
 ST_NAME(float *planes, const int src_plane, float *temp)
 {
-    static_assert(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
-    static_assert(ST_MODE == 2 ? ST_R >= 2 : ST_MODE == 3 ? ST_R == 1 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
+    ST_STATIC_ASSERT(ST_TH > 0 && ST_TW > 0, "the halo leaves no tile: fuse fewer steps or use more rows");
+    ST_STATIC_ASSERT(ST_MODE == 2 ? ST_R >= 2 : ST_MODE == 3 ? ST_R == 1 : ST_R % 2 == 1, "a launch between the two planes advances an odd number of steps");
     __shared__ st_f4 xch[2 * ST_W * 2 * (ST_RAD > 0 ? ST_RAD : 1) * 64];
     ST_PLANES
     const int b = blockIdx.x;
@@ -286,8 +306,8 @@ ST_NAME(float *planes, const int src_plane, float *temp)
 #endif
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: give every XCD a band
     // of consecutive tiles (row-major), so that tiles running together share their halos in L2.
-    constexpr int IW = ST_IBX1 - ST_IBX0 + 1;
-    constexpr int nb = ST_NI;
+    ST_CONSTEXPR int IW = ST_IBX1 - ST_IBX0 + 1;
+    ST_CONSTEXPR int nb = ST_NI;
 #if ST_XCD
     constexpr int XCDS = ttarget::XCDS;
     const int xcd = b % XCDS, per = nb / XCDS, extra = nb % XCDS;

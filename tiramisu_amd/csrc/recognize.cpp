@@ -8,6 +8,7 @@
 #include <sstream>
 
 #include "hip_backend.h"
+#include "stencil_plan.h"
 #include <tiramisu/isl_api.h>
 #include "kernels/target_gfx950.h"
 #include "util.h"
@@ -276,43 +277,11 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     const int LH = WAVES * ROWS, LW = 256;
     // most steps of one launch; a launch between the two planes takes the largest odd number below.  12: the final
     // launch writes two planes and has HBM time to cover one step more than the 11 of the others
-    int rcap = env_int("TIRAMISU_STENCIL_STEPS", 12);
-    // keep at least half of the staged rows and columns as the tile
-    while (rcap > 1 && (4 * rcap * radius > LH || 4 * ((rcap * radius + 3) / 4 * 4) > LW)) rcap -= 1;
-    if (rcap < 1) rcap = 1;
-    const int rmax = rcap % 2 == 0 ? rcap - 1 : rcap;
+    const int rcap = tstencil::step_cap(env_int("TIRAMISU_STENCIL_STEPS", 12), radius, LH);
     if (2 * radius >= LH) return false;
-    struct chunk { long first; int steps; int mode; };   // first step, number of steps, kernel mode (stencil2d_regs.hip.h)
-    auto odd_chunks = [&](long first, long count) {
-        std::vector<chunk> out;
-        while (count > 0) {
-            int c = (int)std::min<long>(rmax, count);
-            if (c % 2 == 0) c -= 1;
-            out.push_back({first, c, 0});
-            first += c;
-            count -= c;
-        }
-        return out;
-    };
-    std::vector<chunk> chunks;
-    const bool temp_plane = !planar && steps >= 3 && env_int("TIRAMISU_STENCIL_TEMP_PLANE", 1) != 0;
-    if (planar) {
-        chunks.push_back({T0, 1, 3});
-    } else if (temp_plane) {
-        // the final launch's length: the one that needs the fewest launches (the longest of those)
-        int best = 2;
-        size_t best_n = 0;
-        for (int fin = (int)std::min<long>(rcap, steps - 1); fin >= 2; fin--) {
-            const size_t n = odd_chunks(T0, steps - fin).size();
-            if (best_n == 0 || n < best_n) { best = fin; best_n = n; }
-        }
-        chunks = odd_chunks(T0, steps - best);
-        chunks.back().mode = 1;
-        chunks.push_back({T0 + steps - best, best, 2});
-    } else {
-        chunks = odd_chunks(T0, steps - 1);
-        chunks.push_back({T0 + steps - 1, 1, 0});
-    }
+    typedef tstencil::chunk chunk;   // first step, number of steps, kernel mode (stencil2d_regs.hip.h)
+    const bool temp_plane = !planar && steps >= 3 && rcap >= 2 && env_int("TIRAMISU_STENCIL_TEMP_PLANE", 1) != 0;
+    const std::vector<chunk> chunks = tstencil::plan_time_loop(T0, steps, rcap, planar, temp_plane);
 
     c_printer dev;
     dev.fct = f;
@@ -320,8 +289,6 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     const std::string point_text = dev.print(point);
     std::map<std::pair<int, int>, std::pair<kernel, kernel>> by_steps;   // (steps, mode) -> (interior tiles, tiles on the fixed boundary)
     std::ostringstream host;
-    auto ceil_div = [](long a, long b) { return a >= 0 ? (a + b - 1) / b : -((-a) / b); };
-    auto floor_div = [](long a, long b) { return a >= 0 ? a / b : -((-a + b - 1) / b); };
     // one launch per chunk: the boundary slices ride behind the interior tiles (TIRAMISU_STENCIL_MERGE=0: two launches)
     const bool merge = env_int("TIRAMISU_STENCIL_MERGE", 1) != 0;
     static const char *const mode_text[] = {"", ", into a third plane", ", from a third plane into both planes", ", out of place"};
@@ -337,18 +304,10 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
             kernel k, ke;
             k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
             ke.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
-            const int HY = ch.steps * radius, HX = (ch.steps * radius + 3) / 4 * 4;
-            const int TH = LH - 2 * HY, TW = LW - 2 * HX;
-            const long GX = (NX + TW - 1) / TW, GY = (NY + TH - 1) / TH;
-            // tiles whose staged region [b*T - H, b*T - H + L) lies inside the iteration domain
-            long bx0 = std::max<long>(0, ceil_div(lo[2] + HX, TW)), bx1 = std::min<long>(GX - 1, floor_div(hi[2] - LW + 1 + HX, TW));
-            long by0 = std::max<long>(0, ceil_div(lo[1] + HY, TH)), by1 = std::min<long>(GY - 1, floor_div(hi[1] - LH + 1 + HY, TH));
-            if (bx0 > bx1 || by0 > by1) { by0 = GY; by1 = GY - 1; bx0 = 0; bx1 = GX - 1; }   // no interior tile
-            const long interior = (bx1 - bx0 + 1) * (by1 - by0 + 1), edge_tiles = GX * GY - interior;
-            // boundary tiles are cut into slices of half the rows per thread when the halo allows it
-            int rows_edge = ROWS / 2;
-            if (rows_edge < radius || WAVES * rows_edge - 2 * HY < 8) rows_edge = ROWS;
-            const int TH_edge = WAVES * rows_edge - 2 * HY, edge_sub = (TH + TH_edge - 1) / TH_edge;
+            const tstencil::launch_geometry g = tstencil::plan_launch(NY, NX, lo[1], hi[1], lo[2], hi[2], radius, ch.steps, WAVES, ROWS);
+            const int TH = g.tile_rows, TW = g.tile_columns, rows_edge = g.rows_edge, TH_edge = g.slice_rows, edge_sub = g.slices;
+            const long GX = g.tiles_x, GY = g.tiles_y, bx0 = g.ibx0, bx1 = g.ibx1, by0 = g.iby0, by1 = g.iby1;
+            const long interior = g.interior, edge_tiles = g.edge_tiles;
             k.how = "stencil: " + std::to_string(ch.steps) + " time step(s) per launch, radius " + std::to_string(radius) +
                     ", tile " + std::to_string(TH) + "x" + std::to_string(TW) + " in registers, " + std::to_string(WAVES) +
                     " wavefronts x " + std::to_string(ROWS) + " rows, " + std::to_string(interior) + " interior tiles" + mode_text[ch.mode];
@@ -1744,15 +1703,17 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         k.params.push_back({true, nm, b->get_elements_type()});
     }
     if (windowed) {
-        // scratch for the pieces of the last round's tiles and their counters: one block per host thread (calls
-        // work on the thread's current stream), allocated at the first call and kept; the counters start at zero
-        // and every launch leaves them at zero
+        // scratch for the pieces of the last round's tiles and their counters: one block per host thread and
+        // stream (a call works on the thread's current stream; calls of one thread on two streams may overlap and
+        // must not share queues and counters), allocated at the first call there and kept; the counters start at
+        // zero and every launch leaves them at zero
         // (buffer parameters stay sorted by name)
         auto at = k.params.begin();
         while (at != k.params.end() && (!at->is_buffer || at->name < "_tail_scratch")) ++at;
         k.params.insert(at, {true, "_tail_scratch", p_float32});
         k.grid[0] = std::to_string(win_grid);
-        host << "        static thread_local float *_tail_scratch = nullptr;\n";
+        host << "        static thread_local std::map<void *, float *> _tail_scratch_of;\n";
+        host << "        float *&_tail_scratch = _tail_scratch_of[tiramisu_hip_get_stream()];\n";
         host << "        if (!_tail_scratch) {\n";
         host << "            _tail_scratch = (float *)tiramisu_hip_malloc((uint64_t)" << win_scratch_floats << " * sizeof(float));\n";
         host << "            static const uint32_t _zeros[" << win_counters << "] = {};\n";

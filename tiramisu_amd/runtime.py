@@ -96,6 +96,9 @@ def wrappers():
         lib.tiramisu_hip_stream_synchronize.argtypes = [ctypes.c_int32]
         lib.tiramisu_hip_set_stream.argtypes = [ctypes.c_void_p]
         lib.tiramisu_hip_get_stream.restype = ctypes.c_void_p
+        lib.tiramisu_hip_stream_create.restype = ctypes.c_void_p
+        lib.tiramisu_hip_stream_destroy.argtypes = [ctypes.c_void_p]
+        lib.tiramisu_hip_sgemm_workspace.restype = ctypes.c_void_p
         lib.tiramisu_hip_event_create.restype = ctypes.c_void_p
         lib.tiramisu_hip_event_record.argtypes = [ctypes.c_void_p]
         lib.tiramisu_hip_event_elapsed_ms.restype = ctypes.c_float
