@@ -53,6 +53,11 @@ void codegen(const std::vector<buffer *> &arguments, const std::string obj_filen
 /** function::set_backend_option on the implicit function. */
 void set_backend_option(const std::string &name, const std::string &value);
 void set_backend_option(const std::string &name, long value);
+/** Lets whoever runs a generator program choose back-end options: every "--backend-option name=value" (or
+  * "--backend-option=name=value") among the arguments becomes an option of every function that tiramisu::init
+  * creates afterwards; the program's own set_backend_option calls still override them.  Other arguments are
+  * left alone; returns the number of options taken.  Call it first thing in main(argc, argv). */
+int backend_options_from_command_line(int argc, char **argv);
 /** The option of the function whose code is being generated (of the implicit function outside code
   * generation); plain getenv when there is no function at all.  For the back-end's own sources. */
 const char *backend_option(const char *env_name);

@@ -5,8 +5,9 @@
 
 using namespace tiramisu;
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     const int M = 96, N = 160, K = 64;
     tiramisu::init("gemm_gpu_tile");
 

@@ -1,7 +1,12 @@
-"""tiramisu_amd.autotune: knob combinations, argument construction from the back-end's description of
-a function, the argument check in runtime.Program, and evaluation by execution -- two candidates of one
-program are generated ahead of time (no GPU needed: the generator calls hipcc), then timed on the GPU
-through evaluate_by_execution, which must give equal results and a positive time for each."""
+"""Evaluation by execution.  tiramisu_amd.autotune: option combinations, argument construction from the back-end's
+description of a function, the argument check in runtime.Program, and two candidates of one program -- option
+sets handed to the generator as --backend-option arguments, nothing through the environment -- generated ahead of
+time (no GPU needed: the generator calls hipcc), then timed on the GPU, which must give equal results and a
+positive time for each.  The C++ class tiramisu::auto_scheduler::evaluate_by_execution (the reference's
+include/tiramisu/auto_scheduler/evaluator.h:34-80) is driven through the compiled tuner
+tiramisu_amd/tuning/square_tiles.cpp: without a GPU with a stand-in wrapper command (candidates are generated,
+compiled, linked, their options recorded in the manifest), on the GPU with the real wrapper, whose kept outputs
+must be alpha * A x B + beta * C."""
 import json
 import os
 
@@ -60,7 +65,7 @@ def test_arguments_are_checked_before_the_call(product_programs_dir):
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 EVAL_DIR = os.path.join(ROOT, "tests", "programs", "build", "evaluate_by_execution")
-CANDIDATES = [{"TIRAMISU_MFMA_BK": "16"}, {"TIRAMISU_MFMA_BK": "32"}]
+CANDIDATES = [{"mfma_bk": "16"}, {"mfma_bk": "32"}]      # back-end options (function::set_backend_option)
 
 
 def evaluator():
@@ -72,8 +77,9 @@ def test_candidates_are_prepared_without_a_gpu():
     for c in CANDIDATES:
         lib = ev.prepare(c)
         assert os.path.exists(lib)
-        slices = "x%s," % c["TIRAMISU_MFMA_BK"]
-        assert any(slices in k["how"] for k in runtime.manifest_of(lib, "gemm_gpu_tile")["kernels"])   # the knob reached the emitter
+        slices = "x%s," % c["mfma_bk"]
+        assert any(slices in k["how"] for k in runtime.manifest_of(lib, "gemm_gpu_tile")["kernels"])   # the option reached the emitter
+        assert ev.options_used(c) == c and "TIRAMISU_MFMA_BK" not in os.environ
 
 
 @pytest.mark.gpu
@@ -95,3 +101,42 @@ def test_evaluate_by_execution_times_candidates_on_the_gpu():
     m = runtime.manifest_of(ev.library(CANDIDATES[0]), "gemm_gpu_tile")
     A, B, C = autotune.make_arguments(m, ev.seed)
     assert np.array_equal(outputs[0][0], C + A @ B)
+
+
+# ---------------------------------------------------------------- the C++ evaluator, through a compiled tuner
+
+TUNER_DIR = os.path.join(ROOT, "tests", "programs", "build", "square_tiles")
+
+
+def test_cpp_evaluator_generates_compiles_and_links_every_candidate():
+    """No GPU: the wrapper command is a stand-in that prints three times.  The tuner must have generated the
+    program once per candidate on one tiramisu::function, and the last manifest records the candidate's option."""
+    import json
+    import shutil
+    shutil.rmtree(TUNER_DIR, ignore_errors=True)
+    lines = autotune.run_tuner("square_tiles", TUNER_DIR, "--wrapper", "echo 1.5 2.5 3.5 #", 256)
+    assert len(lines) == 1
+    r = lines[0]
+    assert r["size"] == 256 and r["model_tile"] in (64, 128, 256)
+    assert set(r["ms"]) == {"default", "64", "128", "256"} and all(v == 2.5 for v in r["ms"].values())   # medians of the stand-in
+    m = json.load(open(os.path.join(TUNER_DIR, "sgemm_tiles_256.o.json")))
+    assert m["options"] == [{"name": "mfma_tile", "value": "256", "from": "program"}]
+    assert "tile 256x256x16" in m["kernels"][0]["how"]
+    assert os.path.exists(os.path.join(TUNER_DIR, "sgemm_tiles_256.o.so"))
+
+
+@pytest.mark.gpu
+def test_cpp_evaluator_times_candidates_and_reproduces_the_product(tmp_path):
+    outputs = str(tmp_path / "outputs.npz")
+    wrapper = "python3 -m tiramisu_amd.autotune --time --repeat 5 --outputs " + outputs
+    lines = autotune.run_tuner("square_tiles", str(tmp_path), "--wrapper", wrapper, 256)
+    r = lines[0]
+    print(r, flush=True)
+    assert all(0 < v < 1e3 for v in r["ms"].values())
+    assert str(r["fastest_tile"]) in r["ms"]
+    got = np.load(outputs)
+    scal, A, B, C0 = autotune.make_arguments(json.load(open(str(tmp_path / "sgemm_tiles_256.o.json"))), 1)   # the wrapper's seeded inputs
+    expected = scal[0] * (A.host.astype(np.float64) @ B.host.astype(np.float64)) + scal[1] * C0.host
+    assert np.array_equal(got["b_C"], expected.astype(np.float32))
+    for a in (A, B, C0):
+        a.free()

@@ -25,7 +25,7 @@ ISL = "-l:libisl.so.23"
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
-COMPILER_SOURCES = ["expr.cpp", "core.cpp", "astgen.cpp", "c_print.cpp", "hip_backend.cpp",
+COMPILER_SOURCES = ["expr.cpp", "core.cpp", "astgen.cpp", "c_print.cpp", "hip_backend.cpp", "evaluator.cpp",
                     "recognize.cpp", "dependences.cpp"]
 
 PROGRAM_DIRS = [os.path.join(PKG, "programs"), os.path.join(ROOT, "tests", "programs")]
@@ -229,6 +229,11 @@ def build_all(force=True, verbose=False):
         for f in sorted(os.listdir(WRAPPER_DIR)):
             if f.endswith(".cpp"):
                 build_wrapper_program(os.path.join(WRAPPER_DIR, f))
+    # the compiled tuners (they drive the C++ evaluator on the GPU machine; compiling them needs none)
+    from . import autotune
+    for f in sorted(os.listdir(autotune.TUNING)):
+        if f.endswith(".cpp"):
+            autotune.build_tuner(f[:-4])
 
 
 if __name__ == "__main__":

@@ -65,9 +65,30 @@ static std::string params_prefix(const std::vector<std::string> &params) {
 
 // ------------------------------------------------------------------ init / codegen
 
+static std::map<std::string, std::string> &command_line_options() {
+    static std::map<std::string, std::string> o;
+    return o;
+}
+
+int backend_options_from_command_line(int argc, char **argv) {
+    int taken = 0;
+    for (int i = 1; i < argc; i++) {
+        std::string a = argv[i], kv;
+        if (a == "--backend-option" && i + 1 < argc) kv = argv[++i];
+        else if (a.rfind("--backend-option=", 0) == 0) kv = a.substr(17);
+        else continue;
+        const size_t eq = kv.find('=');
+        if (eq == std::string::npos || eq == 0) ERROR("--backend-option wants name=value, got: " + kv, true);
+        command_line_options()[kv.substr(0, eq)] = kv.substr(eq + 1);
+        taken++;
+    }
+    return taken;
+}
+
 void init(std::string name) {
     function *f = new function(name);
     global::set_implicit_function(f);
+    for (auto &o : command_line_options()) f->set_backend_option(o.first, o.second);
 }
 
 void init() { init("foo"); }

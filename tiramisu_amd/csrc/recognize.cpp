@@ -1141,7 +1141,8 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         (Ml / 64) * (Nl / 64) <= ttarget::COMPUTE_UNITS) {
         WGK = 2; BK = 64;
     }
-    if (const char *e = backend_option("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; }
+    // a forced square tile starts from that tile's own defaults (no K groups, slices of 32 for 64x64, of 16 above)
+    if (const char *e = backend_option("TIRAMISU_MFMA_TILE")) { BM = BN = std::atoi(e); PADX = BM == 256 ? 0 : 1; WGM = WGN = 2; WGK = 1; DEPTH = 1; BK = BM == 64 ? 32 : 16; }
     if (const char *e = backend_option("TIRAMISU_MFMA_BM")) BM = std::atoi(e);
     if (const char *e = backend_option("TIRAMISU_MFMA_BN")) BN = std::atoi(e);
     if (const char *e = backend_option("TIRAMISU_MFMA_WGM")) WGM = std::atoi(e);

@@ -85,8 +85,9 @@ static void generate(int NB, int CI, int CO, int H)
 #endif
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     if (const char *nb = std::getenv("CONV_ONLY_FULL")) {   // experiments: the benchmark shape alone, with another batch size
         generate(std::atoi(nb) > 1 ? std::atoi(nb) : 32, 64, 64, 112);
         return 0;

@@ -39,8 +39,9 @@ static void generate(int N, int STEPS)
 #endif
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     generate(8192, 32);   // the benchmark configuration
     if (std::getenv("HEAT2D_ONLY_FULL")) return 0;   // for sweeps over the emitter's knobs
     generate(1024, 8);

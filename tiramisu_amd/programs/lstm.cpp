@@ -141,8 +141,9 @@ static void generate(int L, int B, int H, int S)
 #endif
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     generate(4, 64, 512, 100);   // benchmark configuration 5
     if (std::getenv("LSTM_ONLY_FULL")) return 0;
     generate(2, 8, 32, 5);

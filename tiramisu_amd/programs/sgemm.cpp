@@ -75,8 +75,9 @@ static void generate(int M, int N, int K)
 #endif
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     // SGEMM_ONLY_CUBE=<n>: only the n x n x n instance (for sweeps over the emitter's knobs)
     if (const char *n = std::getenv("SGEMM_ONLY_CUBE")) {
         generate(std::atoi(n), std::atoi(n), std::atoi(n));

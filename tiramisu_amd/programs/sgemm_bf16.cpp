@@ -68,8 +68,9 @@ static void generate(int M, int N, int K)
 #endif
 }
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     generate(4096, 4096, 4096);   // benchmark configuration 3, bf16-input variant
     if (std::getenv("SGEMM_BF16_ONLY_FULL")) return 0;   // for sweeps over the emitter's knobs
     generate(4096, 3072, 32);     // 256x256 tiles, a single K-slice

@@ -7,8 +7,9 @@
 
 using namespace tiramisu;
 
-int main()
+int main(int argc, char **argv)
 {
+    tiramisu::backend_options_from_command_line(argc, argv);
     const int N = 8192;
     tiramisu::init("sweep5_8192x8192");
     var yy("yy", 0, N), xx("xx", 0, N), y("y", 1, N - 1), x("x", 1, N - 1);
