@@ -75,3 +75,14 @@ def test_gpu_matches_numpy(programs_dir, name):
             assert np.array_equal(got, expected.astype(np.float32))
         else:
             assert_fp32_parity(got, expected, name + " vs float64 numpy", 1e-4)
+
+
+def test_sum_across_wavefronts_under_a_condition_keeps_the_barrier_out(programs_dir):
+    """tests/programs/thread_reduction_under_condition.cpp: the 256-thread loop sits under `if (block iterator >= 3)`.
+    The lowering across wavefronts ends in a workgroup barrier that every thread must reach, so the emitter must not
+    use it below a condition: the kernel stays as the program states it (no LDS stage, no barrier)."""
+    text = open(os.path.join(programs_dir, "build", "row_sums_from_row_3.o.hip")).read()
+    kernel = text[text.index('extern "C" __global__'):]
+    assert "if ((c1 >= 3))" in kernel
+    assert "block_group_sum" not in kernel and "__syncthreads" not in kernel
+    assert "DPP wavefront reductions" not in re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)

@@ -164,6 +164,18 @@ struct generic_kernel_gen {
         for (int d = 1; d < 3; d++)
             if (loops_per_dim[1][d] > 0 && score[d] > score[best]) best = d;
         if (best == 0) return;
+        if (best == 2) {
+            // what x carried moves to z, and a workgroup is at most 64 deep along z
+            bool fits = true;
+            lir::walk(root, [&](const node_ptr &n) {
+                if (n->kind != node_kind::loop || n->gpu_thread != 0) return;
+                bool guard;
+                expr first;
+                const expr ext = lir::simplify(host_extent(n, first, guard));
+                if (!ext.is_integer_literal() || ext.get_int_val() > 64) fits = false;
+            });
+            if (!fits) return;
+        }
         lir::walk(root, [&](const node_ptr &n) {
             if (n->kind != node_kind::loop) return;
             if (n->gpu_thread == 0) n->gpu_thread = best;
@@ -352,7 +364,7 @@ struct generic_kernel_gen {
     struct thread_reduction { node_ptr leaf; expr term; int width; };
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
-    int guard_depth = 0;          // mapped loops with a guard around the code being emitted
+    int conds_above = 0;          // conditions between the kernel's root and the node that find_reductions is visiting
 
     static bool is_same_element(const expr &e, const buffer *b, const std::vector<expr> &idx) {
         if (e.get_expr_type() != e_op || e.get_op_type() != o_access || e.get_name() != b->get_name() || e.get_access().size() != idx.size())
@@ -370,8 +382,10 @@ struct generic_kernel_gen {
             consider_reduction(n, stack);
         for (auto &c : n->children) find_reductions(c, stack);
         find_reductions(n->body, stack);
+        if (n->kind == node_kind::cond) conds_above++;
         find_reductions(n->then_body, stack);
         find_reductions(n->else_body, stack);
+        if (n->kind == node_kind::cond) conds_above--;
         if (n->kind == node_kind::loop) stack.pop_back();
     }
 
@@ -415,7 +429,11 @@ struct generic_kernel_gen {
         if (!in_wave && !waves) return;
         if (waves) {
             // the barrier of the LDS stage must be reached by every thread: no guarded mapped loop around it,
-            // no serial loop or condition between the kernel entry and the loop
+            // no serial loop and no condition (a separated remainder, a hoisted predicate: it may depend on a
+            // thread iterator) between the kernel entry and the loop.  (Adding the wavefronts' totals with
+            // atomics instead would need no barrier, but nothing would then order them after an initialisation of
+            // the element that other wavefronts of the workgroup execute: the barrier is what does that.)
+            if (conds_above > 0) return;
             for (size_t d = 0; d < at; d++) {
                 bool g;
                 expr f0;

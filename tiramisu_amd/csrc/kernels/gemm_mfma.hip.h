@@ -61,12 +61,26 @@ __device__ __forceinline__ f32x4 load_handed_over(const f32x4 *p) {
 // every store_handed_over of this wavefront has reached memory when this returns.  The wait is written out: a
 // release fence at workgroup scope orders the stores for the wavefronts of this compute unit only and, outside
 // thread-group-split mode, waits for nothing (a reader on another die then sees the counter before the data).
+// This relies on what gfx942 / gfx950 do, not on the HIP memory model: an agent-scope relaxed atomic store is
+// written through to memory (sc1), vmcnt counts it down when memory has acknowledged it, and 0x0F70 is the gfx9
+// encoding of "vmcnt(0) only".  Any other target takes the portable form: an agent-scope release fence (which
+// writes the whole L2 back: correct, slow); TIRAMISU_PORTABLE_HANDOVER forces it here too.
 __device__ __forceinline__ void handed_over_stores_done() {
+#if (defined(__gfx950__) || defined(__gfx942__)) && !defined(TIRAMISU_PORTABLE_HANDOVER)
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0), leaving expcnt and lgkmcnt alone
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+#elif defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#endif
 }
 // no load_handed_over is moved ahead of this point (placed behind the counter's read)
-__device__ __forceinline__ void handed_over_loads_begin() { __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup"); }
+__device__ __forceinline__ void handed_over_loads_begin() {
+#if (defined(__gfx950__) || defined(__gfx942__)) && !defined(TIRAMISU_PORTABLE_HANDOVER)
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#else
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
+}
 
 // An operand stored with one unit stride: element (x, k) lives at base[x*ld + k] (KMAJOR) or
 // base[k*ld + x].  With EDGE, elements outside XE x KE read as zero and rows need not be
