@@ -69,6 +69,15 @@ int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, 
 int tiramisu_hip_sgemm_static_scratch(float *A, float *B, float *C, uint64_t M, uint64_t N, uint64_t K, float alpha,
                                       float beta, uint64_t ldA, uint64_t ldB, uint64_t ldC, uint64_t offsetA,
                                       uint64_t offsetB, uint64_t offsetC, bool transposeA, bool transposeB);
+/* Batch scope (no counterpart in the reference).  Between _begin and _end the calling thread's tiramisu_hip_sgemm
+ * calls are gathered instead of launched; _end launches them in call order, runs of calls of one shape (sizes,
+ * leading dimensions, transposition, alpha, beta) as ONE launch with a problem per blockIdx.z (up to 8 per launch).
+ * The gathered calls must be independent of one another: generated code opens a scope around the GEMM call of a
+ * statement that it runs for all iterations of a host loop tagged parallel.  Scopes do not nest (_begin inside a
+ * scope and _end outside one return 1); tiramisu_hip_sgemm_static_scratch and tiramisu_hip_dgemm are not gathered. */
+int tiramisu_hip_batch_begin(void);
+int tiramisu_hip_batch_end(void);
+
 /* The scratch block that deep reductions of tiramisu_hip_sgemm use on the calling thread's current stream (partial
  * tiles and per-tile counters), or NULL before the first such call: one block per (host thread, stream), so that
  * calls of one thread on two streams may overlap.  No counterpart in the reference; for tests and diagnostics. */

@@ -9,14 +9,18 @@
 //   out(i, j)     = sum over p of s2(p, i, j)             one kernel after the loop
 // More iterations (6) than pool threads; what runs before the loop must be complete when the first
 // iteration starts, the two kernels of an iteration must stay in order, and the last kernel
-// must see every iteration's result.  Generated twice: parallel_host_loop, and
+// must see every iteration's result.  Generated three times: parallel_host_loop (the pool: the distribution of
+// the loop over its statements is switched off through a back-end option), parallel_host_loop_distributed (what the
+// back-end does when left alone: each of the two kernels once, with the six iterations as gridDim.z), and
 // parallel_host_loop_serial with the tag ignored.
 #include <cstdlib>
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
 
-static void generate(const std::string &name, bool threaded)
+enum how_t { pool, distributed, serial };
+
+static void generate(const std::string &name, how_t how)
 {
     const int P = 6, N = 256;
     tiramisu::init(name);
@@ -53,14 +57,15 @@ static void generate(const std::string &name, bool threaded)
     s1.tag_parallel_level(p);
     base.then(s1, computation::root).then(s2, p).then(out_init, computation::root).then(out, jt);
 
-    if (!threaded) setenv("TIRAMISU_HIP_SERIAL_HOST_LOOPS", "1", 1);
+    if (how == serial) tiramisu::set_backend_option("hip_serial_host_loops", "1");
+    if (how == pool) tiramisu::set_backend_option("hip_no_distributed_host_loops", "1");
     tiramisu::codegen({&b_in, &b_out}, "build/" + name + ".o", true);
-    if (!threaded) unsetenv("TIRAMISU_HIP_SERIAL_HOST_LOOPS");
 }
 
 int main()
 {
-    generate("parallel_host_loop", true);
-    generate("parallel_host_loop_serial", false);
+    generate("parallel_host_loop", pool);
+    generate("parallel_host_loop_distributed", distributed);
+    generate("parallel_host_loop_serial", serial);
     return 0;
 }

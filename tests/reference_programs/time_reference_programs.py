@@ -2,7 +2,8 @@
 (build_reference_programs.py) on the GPU of this machine, at the sizes their own wrappers use:
 the eight image pipelines of benchmarks/halide on a 2112 x 3520 image (the size of the tree's
 utils/images; heat2dgpu on its wrapper's 10000 x 10000 grid, edgegpu on the 8192 x 8192 x 3 it is
-written for), the three tuned sgemm schedules, chain_mm and the three baryon correlators (through their own wrappers).  The programs copy to and from the GPU
+written for), the three tuned sgemm schedules, chain_mm, the library LSTM (configuration 5's shape) and the three baryon
+correlators (through their own wrappers).  The programs copy to and from the GPU
 themselves; what is timed is their kernels: HIP events around every launch of a call
 (tiramisu_hip_profile_*), median over the calls.  Bytes are the algorithmic ones: every input and
 output element once.  Prints one markdown table.  Run from the repository root on a machine with a
@@ -148,6 +149,31 @@ def correlator_programs(only):
     return out
 
 
+def lstm_program(only):
+    """benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp, unchanged: 4 layers, batch 64, 512 features, 100 steps.  The
+    program times itself between its device copies (get_time(), timer_hook.c); the kernels of the same call by HIP
+    events (events between the launches of a dependent chain cost a good part of a launch themselves, so their sum
+    is above the program's own figure)."""
+    name = "lstm_gpu_lib"
+    if (only and name not in only) or not os.path.exists(library(name)):
+        return []
+    ctypes.CDLL(library("get_time"), mode=ctypes.RTLD_GLOBAL)
+    L, B, H, S = 4, 64, 512, 100
+    rng = np.random.RandomState(5)
+    weights = rng.uniform(-0.08, 0.08, (L, 2, 4 * H, H)).astype(np.float32)
+    biases = rng.uniform(-0.08, 0.08, (L, 4 * H)).astype(np.float32)
+    x = rng.uniform(-1, 1, (S, B, H)).astype(np.float32)
+    program = runtime.Program(library(name), "lstm")
+    y, t0, t1 = np.zeros((S, B, H), np.float32), np.zeros(1, np.float32), np.zeros(1, np.float32)
+    own = []
+    for _ in range(CALLS + 1):
+        program(weights, biases, x, y, t0, t1)
+        own.append(float(t1[0] - t0[0]))
+    total, by = kernel_times(lambda: program(weights, biases, x, y, t0, t1))
+    return [(name, "4-layer LSTM, batch 64, 512 features, 100 steps: library GEMMs + one point-wise kernel per step", sorted(own[1:])[CALLS // 2], total, by,
+             L * S * 2 * (2.0 * B * 4 * H * H))]
+
+
 def main():
     only = set(sys.argv[1:])
     runtime.wrappers()
@@ -165,6 +191,11 @@ def main():
         kernels = ", ".join("%s %.3f ms" % (k, t / n) for k, (t, n) in sorted(by.items()))
         tf = flop / (total * 1e-3) / 1e12
         print("| %s | %s | %s | %.3f ms | %.1f TFLOP/s | %.2f of %.1f TFLOP/s |" % (name, note, kernels, total, tf, tf / FP32_MFMA_PEAK_TFLOPS, FP32_MFMA_PEAK_TFLOPS), flush=True)
+    for name, note, own_ms, total, by, flop in lstm_program(only):
+        kernels = ", ".join("%s %.1f us x %d" % (k, t / n * 1e3, n) for k, (t, n) in sorted(by.items()))
+        tf = flop / (own_ms * 1e-3) / 1e12
+        print("| `%s` | %s | %s (sum between events %.3f ms) | %.3f ms between the program's own timers | %.1f TFLOP/s | %.2f of %.1f TFLOP/s |"
+              % (name, note, kernels, total, own_ms, tf, tf / FP32_MFMA_PEAK_TFLOPS, FP32_MFMA_PEAK_TFLOPS), flush=True)
 
 
 if __name__ == "__main__":

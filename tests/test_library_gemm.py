@@ -172,3 +172,30 @@ def test_deep_reductions_on_two_streams_of_one_thread_use_separate_scratch():
             d.free()
     for s in streams:
         w.tiramisu_hip_stream_destroy(s)
+
+
+def test_calls_gathered_in_a_batch_scope_give_the_results_of_separate_calls():
+    """tiramisu_hip_batch_begin / _end: four recurrent-cell products of one shape (one launch, a problem per
+    blockIdx.z), then a product of another shape and one that takes the element-per-thread kernel (launched one by
+    one), all exact on small integers; nothing is written before _end."""
+    from gpu_util import DeviceArray
+    w = runtime.wrappers()
+    rng = np.random.RandomState(45)
+    shapes = [(64, 2048, 512)] * 4 + [(640, 256, 128), (16, 16, 4)]
+    jobs = []
+    for M, N, K in shapes:
+        A = rng.randint(-3, 4, (M, K)).astype(np.float32)
+        B = rng.randint(-3, 4, (K, N)).astype(np.float32)
+        C = rng.randint(-3, 4, (M, N)).astype(np.float32)
+        jobs.append((A, B, C, DeviceArray(A), DeviceArray(B), DeviceArray(C)))
+    assert w.tiramisu_hip_batch_end() == 1                     # no scope open
+    assert w.tiramisu_hip_batch_begin() == 0
+    assert w.tiramisu_hip_batch_begin() == 1                   # scopes do not nest
+    for (M, N, K), (A, B, C, dA, dB, dC) in zip(shapes, jobs):
+        assert w.tiramisu_hip_sgemm(dA.ptr, dB.ptr, dC.ptr, M, N, K, 1.0, 1.0, 0, 0, 0, 0, 0, 0, False, False) == 0
+    assert np.array_equal(jobs[0][5].download(), jobs[0][2])   # gathered, not launched
+    assert w.tiramisu_hip_batch_end() == 0
+    for A, B, C, dA, dB, dC in jobs:
+        assert np.array_equal(dC.download(), (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float32))
+        for d in (dA, dB, dC):
+            d.free()

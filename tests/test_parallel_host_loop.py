@@ -1,7 +1,8 @@
-"""Host loops tagged parallel around GPU kernels (tests/programs/parallel_host_loop.cpp): the HIP
-back-end hands the loop body to tiramisu_hip_parallel_for, whose pool threads launch on streams
-of their own.  Exact arithmetic (small integers), compared with numpy and with the same program
-generated with a serial loop."""
+"""Host loops tagged parallel around GPU kernels (tests/programs/parallel_host_loop.cpp).  Left alone, the HIP
+back-end distributes such a loop over its statements: every kernel once with the iterations as gridDim.z, library
+GEMM calls of a statement gathered into one batched launch (tiramisu_hip_batch_begin / _end).  With that switched
+off it hands the loop body to tiramisu_hip_parallel_for, whose pool threads launch on streams of their own.
+Exact arithmetic (small integers), compared with numpy and with the same program generated with a serial loop."""
 import os
 
 import numpy as np
@@ -17,6 +18,17 @@ def test_loop_is_handed_to_the_pool(programs_dir):
     assert "tiramisu_hip_parallel_for" not in serial
 
 
+def test_loop_is_distributed_over_its_kernels(programs_dir):
+    host = open(os.path.join(programs_dir, "build", "parallel_host_loop_distributed.o.host.cpp")).read()
+    device = open(os.path.join(programs_dir, "build", "parallel_host_loop_distributed.o.hip")).read()
+    assert "tiramisu_hip_parallel_for" not in host and "distributed over its statements" in host
+    assert host.count("const int32_t _batch_first = 0;") == 2                 # the two kernels of the body, once each
+    assert device.count("= (int32_t)blockIdx.z + _batch_first;") == 2
+    import json
+    m = json.load(open(os.path.join(programs_dir, "build", "parallel_host_loop.o.json")))
+    assert {"name": "hip_no_distributed_host_loops", "value": "1", "from": "program"} in m["options"]
+
+
 @pytest.mark.gpu
 def test_parallel_iterations_match_numpy_and_the_serial_loop(programs_dir):
     from gpu_util import DeviceArray
@@ -29,7 +41,7 @@ def test_parallel_iterations_match_numpy_and_the_serial_loop(programs_dir):
         s1 = base * (p + 1)
         expected += s1 + s1[::-1]
     outs = {}
-    for name in ("parallel_host_loop", "parallel_host_loop_serial"):
+    for name in ("parallel_host_loop", "parallel_host_loop_distributed", "parallel_host_loop_serial"):
         program = runtime.load(programs_dir, name)
         for repeat in range(3):                      # the pool is reused from call to call
             d_in, d_out = DeviceArray(src), DeviceArray(np.full((N, N), -1, np.float32))

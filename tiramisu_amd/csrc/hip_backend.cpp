@@ -724,7 +724,22 @@ std::string max_text(const std::vector<expr> &v, const c_printer &host) {
 
 }  // namespace
 
+static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const fusion_request *batch, bool &batch_ok);
+
 kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
+    bool ok = true;
+    return emit_generic_kernel_impl(ctx, root, nullptr, ok);
+}
+
+kernel emit_generic_kernel_batched(context &ctx, const node_ptr &root, const fusion_request &batch, bool &ok) {
+    const int first_id = context::peek_next_kernel_id();
+    ok = true;
+    kernel k = emit_generic_kernel_impl(ctx, root, &batch, ok);
+    if (!ok) context::set_next_kernel_id(first_id);
+    return k;
+}
+
+static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const fusion_request *batch, bool &batch_ok) {
     generic_kernel_gen g(ctx);
     g.prepass(root);
     g.emit(root, 1);
@@ -754,8 +769,20 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
         k.block[d] = max_text(g.block_ext[d], host);
     }
     std::vector<std::string> top_decls;
+    bool batch_iterator_used = false;
+    if (batch) {
+        // the nest's own grid must leave z free and must not depend on the iteration
+        if (k.grid[2] != "1" || extent_scalars.count(batch->batch_iterator)) { batch_ok = false; return k; }
+        k.how += ", iterations of the parallel host loop as gridDim.z";
+        c_printer hp;
+        hp.fct = f;
+        k.batch_first = hp.print(batch->batch_first);
+        k.grid[2] = "((" + hp.print(batch->batch_last) + ") >= _batch_first ? (" + hp.print(batch->batch_last) + ") - _batch_first + 1 : 0)";
+        k.params.push_back({false, "_batch_first", global::get_loop_iterator_data_type()});
+    }
     for (auto &nm : g.used_scalars) {
         if (g.inner.count(nm)) continue;
+        if (batch && nm == batch->batch_iterator) { batch_iterator_used = true; continue; }
         primitive_t t = global::get_loop_iterator_data_type();
         for (auto c : f->get_invariants())
             if (c->get_name() == nm) t = c->get_data_type();
@@ -808,6 +835,8 @@ kernel emit_generic_kernel(context &ctx, const node_ptr &root) {
         else os << "const " << primitive_c_name(p.type) << " " << p.name;
     }
     os << ")\n{\n";
+    if (batch && batch_iterator_used)
+        os << "    const " << primitive_c_name(global::get_loop_iterator_data_type()) << " " << batch->batch_iterator << " = (int32_t)blockIdx.z + _batch_first;\n";
     for (auto &d : top_decls) os << "    " << d << "\n";
     if (g.needs_reduction_scratch) os << "    __shared__ float _reduction_scratch[16];\n";
     if (g.fast_block_dim >= 0) {
@@ -840,6 +869,7 @@ std::string launch_text(const kernel &k, const std::string &ind_outer) {
         }
     }
     os << ind << "{\n";
+    if (!k.batch_first.empty()) os << ind << "    const int32_t _batch_first = " << k.batch_first << ";\n";
     os << ind << "    void *_args[] = {";
     for (size_t i = 0; i < k.params.size(); i++) os << (i ? ", " : "") << "(void *)&" << k.params[i].name;
     if (k.params.empty()) os << "nullptr";
@@ -942,6 +972,7 @@ struct host_gen {
                     break;
                 }
                 if (runs_in_parallel(n) && emit_batched(n, ind)) break;
+                if (runs_in_parallel(n) && emit_distributed(n, ind)) break;
                 if (runs_in_parallel(n)) {
                     // iterations on pool threads, each with a stream of its own (what the reference's
                     // Halide parallel loop around kernel calls does: tiramisu_codegen_halide.cpp:2104-2145)
@@ -1035,6 +1066,105 @@ struct host_gen {
             return false;
         }
         for (auto &p : plans) take(p, ind);
+        return true;
+    }
+
+    // A host loop tagged parallel whose body is a sequence of library GEMM calls, kernels and serial loops around
+    // them (the reference's library LSTM: per layer one batched input product, then per time step a recurrent
+    // product and a point-wise kernel) is distributed over its statements: every statement runs for all
+    // iterations of the parallel loop at once -- a kernel as one launch with the iterations as gridDim.z, GEMM
+    // calls of one statement as one batched launch (tiramisu_hip_batch_begin / _end) -- in the order of the body,
+    // on the calling thread's stream.  The tag asserts that iterations are independent, and the order of the
+    // statements within an iteration is kept, so every dependence of the serial program holds; what it buys is
+    // launches that fill the chip instead of one small launch per iteration on streams that slow each other
+    // down.  Serial loops inside the body must not have bounds that involve the parallel iterator.
+    bool distributable(const node_ptr &x, const std::string &it, int &gpu_statements) const {
+        if (!x) return true;
+        switch (x->kind) {
+        case node_kind::block:
+            for (auto &c : x->children)
+                if (!distributable(c, it, gpu_statements)) return false;
+            return true;
+        case node_kind::cond: return false;
+        case node_kind::loop: {
+            if (is_gpu_loop(x)) {
+                bool z_used = false;
+                lir::walk(x, [&](const node_ptr &y) { if (y->kind == node_kind::loop && y->gpu_block == 2) z_used = true; });
+                gpu_statements++;
+                return !z_used;
+            }
+            if (x->parallel) return false;
+            for (const expr &e : {x->init, x->upper, x->increment})
+                if (e.is_defined() && lir::mentions(e, it)) return false;
+            return distributable(x->body, it, gpu_statements);
+        }
+        case node_kind::leaf:
+            if (x->lkind == leaf_kind::allocate || x->lkind == leaf_kind::release || x->lkind == leaf_kind::let || x->lkind == leaf_kind::copy) return false;
+            if (is_library_gemm(x)) gpu_statements++;
+            return true;
+        }
+        return false;
+    }
+    static bool is_library_gemm(const node_ptr &x) {
+        bool gemm = false;
+        if (x->kind == node_kind::leaf && x->rhs.is_defined())
+            x->rhs.visit([&](const expr &e) {
+                if (e.get_expr_type() == e_op && e.get_op_type() == o_call && (e.get_name() == "tiramisu_hip_sgemm" || e.get_name() == "tiramisu_hip_dgemm")) gemm = true;
+            });
+        return gemm;
+    }
+    void emit_for_all_iterations(const node_ptr &x, const node_ptr &par, int ind) {
+        switch (x->kind) {
+        case node_kind::block:
+            for (auto &c : x->children) emit_for_all_iterations(c, par, ind);
+            return;
+        case node_kind::loop:
+            if (is_gpu_loop(x)) {
+                fusion_request req;
+                req.batch_iterator = par->iterator;
+                req.batch_first = par->init;
+                req.batch_last = par->upper;
+                ctx.host_iterators.push_back(par->iterator);
+                launch_plan plan;
+                if (emit_contraction(ctx, x, plan, &req)) {
+                    take(plan, ind);
+                } else {
+                    bool ok = true;
+                    kernel k = emit_generic_kernel_batched(ctx, x, req, ok);
+                    if (!ok) ERROR("a kernel inside a distributed parallel host loop could not take the loop's iterations as gridDim.z", true);
+                    ctx.kernels.push_back(k);
+                    out << launch_text(k, pad(ind));
+                }
+                ctx.host_iterators.pop_back();
+                return;
+            }
+            out << pad(ind) << "for (int32_t " << x->iterator << " = " << hp.print(x->init) << "; " << x->iterator
+                << " <= " << hp.print(x->upper) << "; " << x->iterator << " += " << hp.print(x->increment) << ") {\n";
+            ctx.host_iterators.push_back(x->iterator);
+            emit_for_all_iterations(x->body, par, ind + 1);
+            ctx.host_iterators.pop_back();
+            out << pad(ind) << "}\n";
+            return;
+        case node_kind::leaf: {
+            const bool gemm = is_library_gemm(x);
+            if (gemm) out << pad(ind) << "tiramisu_hip_batch_begin();\n";
+            out << pad(ind) << "for (int32_t " << par->iterator << " = " << hp.print(par->init) << "; " << par->iterator
+                << " <= " << hp.print(par->upper) << "; " << par->iterator << " += 1) {\n";
+            emit_leaf(x, ind + 1);
+            out << pad(ind) << "}\n";
+            if (gemm) out << pad(ind) << "tiramisu_hip_batch_end();\n";
+            return;
+        }
+        default: return;
+        }
+    }
+    bool emit_distributed(const node_ptr &n, int ind) {
+        if (backend_option("TIRAMISU_HIP_NO_DISTRIBUTED_HOST_LOOPS")) return false;
+        int gpu_statements = 0;
+        if (!n->body || !distributable(n->body, n->iterator, gpu_statements) || gpu_statements == 0) return false;
+        out << pad(ind) << "{   // parallel host loop " << n->iterator << ", distributed over its statements\n";
+        emit_for_all_iterations(n->body, n, ind + 1);
+        out << pad(ind) << "}\n";
         return true;
     }
 

@@ -31,6 +31,7 @@ struct kernel {
     std::string grid[3] = {"1", "1", "1"};
     std::string block[3] = {"1", "1", "1"};
     std::string lds_bytes = "0";
+    std::string batch_first;            // not empty: the launch site declares `_batch_first` with this value (a parameter)
     std::string how;                    // "generic", "mfma-contraction", "stencil", ...
     /** Host buffers that the kernel names (only with implicit copies): the launch site gives it
       * device copies of them, copied in before the launch and, when written, back after it. */
@@ -77,6 +78,11 @@ struct fusion_request {
 /** Schedule-faithful kernel: one thread per (block-iterator, thread-iterator) point, untagged
   * inner loops serial in the thread (reference: tiramisu_codegen_cuda.cpp:239-326, :549-707). */
 kernel emit_generic_kernel(context &ctx, const lir::node_ptr &root);
+/** The same with the iterations of a host loop tagged parallel around the nest as gridDim.z of one launch: the
+  * kernel recomputes the loop's iterator from blockIdx.z (fusion_request's batch_* fields; its consumer is not
+  * used).  \p ok is false, and nothing is kept, when the nest's own grid already uses z or its extents involve the
+  * iterator. */
+kernel emit_generic_kernel_batched(context &ctx, const lir::node_ptr &root, const fusion_request &batch, bool &ok);
 
 /** Pattern-directed emitters.  Each returns false when the nest is not provably of its kind, in
   * which case the generic emitter is used. */

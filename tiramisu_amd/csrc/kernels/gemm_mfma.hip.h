@@ -519,5 +519,25 @@ __global__ void __launch_bounds__(CFG::NT) sgemm_kernel(const float *__restrict_
                        axpby_store{C, ldc});
 }
 
+// Up to eight problems of one shape in one launch: blockIdx.z picks the operands.
+constexpr int BATCH_MAX = 8;
+struct sgemm_batch {
+    const float *A[BATCH_MAX];
+    const float *B[BATCH_MAX];
+    float *C[BATCH_MAX];
+};
+
+template <class CFG>
+__global__ void __launch_bounds__(CFG::NT) sgemm_batched_kernel(const sgemm_batch batch, int M, int N, int K, long lda, long ldb,
+                                                                 long ldc, float alpha, float beta, int vec_ok) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    int tm, tn;
+    tile_of_block((M + CFG::BM - 1) / CFG::BM, (N + CFG::BN - 1) / CFG::BN, tm, tn);
+    const float *A = batch.A[blockIdx.z], *B = batch.B[blockIdx.z];
+    float *C = batch.C[blockIdx.z];
+    tile_mainloop<CFG>(A, lda, B, ldb, M, N, K, tm * CFG::BM, tn * CFG::BN, vec_ok != 0, lds, axpby_value{C, ldc, alpha, beta},
+                       axpby_store{C, ldc});
+}
+
 }  // namespace tgemm
 #endif
