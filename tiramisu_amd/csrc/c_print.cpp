@@ -82,6 +82,8 @@ std::string c_printer::store(const buffer *b, const std::vector<expr> &index, co
     primitive_t bt = b->get_elements_type();
     if (bt == p_bfloat16) v = "t_f32_to_bf16(" + v + ")";
     else if (bt != value_type && value_type != p_none) v = "(" + primitive_c_name(bt) + ")(" + v + ")";
+    if (device && streaming_stores && streaming_stores->count(b->get_name()))
+        return "__builtin_nontemporal_store((" + primitive_c_name(bt == p_bfloat16 ? p_uint16 : bt) + ")(" + v + "), &" + element(b, index) + ");";
     return element(b, index) + " = " + v + ";";
 }
 

@@ -22,6 +22,8 @@ struct c_printer {
     /** Records every buffer and free variable printed (for kernel parameter discovery). */
     std::set<std::string> *used_buffers = nullptr;
     std::set<std::string> *used_scalars = nullptr;
+    /** Device code: buffers whose stores carry the non-temporal hint (written and never read by the kernel). */
+    const std::set<std::string> *streaming_stores = nullptr;
 
     std::string print(const expr &e) const;
     /** "buf[linear index]" or the bare name for register buffers. */

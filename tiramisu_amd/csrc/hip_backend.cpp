@@ -66,7 +66,31 @@ struct generic_kernel_gen {
         dev.used_scalars = &used_scalars;
     }
 
+    std::set<std::string> streamed;      // global buffers that the kernel writes and never reads
+    void find_streaming_stores(const node_ptr &root) {
+        const char *o = backend_option("TIRAMISU_HIP_STREAMING_STORES");
+        if (!o || std::string(o) == "0") return;
+        std::set<std::string> written, read;
+        lir::walk(root, [&](const node_ptr &n) {
+            if (n->kind != node_kind::leaf) return;
+            if (n->lhs && n->lhs->get_location() == memory_location::global) written.insert(n->lhs->get_name());
+            auto scan = [&](const expr &e) {
+                if (e.is_defined()) e.visit([&](const expr &x) { if (x.get_expr_type() == e_op && (x.get_op_type() == o_access || x.get_op_type() == o_address_of || x.get_op_type() == o_buffer)) read.insert(x.get_name()); });
+            };
+            scan(n->rhs);
+            scan(n->predicate);
+            for (auto &l : n->lets) scan(l.second);
+            for (auto &ix : n->lhs_index) scan(ix);
+            if (n->copy_from) read.insert(n->copy_from->get_name());
+            if (n->copy_to) read.insert(n->copy_to->get_name());
+        });
+        for (auto &w : written)
+            if (!read.count(w)) streamed.insert(w);
+        dev.streaming_stores = &streamed;
+    }
+
     void prepass(const node_ptr &root) {
+        find_streaming_stores(root);
         lir::walk(root, [&](const node_ptr &n) {
             if (n->kind == node_kind::loop) {
                 inner.insert(n->iterator);
