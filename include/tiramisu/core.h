@@ -33,6 +33,7 @@ class computation;
 class buffer;
 class constant;
 class input;
+class view;
 class block;
 namespace lir { struct program; }
 
@@ -666,6 +667,13 @@ public:
     input(std::vector<var> iterator_variables, primitive_t t);
     input(std::string name, std::vector<std::string> dimension_names,
           std::vector<expr> dimension_sizes, primitive_t t);
+};
+
+/** A named window on a buffer: indexed like a computation, computes nothing and is not scheduled; map it with
+  * store_in() to read (or name) what other computations stored there (reference: core.h:5159-5203). */
+class view : public computation {
+public:
+    view(std::string name, std::vector<var> iterator_variables, primitive_t t);
 };
 
 class Input : public input {

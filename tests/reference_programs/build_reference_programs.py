@@ -177,6 +177,33 @@ def build_lstm_naive():
     build._run(["g++", "-shared", "-fopenmp", "-o", library("lstm_ref"), os.path.join(work, "lstm_ref.o")])
 
 
+# The reference's tuned CPU schedules of two benchmark configurations, unchanged, through the oracle's CPU emitter:
+#  * benchmarks/linear_algebra/blas/level3/sgemm/cpu/sgemm_generator.cpp (packed B, three-level tiling, separated
+#    partial tiles; sizes at run time);
+#  * benchmarks/DNN/layers/convolution/direct/cpu/conv_layer_generator_tiramisu.cpp (blocked layouts, a register tile
+#    named through a tiramisu::view; its configure.h uses std::sort without <algorithm>, which is forced in here).
+#    Its register tile is one temporary buffer shared by the iterations of its parallel loops -- the reference counts
+#    on LLVM keeping it in registers -- so the generated code is only right on one thread.
+CPU_BENCHMARKS = [("benchmarks/linear_algebra/blas/level3/sgemm/cpu/sgemm_generator.cpp", "sgemm_cpu_tuned", "generated_sgemm.o", ["-I" + os.path.join(REFERENCE, "benchmarks")]),
+                  ("benchmarks/DNN/layers/convolution/direct/cpu/conv_layer_generator_tiramisu.cpp", "conv_cpu_tuned", "generated_conv_layer.o", ["-include", "algorithm"])]
+
+
+def build_cpu_benchmark(rel, stem, obj, extra):
+    from oracle import build as oracle_build
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, stem)
+    os.makedirs(work, exist_ok=True)
+    src = os.path.join(REFERENCE, rel)
+    gen = os.path.join(work, "gen")
+    cpu_dir = os.path.dirname(oracle_build.CPU_BACKEND)
+    build._run(["g++", "-std=c++17", "-O1"] + extra + ["-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
+                "-I" + os.path.dirname(src), "-o", gen, src,
+                "-L" + build.PKG, "-ltiramisu", "-Wl,--no-as-needed", "-L" + cpu_dir, "-ltiramisu_cpu_backend", "-Wl,--as-needed",
+                "-Wl,-rpath," + build.PKG, "-Wl,-rpath," + cpu_dir])
+    build._run([gen], cwd=work)
+    build._run(["g++", "-shared", "-fopenmp", "-o", library(stem), os.path.join(work, obj)])
+
+
 # The reference's own test-suite (tests/test_N.cpp + wrapper_test_N.cpp, both unchanged) through this
 # front-end and the oracle's CPU emitter (GPU tests among them with TIRAMISU_FORCE_ARCH=cpu): each wrapper
 # fills its inputs, calls the generated function and compares with the expectation its authors wrote.
@@ -279,6 +306,10 @@ def build_all(verbose=False):
     if verbose:
         print("[reference programs]", LSTM_NAIVE, "(CPU)", flush=True)
     build_lstm_naive()
+    for rel, stem, obj, extra in CPU_BENCHMARKS:
+        if verbose:
+            print("[reference programs]", rel, "(CPU)", flush=True)
+        build_cpu_benchmark(rel, stem, obj, extra)
     build_suite(verbose)
     return True
 

@@ -1958,6 +1958,13 @@ input::input(std::string nm, std::vector<var> iterator_variables, primitive_t t)
 
 input::input(std::vector<var> iterator_variables, primitive_t t) : input(fresh_input_name(), iterator_variables, t) {}
 
+view::view(std::string nm, std::vector<var> iterator_variables, primitive_t t) {
+    fct = global::get_implicit_function();
+    if (!fct) ERROR("call tiramisu::init() first", true);
+    declared_vars = iterator_variables;
+    init_computation(construct_iteration_domain(nm, iterator_variables), fct, expr(), false, t);
+}
+
 static std::vector<var> vars_from_names_sizes(const std::vector<std::string> &names, const std::vector<expr> &sizes) {
     if (names.size() != sizes.size()) ERROR("input: as many dimension names as sizes are needed", true);
     std::vector<var> v;
