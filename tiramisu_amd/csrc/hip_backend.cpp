@@ -109,6 +109,230 @@ struct generic_kernel_gen {
             std::vector<node_ptr> stack;
             find_reductions(root, stack);
         }
+        check_shared_memory(root);
+    }
+
+    // ---- the race check of LDS (option hip_check_shared_memory: "1" stops code generation at a finding, "warn"
+    // prints it and goes on).  The reference leaves barriers to the program (tiramisu_codegen_cuda.cpp:1240-1242)
+    // and this emitter drops barriers that it takes to be redundant, so the check looks at the kernel as it will be
+    // emitted.  Between two barriers every thread of the workgroup may be anywhere, so two accesses of that region
+    // to one element of a shared buffer, one of them a write, must come from one thread.  The check finds who
+    // touches what by evaluation: for every access it runs through all values of the thread loops and of the serial
+    // loops without a barrier around it (their iterations all lie in one region) and notes the thread of each
+    // element.  Serial loops with a barrier inside are walked for three consecutive values of their iterator, with
+    // what one iteration leaves pending meeting the next; block iterators take their first value (workgroups do not
+    // share LDS); conditions and predicates that evaluate to false exclude the access.  An access whose index or
+    // loop bounds do not evaluate (a size known only at run time) is reported as not analysed and stops nothing.
+    struct shared_access {
+        std::string buffer, text, who, key;
+        bool write = false, known = true;
+        std::map<long, long> owner;       // element -> thread, or -2: several threads
+    };
+    static bool evaluate(const expr &e, const std::map<std::string, long> &env, long &out) {
+        if (!e.is_defined()) return false;
+        if (e.get_expr_type() == e_val) {
+            if (e.get_data_type() == p_float32 || e.get_data_type() == p_float64) return false;
+            out = (long)e.get_int_val();
+            return true;
+        }
+        if (e.get_expr_type() == e_var) {
+            auto it = env.find(e.get_name());
+            if (it == env.end()) return false;
+            out = it->second;
+            return true;
+        }
+        if (e.get_expr_type() != e_op) return false;
+        long a = 0, b = 0, c = 0;
+        const op_t op = e.get_op_type();
+        if (op == o_access || op == o_call || op == o_address_of || op == o_lin_index || op == o_buffer) return false;
+        const int n = e.get_n_arg();
+        if (n >= 1 && !evaluate(e.get_operand(0), env, a)) return false;
+        if (op == o_select || op == o_cond) {           // only the branch taken must evaluate
+            return n == 3 && evaluate(e.get_operand(a ? 1 : 2), env, out);
+        }
+        if (n >= 2 && !evaluate(e.get_operand(1), env, b)) return false;
+        if (n >= 3 && !evaluate(e.get_operand(2), env, c)) return false;
+        switch (op) {
+        case o_minus: out = -a; return true;
+        case o_cast: out = a; return e.get_data_type() != p_float32 && e.get_data_type() != p_float64;
+        case o_add: out = a + b; return true;
+        case o_sub: out = a - b; return true;
+        case o_mul: out = a * b; return true;
+        case o_div: if (!b) return false; out = a / b; return true;
+        case o_mod: if (!b) return false; out = a % b; return true;
+        case o_floordiv: if (!b) return false; out = a / b - ((a % b != 0) && ((a < 0) != (b < 0))); return true;
+        case o_floormod: if (!b) return false; out = ((a % b) + b) % b; return true;
+        case o_logical_and: out = a && b; return true;
+        case o_logical_or: out = a || b; return true;
+        case o_logical_not: out = !a; return true;
+        case o_eq: out = a == b; return true;
+        case o_ne: out = a != b; return true;
+        case o_le: out = a <= b; return true;
+        case o_lt: out = a < b; return true;
+        case o_ge: out = a >= b; return true;
+        case o_gt: out = a > b; return true;
+        case o_max: out = std::max(a, b); return true;
+        case o_min: out = std::min(a, b); return true;
+        case o_right_shift: out = a >> b; return true;
+        case o_left_shift: out = a << b; return true;
+        default: return false;
+        }
+    }
+    static bool contains_sync(const node_ptr &n) {
+        bool found = false;
+        lir::walk(n, [&](const node_ptr &x) { if (is_sync(x)) found = true; });
+        return found;
+    }
+    void check_shared_memory(const node_ptr &root) {
+        const char *mode = backend_option("TIRAMISU_HIP_CHECK_SHARED_MEMORY");
+        if (!mode || std::string(mode) == "0") return;
+        std::vector<shared_access> pending;
+        std::vector<std::string> findings, unanalysed;
+        std::map<std::string, long> env;                          // iterators with one value at a time
+        std::vector<node_ptr> run_through;                        // thread loops and barrier-free serial loops around the statement
+        std::vector<std::pair<expr, bool>> conditions;            // conditions around the statement and the truth value that leads to it
+        c_printer pr;
+        pr.fct = f;
+        pr.device = true;
+        auto note = [](std::vector<std::string> &list, const std::string &line) {
+            if (std::find(list.begin(), list.end(), line) == list.end()) list.push_back(line);
+        };
+        auto thread_name = [](long t) {
+            if (t == -2) return std::string("several threads");
+            std::string s;
+            for (int d = 2; d >= 0; d--) s += (s.empty() ? "" : ",") + std::to_string((t >> (12 * d)) & 4095);
+            return "thread (z,y,x) = (" + s + ")";
+        };
+        // who touches which element: all values of the loops of run_through, innermost last
+        auto owners = [&](shared_access &acc, const buffer *b, const std::vector<expr> &index, const node_ptr &leaf) {
+            const expr element = lir::simplify(lir::linearize(b, index));
+            long budget = 1L << 22;
+            std::map<std::string, long> at = env;
+            std::function<void(size_t, long)> level = [&](size_t d, long thread) {
+                if (!acc.known) return;
+                if (d == run_through.size()) {
+                    if (--budget < 0) { acc.known = false; return; }
+                    long v = 0;
+                    for (auto &c : conditions) {
+                        if (!evaluate(c.first, at, v)) continue;                // unknown: taken to hold
+                        if ((v != 0) != c.second) return;
+                    }
+                    for (auto &l : leaf->lets) { if (evaluate(l.second, at, v)) at[l.first] = v; else at.erase(l.first); }
+                    if (leaf->predicate.is_defined() && evaluate(leaf->predicate, at, v) && !v) return;
+                    if (!evaluate(element, at, v)) { acc.known = false; return; }
+                    auto it = acc.owner.find(v);
+                    if (it == acc.owner.end()) acc.owner[v] = thread;
+                    else if (it->second != thread) it->second = -2;
+                    return;
+                }
+                const node_ptr &l = run_through[d];
+                long first = 0, last = 0, step = 1;
+                if (!evaluate(l->init, at, first) || !evaluate(l->upper, at, last) ||
+                    (l->increment.is_defined() && !evaluate(l->increment, at, step)) || step <= 0) { acc.known = false; return; }
+                for (long v = first; v <= last && acc.known; v += step) {
+                    at[l->iterator] = v;
+                    level(d + 1, l->gpu_thread >= 0 ? thread | ((v & 4095) << (12 * l->gpu_thread)) : thread);
+                }
+                at.erase(l->iterator);
+            };
+            level(0, 0);
+        };
+        auto meet = [&](shared_access now) {
+            for (auto &p : pending) if (p.key == now.key) return;               // has met everything already
+            const std::string here = now.who + (now.write ? " writes " : " reads ") + now.buffer + now.text;
+            if (!now.known) note(unanalysed, here + ": the index or a loop bound around it has no value at compile time");
+            if (now.known && now.write)
+                for (auto &o : now.owner)
+                    if (o.second == -2) { note(findings, here + ": several threads write element " + std::to_string(o.first)); break; }
+            for (auto &p : pending) {
+                if (p.buffer != now.buffer || (!p.write && !now.write) || !p.known || !now.known) continue;
+                const bool p_smaller = p.owner.size() < now.owner.size();
+                const auto &small = p_smaller ? p.owner : now.owner;
+                const auto &large = p_smaller ? now.owner : p.owner;
+                for (auto &o : small) {
+                    auto it = large.find(o.first);
+                    if (it == large.end() || (it->second == o.second && o.second != -2)) continue;
+                    const long tp = p_smaller ? o.second : it->second, tn = p_smaller ? it->second : o.second;
+                    note(findings, "no sync between \"" + p.who + (p.write ? " writes " : " reads ") + p.buffer + p.text + "\" and \"" + here +
+                                   "\": element " + std::to_string(o.first) + " is touched by " + thread_name(tp) + " in the first and by " +
+                                   thread_name(tn) + " in the second");
+                    break;
+                }
+            }
+            pending.push_back(std::move(now));
+        };
+        auto access = [&](const buffer *b, const std::vector<expr> &index, bool write, const node_ptr &leaf) {
+            shared_access acc;
+            acc.buffer = b->get_name();
+            for (auto &e : index) acc.text += "[" + pr.print(lir::simplify(e)) + "]";
+            acc.who = leaf->comp ? leaf->comp->get_name() : std::string("a statement");
+            acc.write = write;
+            acc.key = acc.who + (write ? " W " : " R ") + acc.buffer + acc.text;
+            for (auto &v : env) acc.key += " " + v.first + "=" + std::to_string(v.second);
+            for (auto &p : pending) if (p.key == acc.key) return;
+            owners(acc, b, index, leaf);
+            meet(std::move(acc));
+        };
+        std::function<void(const node_ptr &)> go = [&](const node_ptr &n) {
+            if (!n) return;
+            switch (n->kind) {
+            case node_kind::block:
+                for (auto &c : without_redundant_barriers(n->children)) go(c);
+                return;
+            case node_kind::cond:
+                conditions.push_back({n->condition, true});
+                go(n->then_body);
+                conditions.back().second = false;
+                go(n->else_body);
+                conditions.pop_back();
+                return;
+            case node_kind::loop: {
+                long first = 0, last = 0, step = 1;
+                const bool bounded = evaluate(n->init, env, first) && evaluate(n->upper, env, last) &&
+                                     (!n->increment.is_defined() || evaluate(n->increment, env, step)) && step > 0;
+                if (n->gpu_block >= 0) {
+                    if (bounded) env[n->iterator] = first;
+                    go(n->body);
+                    env.erase(n->iterator);
+                } else if (n->gpu_thread >= 0 || !contains_sync(n->body)) {
+                    run_through.push_back(n);
+                    go(n->body);
+                    run_through.pop_back();
+                } else {
+                    // a barrier inside: one value at a time, what an iteration leaves pending meets the next one
+                    for (int k = 0; k < 3; k++) {
+                        if (bounded && first + k * step > last) break;
+                        if (bounded) env[n->iterator] = first + k * step;
+                        go(n->body);
+                    }
+                    env.erase(n->iterator);
+                }
+                return;
+            }
+            case node_kind::leaf: {
+                if (n->lkind == leaf_kind::sync) { pending.clear(); return; }
+                auto reads = [&](const expr &e) {
+                    if (!e.is_defined()) return;
+                    e.visit([&](const expr &x) {
+                        if (x.get_expr_type() != e_op || x.get_op_type() != o_access) return;
+                        auto it = f->get_buffers().find(x.get_name());
+                        if (it != f->get_buffers().end() && it->second->get_location() == memory_location::shared)
+                            access(it->second, x.get_access(), false, n);
+                    });
+                };
+                reads(n->rhs);
+                reads(n->predicate);
+                for (auto &l : n->lets) reads(l.second);
+                for (auto &ix : n->lhs_index) reads(ix);
+                if (n->lhs && n->lhs->get_location() == memory_location::shared) access(n->lhs, n->lhs_index, true, n);
+                return;
+            }
+            }
+        };
+        go(root);
+        for (auto &l : unanalysed) std::cerr << "LDS race check, not analysed: " << l << std::endl;
+        for (auto &l : findings) std::cerr << "LDS race check: " << l << std::endl;
+        if (!findings.empty() && std::string(mode) != "warn") ERROR("shared-memory accesses of different threads are not separated by a sync", true);
     }
 
     // ---- which thread-mapped loop runs along the lanes.  The front-end numbers the tagged thread levels from
