@@ -74,8 +74,11 @@ def kernel_source_hash(name):
     import hashlib
     import re
     text = open(os.path.join(PROGRAMS, "build", name + ".o.hip")).read()
-    h = hashlib.sha1(re.sub(r'#include "[^"]*/kernels/', '#include "kernels/', text).encode())
-    for inc in sorted(set(re.findall(r'#include "([^"]*/kernels/[^"]+)"', text))):
+    # kernel headers are included by file name (the device compiler gets their directory); the hash is taken over
+    # the text with the directory spelled "kernels/", as generated code of earlier versions named it by path
+    text = re.sub(r'#include "(?:[^"]*/kernels/)?([A-Za-z0-9_]+\.hip\.h)"', r'#include "kernels/\1"', text)
+    h = hashlib.sha1(text.encode())
+    for inc in sorted(set(re.findall(r'#include "(kernels/[^"]+)"', text))):
         path = os.path.join(ROOT, "tiramisu_amd", "csrc", "kernels", os.path.basename(inc))
         h.update(open(path, "rb").read())
     return h.hexdigest()[:12]

@@ -83,6 +83,22 @@ int tiramisu_hip_batch_end(void);
  * calls of one thread on two streams may overlap.  No counterpart in the reference; for tests and diagnostics. */
 void *tiramisu_hip_sgemm_workspace(void);
 
+/* ---- memory the library keeps between calls.  No counterpart in the reference, whose generated code allocates and
+ *      frees everything on every call. ---- */
+/* Scratch that a generated function keeps from one call to the next (the third plane of a time-tiled stencil, the
+ * hand-over area of the windowed convolution): one block per requesting site (generated code passes the address of
+ * a static of its own), host thread and stream, at least `bytes` large, allocated at the first request and handed
+ * out again at every later one.  *fresh (may be NULL) is 1 when this call allocated the block -- its contents are
+ * undefined then -- and 0 when it is the block of the call before. */
+void *tiramisu_hip_kept_scratch(const void *site, uint64_t bytes, int32_t *fresh);
+/* Waits for the device, then gives back to HIP everything the library holds without anyone using it: the kept
+ * scratch of all generated functions, the workspaces of tiramisu_hip_sgemm, the idle blocks of the pool behind
+ * tiramisu_hip_malloc.  Returns the number of bytes released.  The caller makes sure that no generated function and
+ * no GEMM call is running; later calls allocate again what they need. */
+uint64_t tiramisu_hip_release_cached_memory(void);
+/* What tiramisu_hip_release_cached_memory would release now. */
+uint64_t tiramisu_hip_cached_memory_bytes(void);
+
 /* ---- code objects and launches.  The reference links nvcc-compiled kernel wrappers
  *      (_kernel_N_wrapper, tiramisu_codegen_cuda.cpp:1288-1318) into the program; here
  *      generated host code is plain C++ that embeds a gfx950 code object and launches
@@ -127,7 +143,8 @@ int tiramisu_hip_set_stream(void *stream);
 void *tiramisu_hip_get_stream(void);
 /* A new stream that does not synchronise with the default stream (default priority), for callers that overlap
  * calls; destroy waits for the stream's work and, if it is the calling thread's current stream, restores the
- * per-thread default stream.  Scratch blocks that the runtime keeps per (thread, stream) stay allocated. */
+ * per-thread default stream.  Scratch blocks that the runtime keeps per (thread, stream) stay allocated until
+ * tiramisu_hip_release_cached_memory. */
 void *tiramisu_hip_stream_create(void);
 int tiramisu_hip_stream_destroy(void *stream);
 void *tiramisu_hip_event_create(void);

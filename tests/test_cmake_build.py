@@ -51,6 +51,35 @@ def test_cmake_runtime_exports_the_declared_abi(cmake_build):
     assert mine == exported(build.wrappers_library())       # the library build.py makes exports the same set
 
 
+def test_installed_tree_is_self_contained(cmake_build, tmp_path):
+    """cmake --install: lib/, include/ and share/tiramisu/kernels.  A generator compiled against the installed headers
+    and library alone generates a GPU function whose device code (kernel headers included by file name) was compiled
+    against the installed kernel headers, found relative to the installed library -- not through a path into this
+    source tree -- and whose host glue was compiled against the installed tiramisu_hip_wrappers.h."""
+    import json
+    bdir, _ = cmake_build
+    prefix = os.path.join(str(tmp_path), "prefix")
+    run(["cmake", "--install", bdir, "--prefix", prefix])
+    for rel in ("lib/libtiramisu.so", "lib/libtiramisu_hip_wrappers.so", "include/tiramisu/tiramisu.h",
+                "include/tiramisu_hip_wrappers.h", "share/tiramisu/kernels/gemm_mfma.hip.h",
+                "share/tiramisu/kernels/stencil2d_regs.hip.h", "share/tiramisu/kernels/wave_reduce.hip.h"):
+        assert os.path.exists(os.path.join(prefix, rel)), rel
+    work = os.path.join(str(tmp_path), "work")
+    os.makedirs(os.path.join(work, "build"))
+    gen = os.path.join(work, "gen")
+    run(["g++", "-std=c++17", "-O1", "-I" + os.path.join(prefix, "include"), "-o", gen,
+         os.path.join(ROOT, "tiramisu_amd", "programs", "sgemm.cpp"), "-L" + os.path.join(prefix, "lib"), "-ltiramisu",
+         "-Wl,-rpath," + os.path.join(prefix, "lib")])
+    env = {k: v for k, v in os.environ.items() if k not in ("TIRAMISU_AMD_KERNEL_DIR", "TIRAMISU_AMD_INCLUDE")}
+    subprocess.run([gen], cwd=work, env=env, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    manifest = json.load(open(os.path.join(work, "build", "sgemm_1024x1024x1024.o.json")))
+    assert os.path.realpath(manifest["kernel_headers"]) == os.path.realpath(os.path.join(prefix, "share", "tiramisu", "kernels"))
+    text = open(os.path.join(work, "build", "sgemm_1024x1024x1024.o.hip")).read()
+    assert '#include "gemm_mfma.hip.h"' in text
+    assert ROOT not in text                    # no path into the source tree in the generated device code
+    assert os.path.getsize(os.path.join(work, "build", "sgemm_1024x1024x1024.o.hsaco")) > 0
+
+
 def test_reference_gpu_tests_are_registered_with_the_hip_label(cmake_build):
     bdir, with_tests = cmake_build
     if not with_tests:

@@ -722,7 +722,7 @@ struct generic_kernel_gen {
         body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << ") "
              << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, p_float32) << "\n";
         body << pad(ind) << "}\n";
-        add_include_once(ctx, "#include \"" + kernel_dir() + "/wave_reduce.hip.h\"");
+        add_include_once(ctx, "#include \"wave_reduce.hip.h\"");
         wave_reductions++;
     }
     std::string pending_partial;
@@ -1659,6 +1659,7 @@ public:
             std::vector<std::string> cmd = {hipcc ? hipcc : TIRAMISU_DEFAULT_HIPCC, "--genco",
                                             std::string("--offload-arch=") + (arch ? arch : TIRAMISU_DEFAULT_HIP_ARCH), "-std=c++17"};
             for (auto &w : words(flags ? flags : "-O3")) cmd.push_back(w);
+            cmd.push_back("-I" + kernel_dir());            // the kernel headers are included by file name
             for (const char *w : {"-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o"}) cmd.push_back(w);
             cmd.push_back(hsaco);
             cmd.push_back(hip_file);
@@ -1694,8 +1695,7 @@ public:
         }
         {
             const char *cxx = std::getenv("TIRAMISU_HOST_CXX");
-            std::string inc = TIRAMISU_AMD_INCLUDE_DIR;
-            if (const char *e = std::getenv("TIRAMISU_AMD_INCLUDE")) inc = e;
+            const std::string inc = include_dir();
             const std::vector<std::string> cmd = {cxx ? cxx : "g++", "-std=c++17", "-O2", "-fPIC", "-I" + inc, "-c", host_file, "-o", obj};
             if (run(cmd) != 0) ERROR("host compiler failed on " + host_file, true);
         }
@@ -1722,7 +1722,7 @@ public:
                 }
                 m << "]}";
             }
-            m << "\n  ],\n  \"kernels\": [";
+            m << "\n  ],\n  \"kernel_headers\": " << quoted(device_code ? kernel_dir() : std::string()) << ",\n  \"kernels\": [";
             for (size_t i = 0; i < ctx.kernels.size(); i++)
                 m << (i ? "," : "") << "\n    {\"name\": " << quoted(ctx.kernels[i].name) << ", \"how\": " << quoted(ctx.kernels[i].how) << "}";
             m << "\n  ],\n  \"options\": [";

@@ -92,6 +92,7 @@ bool emit_stencil(context &ctx, const lir::node_ptr &root, const lir::node_ptr &
 /** Directory of the kernel headers that emitted code includes (TIRAMISU_AMD_KERNEL_DIR overrides the
   * one compiled in), and the helper that adds an #include line to the kernel file once. */
 std::string kernel_dir();
+std::string include_dir();
 void add_include_once(context &ctx, const std::string &line);
 
 /** Text of the launch of \p k with the argument list taken from host variables of the same names. */

@@ -336,7 +336,13 @@ void dispatch_splitk(const splitk_plan &p, bool tA, bool tB, bool edge, const fl
 // current stream, and two calls of one thread on two streams may run at the same time: they must not share partial
 // tiles and counters), grown on demand, kept until the process ends.
 struct splitk_block { void *ptr = nullptr; uint64_t bytes = 0; };
-thread_local std::map<hipStream_t, splitk_block> splitk_workspaces;
+// (the per-thread default stream is one handle that names a different stream in every thread, hence the thread in the key)
+typedef std::pair<std::thread::id, hipStream_t> thread_and_stream;
+thread_and_stream here() { return {std::this_thread::get_id(), current_stream}; }
+std::mutex kept_mutex;                                                    // guards the two maps below
+std::map<thread_and_stream, splitk_block> splitk_workspaces;
+// Scratch that generated functions keep between their calls (tiramisu_hip_kept_scratch): by requesting site, thread and stream.
+std::map<std::pair<const void *, thread_and_stream>, splitk_block> kept_scratch;
 constexpr uint64_t SPLITK_WORKSPACE_LIMIT = (uint64_t)256 << 20;
 
 // Scratch of the entry point that allocates nothing: lives in the code object, one copy per device.
@@ -561,7 +567,8 @@ static int sgemm_impl(const char *fn, bool static_scratch, float *A, float *B, f
             }
             ws = static_scratch_here();
         } else {
-            splitk_block &block = splitk_workspaces[current_stream];
+            std::lock_guard<std::mutex> g(kept_mutex);
+            splitk_block &block = splitk_workspaces[here()];
             if (block.bytes < plan.scratch_bytes) {
                 if (block.ptr) {
                     check(hipStreamSynchronize(current_stream), fn);
@@ -637,8 +644,54 @@ int tiramisu_hip_batch_end(void) {
 }
 
 void *tiramisu_hip_sgemm_workspace(void) {
-    auto it = splitk_workspaces.find(current_stream);
+    std::lock_guard<std::mutex> g(kept_mutex);
+    auto it = splitk_workspaces.find(here());
     return it == splitk_workspaces.end() ? nullptr : it->second.ptr;
+}
+
+void *tiramisu_hip_kept_scratch(const void *site, uint64_t bytes, int32_t *fresh) {
+    std::lock_guard<std::mutex> g(kept_mutex);
+    splitk_block &block = kept_scratch[{site, here()}];
+    if (fresh) *fresh = 0;
+    if (block.bytes < bytes) {
+        if (block.ptr) {
+            check(hipStreamSynchronize(current_stream), __FUNCTION__);
+            check(hipFree(block.ptr), __FUNCTION__);
+        }
+        check(hipMalloc(&block.ptr, bytes), __FUNCTION__);
+        block.bytes = bytes;
+        if (fresh) *fresh = 1;
+    }
+    return block.ptr;
+}
+
+uint64_t tiramisu_hip_release_cached_memory(void) {
+    check(hipDeviceSynchronize(), __FUNCTION__);
+    uint64_t released = 0;
+    {
+        std::lock_guard<std::mutex> g(kept_mutex);
+        for (auto &kv : splitk_workspaces) if (kv.second.ptr) { check(hipFree(kv.second.ptr), __FUNCTION__); released += kv.second.bytes; }
+        for (auto &kv : kept_scratch) if (kv.second.ptr) { check(hipFree(kv.second.ptr), __FUNCTION__); released += kv.second.bytes; }
+        splitk_workspaces.clear();
+        kept_scratch.clear();
+    }
+    std::lock_guard<std::mutex> g(pool_mutex);
+    for (auto &kv : pool_free)
+        for (void *q : kv.second) { check(hipFree(q), __FUNCTION__); released += kv.first; }
+    pool_free.clear();
+    pool_idle_bytes = 0;
+    return released;
+}
+
+uint64_t tiramisu_hip_cached_memory_bytes(void) {
+    uint64_t held = 0;
+    {
+        std::lock_guard<std::mutex> g(kept_mutex);
+        for (auto &kv : splitk_workspaces) held += kv.second.bytes;
+        for (auto &kv : kept_scratch) held += kv.second.bytes;
+    }
+    std::lock_guard<std::mutex> g(pool_mutex);
+    return held + pool_idle_bytes;
 }
 
 int tiramisu_hip_dgemm(double *A, double *B, double *C, uint64_t M, uint64_t N, uint64_t K, double alpha, double beta,

@@ -3,6 +3,8 @@
 // domains and store relations, with isl where sets and maps are compared -- that the nest is of
 // its kind, and only then replaces it by kernels shaped for gfx950.  Anything that fails a check
 // falls back to the generic emitter, which reproduces the reference's behaviour.
+#include <dlfcn.h>
+#include <unistd.h>
 #include <algorithm>
 #include <cstdlib>
 #include <sstream>
@@ -25,9 +27,38 @@ using lir::node_ptr;
 #define TIRAMISU_AMD_KERNEL_DIR "."
 #endif
 
+#ifndef TIRAMISU_AMD_INCLUDE_DIR
+#define TIRAMISU_AMD_INCLUDE_DIR "."
+#endif
+
+// A directory of files that generated code needs at code-generation time.  An installed library (lib/libtiramisu.so
+// with share/ and include/ beside lib/) finds them relative to its own file, so that an installation can be moved;
+// a library in its build tree falls back to the source directories it was built from.
+static std::string beside_library(const char *relative, const char *probe) {
+    Dl_info info;
+    if (!dladdr((void *)&beside_library, &info) || !info.dli_fname) return "";
+    const std::string lib = info.dli_fname;
+    const size_t slash = lib.rfind('/');
+    const std::string dir = (slash == std::string::npos ? std::string(".") : lib.substr(0, slash)) + "/" + relative;
+    if (access((dir + "/" + probe).c_str(), R_OK) != 0) return "";
+    char *real = realpath(dir.c_str(), nullptr);
+    const std::string out = real ? real : dir;
+    free(real);
+    return out;
+}
+
+// the kernel headers (generated device code includes them by file name; the device compiler gets this directory as -I)
 std::string kernel_dir() {
     if (const char *e = std::getenv("TIRAMISU_AMD_KERNEL_DIR")) return e;
-    return TIRAMISU_AMD_KERNEL_DIR;
+    const std::string installed = beside_library("../share/tiramisu/kernels", "gemm_mfma.hip.h");
+    return installed.empty() ? TIRAMISU_AMD_KERNEL_DIR : installed;
+}
+
+// tiramisu_hip_wrappers.h for the generated host code
+std::string include_dir() {
+    if (const char *e = std::getenv("TIRAMISU_AMD_INCLUDE")) return e;
+    const std::string installed = beside_library("../include", "tiramisu_hip_wrappers.h");
+    return installed.empty() ? TIRAMISU_AMD_INCLUDE_DIR : installed;
 }
 
 void add_include_once(context &ctx, const std::string &line) {
@@ -294,8 +325,8 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
     static const char *const mode_text[] = {"", ", into a third plane", ", from a third plane into both planes", ", out of place"};
     host << "    {\n";
     if (temp_plane)
-        host << "        static thread_local float *_st_temp = nullptr;   // third plane: allocated at the first call, kept\n"
-             << "        if (!_st_temp) _st_temp = (float *)tiramisu_hip_malloc((uint64_t)" << NY << " * " << NX << " * sizeof(float));\n";
+        host << "        static const char _st_site = 0;   // third plane: the runtime keeps it from call to call (per thread and stream)\n"
+             << "        float *_st_temp = (float *)tiramisu_hip_kept_scratch(&_st_site, (uint64_t)" << NY << " * " << NX << " * sizeof(float), nullptr);\n";
     else if (!planar)
         host << "        float *_st_temp = nullptr;\n";
     for (auto &ch : chunks) {
@@ -321,7 +352,7 @@ bool emit_stencil(context &ctx, const node_ptr &root, const node_ptr &time_loop,
               << "\n#define ST_IBY0 " << by0 << "\n#define ST_IBY1 " << by1 << "\n#define ST_W " << WAVES
               << "\n#define ST_MERGE " << (merge ? 1 : 0) << "\n#define ST_XCD " << env_int("TIRAMISU_STENCIL_XCD", 1) << "\n#define ST_OCC " << env_int("TIRAMISU_STENCIL_OCCUPANCY", 0) << "\n#define ST_STREAM " << env_int("TIRAMISU_STENCIL_STREAM", 2)
               << "\n#define ST_RPT " << ROWS << "\n#define ST_RPT_EDGE " << rows_edge << "\n#define ST_R " << ch.steps << "\n#define ST_MODE " << ch.mode << "\n#define ST_RAD " << radius
-              << "\n#define ST_EXPR " << point_text << "\n#include \"" << kernel_dir() << "/stencil2d_regs.hip.h\"\n"
+              << "\n#define ST_EXPR " << point_text << "\n#include \"stencil2d_regs.hip.h\"\n"
               << "#undef ST_NAME\n#undef ST_NAME_EDGE\n#undef ST_NY\n#undef ST_NX\n#undef ST_Y0\n#undef ST_Y1\n#undef ST_X0\n#undef ST_X1\n"
               << "#undef ST_GX\n#undef ST_GY\n#undef ST_IBX0\n#undef ST_IBX1\n#undef ST_IBY0\n#undef ST_IBY1\n#undef ST_W\n#undef ST_OCC\n#undef ST_STREAM\n"
               << "#undef ST_MERGE\n#undef ST_XCD\n#undef ST_RPT\n#undef ST_RPT_EDGE\n#undef ST_R\n#undef ST_MODE\n#undef ST_RAD\n#undef ST_EXPR\n";
@@ -1704,19 +1735,19 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
         k.params.push_back({true, nm, b->get_elements_type()});
     }
     if (windowed) {
-        // scratch for the pieces of the last round's tiles and their counters: one block per host thread and
-        // stream (a call works on the thread's current stream; calls of one thread on two streams may overlap and
-        // must not share queues and counters), allocated at the first call there and kept; the counters start at
-        // zero and every launch leaves them at zero
+        // scratch for the pieces of the last round's tiles and their counters: kept by the runtime, one block per host
+        // thread and stream (a call works on the thread's current stream; calls of one thread on two streams may overlap
+        // and must not share queues and counters), allocated at the first call there; the counters start at zero and
+        // every launch leaves them at zero
         // (buffer parameters stay sorted by name)
         auto at = k.params.begin();
         while (at != k.params.end() && (!at->is_buffer || at->name < "_tail_scratch")) ++at;
         k.params.insert(at, {true, "_tail_scratch", p_float32});
         k.grid[0] = std::to_string(win_grid);
-        host << "        static thread_local std::map<void *, float *> _tail_scratch_of;\n";
-        host << "        float *&_tail_scratch = _tail_scratch_of[tiramisu_hip_get_stream()];\n";
-        host << "        if (!_tail_scratch) {\n";
-        host << "            _tail_scratch = (float *)tiramisu_hip_malloc((uint64_t)" << win_scratch_floats << " * sizeof(float));\n";
+        host << "        static const char _tail_site = 0;\n";
+        host << "        int32_t _tail_fresh = 0;\n";
+        host << "        float *_tail_scratch = (float *)tiramisu_hip_kept_scratch(&_tail_site, (uint64_t)" << win_scratch_floats << " * sizeof(float), &_tail_fresh);\n";
+        host << "        if (_tail_fresh) {\n";
         host << "            static const uint32_t _zeros[" << win_counters << "] = {};\n";
         host << "            tiramisu_hip_memcpy_to_device((void *)(_tail_scratch + " << (win_scratch_floats - win_counters) << "), (void *)_zeros, sizeof(_zeros));\n";
         host << "        }\n";
@@ -1745,9 +1776,9 @@ bool emit_contraction(context &ctx, const node_ptr &root, launch_plan &plan, con
     }
     src << ")\n{\n" << batch_prologue.str() << body.str() << "}\n";
     k.source = src.str();
-    add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma.hip.h\"");
-    if (bf16) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_bf16.hip.h\"");
-    if (windowed) add_include_once(ctx, "#include \"" + kernel_dir() + "/gemm_mfma_window.hip.h\"");
+    add_include_once(ctx, "#include \"gemm_mfma.hip.h\"");
+    if (bf16) add_include_once(ctx, "#include \"gemm_mfma_bf16.hip.h\"");
+    if (windowed) add_include_once(ctx, "#include \"gemm_mfma_window.hip.h\"");
     host << launch_text(k, "        ") << "    }\n";
     plan.kernels.push_back(k);
     plan.host_code = host.str();

@@ -71,6 +71,22 @@ class Buffer:
         """A buffer that already lives in GPU memory (an argument tagged tag_gpu_global())."""
         return Buffer(shape, dtype, host_ptr=0, device_ptr=int(ptr), keepalive=keepalive)
 
+    @staticmethod
+    def from_tensor(t):
+        """A ``torch.Tensor`` as an argument, without a copy: a tensor on the GPU describes a buffer tagged
+        tag_gpu_global() (its storage is the device pointer), a CPU tensor a host buffer.  bfloat16 tensors
+        are the 16-bit storage of p_bfloat16 buffers.  The tensor stays referenced while the buffer lives."""
+        import torch
+        if not t.is_contiguous():
+            raise ValueError("Tiramisu buffers are dense row-major: pass a contiguous tensor")
+        if t.dtype == torch.bfloat16:
+            dtype = np.dtype(np.uint16)
+        else:
+            dtype = np.dtype(str(t.dtype).replace("torch.", ""))
+        if t.is_cuda:
+            return Buffer(tuple(t.shape), dtype, device_ptr=t.data_ptr(), keepalive=t)
+        return Buffer(tuple(t.shape), dtype, host_ptr=t.data_ptr(), keepalive=t)
+
     def pointer(self):
         return ctypes.byref(self.raw)
 
@@ -99,6 +115,10 @@ def wrappers():
         lib.tiramisu_hip_stream_create.restype = ctypes.c_void_p
         lib.tiramisu_hip_stream_destroy.argtypes = [ctypes.c_void_p]
         lib.tiramisu_hip_sgemm_workspace.restype = ctypes.c_void_p
+        lib.tiramisu_hip_kept_scratch.restype = ctypes.c_void_p
+        lib.tiramisu_hip_kept_scratch.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int32)]
+        lib.tiramisu_hip_release_cached_memory.restype = ctypes.c_uint64
+        lib.tiramisu_hip_cached_memory_bytes.restype = ctypes.c_uint64
         lib.tiramisu_hip_event_create.restype = ctypes.c_void_p
         lib.tiramisu_hip_event_record.argtypes = [ctypes.c_void_p]
         lib.tiramisu_hip_event_elapsed_ms.restype = ctypes.c_float
@@ -178,10 +198,43 @@ class Program:
                     raise ValueError("%s: buffer %s has shape %s, %s given" % (self.name, e["name"], e["shape"], list(b.shape)))
 
     def __call__(self, *args):
-        bufs = [a if isinstance(a, Buffer) else Buffer.from_numpy(a) for a in args]
+        """Arguments: ``Buffer`` objects, numpy arrays (host buffers) or torch tensors (host or GPU buffers by where
+        they live).  With a GPU tensor among them the function's kernels run on torch's current stream of that
+        tensor's device, in order with the torch work around the call (the runtime's stream of the calling thread is
+        put back afterwards); when that is torch's default stream the call waits for it first and for its own
+        kernels afterwards."""
+        bufs, torch_stream = [], None
+        for a in args:
+            if isinstance(a, Buffer):
+                bufs.append(a)
+            elif isinstance(a, np.ndarray):
+                bufs.append(Buffer.from_numpy(a))
+            elif type(a).__module__.split(".")[0] == "torch":
+                bufs.append(Buffer.from_tensor(a))
+                if a.is_cuda and torch_stream is None:
+                    import torch
+                    torch_stream = torch.cuda.current_stream(a.device).cuda_stream
+            else:
+                bufs.append(Buffer.from_numpy(a))
         if self.manifest is not None:
             self.check(bufs)
-        rc = self.fn(*[b.pointer() for b in bufs])
+        if torch_stream is None:
+            rc = self.fn(*[b.pointer() for b in bufs])
+        elif torch_stream == 0:
+            # torch's default stream is the device's null stream, which the runtime has no handle for: order the
+            # call by waiting on both sides instead
+            import torch
+            torch.cuda.current_stream().synchronize()
+            rc = self.fn(*[b.pointer() for b in bufs])
+            wrappers().tiramisu_hip_stream_synchronize(0)
+        else:
+            w = wrappers()
+            before = w.tiramisu_hip_get_stream()
+            w.tiramisu_hip_set_stream(torch_stream)
+            try:
+                rc = self.fn(*[b.pointer() for b in bufs])
+            finally:
+                w.tiramisu_hip_set_stream(before)
         if rc != 0:
             raise RuntimeError("Tiramisu function returned %d" % rc)
         return rc
