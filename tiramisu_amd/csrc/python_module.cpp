@@ -200,6 +200,8 @@ void define_computation(py::module &m) {
         .def("__rsub__", [](constant &c, const expr &o) { return o - (expr)c; })
         .def("__mul__", [](constant &c, const expr &o) { return (expr)c * o; })
         .def("__rmul__", [](constant &c, const expr &o) { return o * (expr)c; });
+    // a constant where an expression is expected (loop bounds: var("i", 0, N)), as constant::operator expr() gives in C++
+    py::reinterpret_borrow<py::class_<expr>>(m.attr("expr")).def(py::init([](constant &c) { return (expr)c; }));
     py::implicitly_convertible<constant, expr>();
 }
 

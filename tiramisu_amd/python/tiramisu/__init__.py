@@ -35,8 +35,12 @@ def pycodegen(arguments, obj_filename, gen_gpu=True, *unused, _function=None):
     name = (_function or _ext.get_implicit_function()).get_name()
     directory = os.path.dirname(os.path.abspath(obj_filename))
     library = os.path.join(directory, "lib%s.so" % name)
-    subprocess.run(["g++", "-shared", "-o", library, os.path.abspath(obj_filename), "-L" + _PKG, "-ltiramisu_hip_wrappers",
-                    "-Wl,-rpath," + _PKG], check=True)
+    for_gpu = gen_gpu != _ext.hardware_architecture_t.arch_cpu if isinstance(gen_gpu, _ext.hardware_architecture_t) else bool(gen_gpu)
+    if for_gpu:
+        link = ["-L" + _PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath," + _PKG]
+    else:
+        link = ["-fopenmp"]         # an object of a CPU back-end (none ships with this package; one can be registered)
+    subprocess.run(["g++", "-shared", "-o", library, os.path.abspath(obj_filename)] + link, check=True)
     sys.path.insert(0, os.path.dirname(_PKG))
     try:
         from tiramisu_amd import runtime
@@ -44,7 +48,7 @@ def pycodegen(arguments, obj_filename, gen_gpu=True, *unused, _function=None):
         sys.path.pop(0)
     module = types.ModuleType(name)
     module.__file__ = library
-    setattr(module, name, runtime.Program(library, name))
+    setattr(module, name, runtime.Program(library, name, needs_gpu_runtime=for_gpu))
     sys.modules[name] = module
     return module
 
