@@ -97,7 +97,7 @@ struct cpu_gen {
                        b->get_location() != memory_location::host) {
                 out << pad(ind) << t << " " << b->get_name() << "[" << cp.element_count(b) << "];\n";
             } else {
-                out << pad(ind) << b->get_name() << " = (" << t << " *)malloc((size_t)(" << cp.element_count(b)
+                out << pad(ind) << b->get_name() << " = (" << t << " *)malloc((size_t)(" << cp.element_count(b, n->iterators)
                     << ") * sizeof(" << t << "));\n";
             }
             return;
@@ -114,8 +114,9 @@ struct cpu_gen {
                 std::string s = "extern \"C\" " + primitive_c_name(e.get_data_type()) + " " + e.get_name() + "(";
                 for (size_t i = 0; i < e.get_arguments().size(); i++) {
                     const expr &a = e.get_arguments()[i];
-                    s += (i ? ", " : "") + ((a.get_expr_type() == e_op && a.get_op_type() == o_buffer)
-                                                 ? std::string("void *") : primitive_c_name(a.get_data_type()));
+                    s += (i ? ", " : "") + ((a.get_expr_type() == e_op && a.get_op_type() == o_buffer) ? std::string("void *")
+                                             : (a.get_expr_type() == e_op && a.get_op_type() == o_address) ? std::string("halide_buffer_t *")
+                                             : primitive_c_name(a.get_data_type()));
                 }
                 extern_decls.push_back(s + ");");
             }

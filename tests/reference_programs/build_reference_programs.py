@@ -217,8 +217,8 @@ def build_cpu_benchmark(rel, stem, obj, extra):
 # (wrapper and generator disagree in the reference itself: expected value 2 against a generated 1, a
 # 10-element buffer handed to a 100-iteration loop); 133-140 (a recurrence whose dependent loop the test
 # tags parallel: the result depends on thread timing).
-SUITE = """01 02 03 04 06 07 08 09 10 11 12 13 16 17 18 19 20 22 23 24 25 26 29 30 31 32 33 34 35 36 37 38 39 40 41 42 43 44 45 46 47 48 51 52 53 54 55 56 57 58 59 60 61 62 63 64
-65 66 67 68 69 70 71 72 73 74 75 76 77 78 80 81 84 86 87 88 89 91 97 103 104 105 106 107 108 109 110 111 112 113 114 115 116 117 118 119 120 121 122 123
+SUITE = """01 02 03 04 06 07 08 09 10 11 12 13 16 17 18 19 20 21 22 23 24 25 26 29 30 31 32 33 34 35 36 37 38 39 40 41 42 43 44 45 46 47 48 51 52 53 54 55 56 57 58 59 60 61 62 63 64
+65 66 67 68 69 70 71 72 73 74 75 76 77 78 79 80 81 84 86 87 88 89 91 92 97 103 104 105 106 107 108 109 110 111 112 113 114 115 116 117 118 119 120 121 122 123
 124 125 126 127 128 129 131 141 142 143 144 145 146 147 148 149 150 151 152 153 154 155 156 157 158 159 161 163 167 168 169 170 171 175
 176 177 178 179 180 181 182 183 184 185 186 187 188 189 190 191 192 193 194 195 196 197 198 199""".split()
 

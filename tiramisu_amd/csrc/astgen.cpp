@@ -181,6 +181,15 @@ struct lowering {
                 }
                 ERROR("access to undeclared computation " + e.get_name(), true);
             }
+            if (e.get_op_type() == o_address) {
+                // expr(o_address, var("S0")): the halide_buffer_t of the buffer that computation S0 is stored in, for
+                // an external function (reference: tiramisu_codegen_halide.cpp:3830-3835, "<buffer>.buffer")
+                const std::string &nm = e.get_operand(0).get_name();
+                computation *X = find_computation(nm);
+                const buffer *b = X ? X->get_buffer() : (f->get_buffers().count(nm) ? f->get_buffers().at(nm) : nullptr);
+                if (!b) ERROR("address of " + nm + ": neither a computation with a buffer nor a buffer", true);
+                return expr(o_address, expr(o_buffer, b->get_name()));
+            }
             expr r = e;
             std::vector<expr> ops, args;
             for (auto &o : e.get_operands()) ops.push_back(lower_expr(build, L, iters, o));

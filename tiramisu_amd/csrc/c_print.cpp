@@ -88,8 +88,17 @@ std::string c_printer::store(const buffer *b, const std::vector<expr> &index, co
 }
 
 std::string c_printer::element_count(const buffer *b) const {
+    return element_count(b, {});
+}
+
+// extents of a buffer allocated inside a loop nest may name the allocating computation's iterators
+// (f_b[i + 1] allocated at loop i): they are written in the loop iterators of the generated code
+std::string c_printer::element_count(const buffer *b, const std::map<std::string, expr> &iterators) const {
     expr n;
-    for (auto &d : b->get_dim_sizes()) n = n.is_defined() ? lir::simplify(n * cast(p_int64, d)) : cast(p_int64, d);
+    for (auto &d0 : b->get_dim_sizes()) {
+        const expr d = iterators.empty() ? d0 : lir::simplify(d0.substitute(iterators));
+        n = n.is_defined() ? lir::simplify(n * cast(p_int64, d)) : cast(p_int64, d);
+    }
     return n.is_defined() ? print(n) : "1";
 }
 
@@ -161,6 +170,16 @@ std::string c_printer::print(const expr &e) const {
     case o_buffer: {
         if (used_buffers) used_buffers->insert(e.get_name());
         return e.get_name();
+    }
+    case o_address: {
+        // the halide_buffer_t of an argument buffer: generated host functions name their arguments _a0, _a1, ...
+        const std::string &nm = e.get_operand(0).get_name();
+        if (device) ERROR("address of buffer " + nm + " inside a GPU kernel", true);
+        if (used_buffers) used_buffers->insert(nm);
+        const auto &args = fct->get_arguments();
+        for (size_t i = 0; i < args.size(); i++)
+            if (args[i]->get_name() == nm) return "_a" + std::to_string(i);
+        ERROR("address of buffer " + nm + ", which is not an argument of the function (only arguments have a halide_buffer_t)", true);
     }
     case o_address_of: {
         auto it = fct->get_buffers().find(e.get_name());

@@ -3,6 +3,7 @@
 // three agree on the meaning of every operator by construction.
 #ifndef TIRAMISU_AMD_C_PRINT_H
 #define TIRAMISU_AMD_C_PRINT_H
+#include <map>
 #include <functional>
 #include <set>
 #include <string>
@@ -34,6 +35,7 @@ struct c_printer {
     std::string literal(const expr &e) const;
     /** Number of elements of \p b as an expression text. */
     std::string element_count(const buffer *b) const;
+    std::string element_count(const buffer *b, const std::map<std::string, expr> &iterators) const;
 };
 
 /** Helper functions (floor division, min/max, bf16 conversion) that printed code relies on;

@@ -685,6 +685,7 @@ void function::allocate_and_map_buffers_automatically() {
     }
     for (computation *c : body) {
         if (!c->has_accesses() || c->get_access_relation() || c->get_automatically_allocated_buffer()) continue;
+        if (c->is_inline_computation()) continue;    // replaced by its expression wherever it is read: no storage (its domain may be unbounded)
         if (!c->is_first_definition()) continue;      // updates share the first definition's buffer, below
         const argument_t kind = !c->should_schedule_this_computation() ? a_input : (read.count(c->get_name()) ? a_temporary : a_output);
         c->allocate_and_map_buffer_automatically(kind);

@@ -1186,8 +1186,9 @@ struct host_gen {
         std::string s = "extern \"C\" " + primitive_c_name(call.get_data_type()) + " " + nm + "(";
         for (size_t i = 0; i < call.get_arguments().size(); i++) {
             const expr &a = call.get_arguments()[i];
-            std::string t = (a.get_expr_type() == e_op && a.get_op_type() == o_buffer)
-                                ? "void *" : primitive_c_name(a.get_data_type());
+            std::string t = (a.get_expr_type() == e_op && a.get_op_type() == o_buffer) ? "void *"
+                            : (a.get_expr_type() == e_op && a.get_op_type() == o_address) ? "halide_buffer_t *"
+                            : primitive_c_name(a.get_data_type());
             s += (i ? ", " : "") + t;
         }
         extern_decls.push_back(s + ");");
@@ -1450,7 +1451,7 @@ struct host_gen {
         case leaf_kind::allocate: {
             buffer *b = n->target;
             std::string t = primitive_c_name(b->get_elements_type());
-            std::string bytes = "(uint64_t)(" + hp.element_count(b) + ") * sizeof(" + t + ")";
+            std::string bytes = "(uint64_t)(" + hp.element_count(b, n->iterators) + ") * sizeof(" + t + ")";
             if (b->get_location() == memory_location::global)
                 out << pad(ind) << b->get_name() << " = (" << t << " *)tiramisu_hip_malloc(" << bytes << ");\n";
             else if (b->get_location() == memory_location::host)
