@@ -1,5 +1,5 @@
 """Runs one of the reference's Python tutorials (python_bindings/tutorials/*.py, read where it lies, unchanged) against
-this build's `tiramisu` module: usage  run_reference_tutorial.py <path of the tutorial>  from the directory that is
+this build's `tiramisu` module: usage  run_python_tutorial.py <path of the tutorial>  from the directory that is
 to receive the generated files.  The tutorials generate CPU code; this package ships no CPU back-end, so the test
 harness registers the oracle's restatement of it (loading the library is what registers it) -- test infrastructure,
 not a product path."""

@@ -1,7 +1,7 @@
 """The reference's Python tutorials (python_bindings/tutorials/tutorial_01 ... tutorial_05.py), unchanged, through this
 build's Python front-end (tiramisu_amd/csrc/python_module.cpp, names and overloads of python_bindings/tiramisu.pyi).
 They are CPU programs: the object each one generates comes from the oracle's CPU emitter, registered by the
-runner (tests/python_programs/run_reference_tutorial.py), is linked into a shared library here and called on seeded
+runner (tests/reference_programs/run_python_tutorial.py), is linked into a shared library here and called on seeded
 data; the expectations are what the tutorials' own comments state, restated in numpy."""
 import os
 import subprocess
@@ -16,7 +16,7 @@ from tiramisu_amd import runtime
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REFERENCE = os.environ.get("TIRAMISU_REFERENCE_TREE", "/root/reference")
 TUTORIALS = os.path.join(REFERENCE, "python_bindings", "tutorials")
-RUNNER = os.path.join(ROOT, "tests", "python_programs", "run_reference_tutorial.py")
+RUNNER = os.path.join(ROOT, "tests", "reference_programs", "run_python_tutorial.py")
 
 pytestmark = pytest.mark.skipif(not os.path.isdir(TUTORIALS) or not os.path.exists(oracle_build.CPU_BACKEND),
                                 reason="needs the reference's tutorials and the oracle's CPU emitter")

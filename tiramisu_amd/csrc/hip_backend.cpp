@@ -894,13 +894,42 @@ struct generic_kernel_gen {
             body << pad(ind) << "}\n";
             return;
         }
+        // Short loops are unrolled (register tiles are arrays that must end up in registers, and index arithmetic folds),
+        // but within a budget: the statements that unrolling this loop and every short loop below it would lay out.
+        // Beyond it the loop is left to the compiler's own judgement -- nests of many short loops (tensor contractions
+        // over spin and colour indices: 3 x 2 x 3 x 2 x 8 x 3 x 2) would otherwise become tens of thousands of
+        // statements, minutes of device compilation and code that misses the instruction cache.
         expr lo = lir::simplify(n->init), up = lir::simplify(n->upper);
-        bool small = lo.is_integer_literal() && up.is_integer_literal() && up.get_int_val() - lo.get_int_val() < 32;
+        const bool small_loop = lo.is_integer_literal() && up.is_integer_literal() && up.get_int_val() - lo.get_int_val() < 32;
+        const bool small = small_loop && unrolled_statements(n) <= unroll_budget();
         if (n->unrolled || small) body << pad(ind) << "#pragma unroll\n";
         body << pad(ind) << "for (int32_t " << n->iterator << " = " << dev.print(n->init) << "; " << n->iterator
              << " <= " << dev.print(n->upper) << "; " << n->iterator << " += " << dev.print(n->increment) << ") {\n";
         emit(n->body, ind + 1);
         body << pad(ind) << "}\n";
+    }
+
+    long unroll_budget() const {
+        const char *e = backend_option("TIRAMISU_HIP_UNROLL_BUDGET");
+        return e ? std::atol(e) : 1024;
+    }
+    // statements of the loop nest below n with every loop of constant extent unrolled (other loops count once)
+    static long unrolled_statements(const node_ptr &n) {
+        if (!n) return 0;
+        switch (n->kind) {
+        case node_kind::leaf: return n->lkind == leaf_kind::assign || n->lkind == leaf_kind::call ? 1 : 0;
+        case node_kind::block: { long s = 0; for (auto &c : n->children) s += unrolled_statements(c); return s; }
+        case node_kind::cond: return unrolled_statements(n->then_body) + unrolled_statements(n->else_body);
+        case node_kind::loop: {
+            const expr lo = lir::simplify(n->init), up = lir::simplify(n->upper);
+            long trip = 1;
+            if (n->gpu_block < 0 && n->gpu_thread < 0 && lo.is_integer_literal() && up.is_integer_literal())
+                trip = std::max<long>(1, up.get_int_val() - lo.get_int_val() + 1);
+            const long below = unrolled_statements(n->body);
+            return below > (1L << 40) / trip ? (1L << 40) : trip * below;
+        }
+        }
+        return 0;
     }
 
     std::string declaration(const buffer *b) {
@@ -1026,12 +1055,15 @@ static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const
         hp.fct = f;
         k.batch_first = hp.print(batch->batch_first);
         k.grid[2] = "((" + hp.print(batch->batch_last) + ") >= _batch_first ? (" + hp.print(batch->batch_last) + ") - _batch_first + 1 : 0)";
-        k.params.push_back({false, "_batch_first", global::get_loop_iterator_data_type()});
+        k.params.push_back({false, "_batch_first", p_int32});            // as the launch declares it
     }
     for (auto &nm : g.used_scalars) {
         if (g.inner.count(nm)) continue;
         if (batch && nm == batch->batch_iterator) { batch_iterator_used = true; continue; }
-        primitive_t t = global::get_loop_iterator_data_type();
+        // An iterator of a host loop around the launch: host loops are declared int32_t whatever the program's loop
+        // iterator type is (set_loop_iterator_type(p_int64) types the expressions, not the generated loops), and the
+        // launch passes the variable's address -- the parameter must have the variable's own width.
+        primitive_t t = p_int32;
         for (auto c : f->get_invariants())
             if (c->get_name() == nm) t = c->get_data_type();
         for (auto c : f->get_computation_by_name(nm))   // a constant scheduled on the host
