@@ -95,6 +95,46 @@ def build_baryon(rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
+# One of the four dibaryon correlators (benchmarks/tensors/dibaryon/gpu_*): ten kernels, 1.3 MB of kernel source.
+# Compiling its generator takes four minutes and running it five (three quarters of that inside isl's ordering of
+# the statements' domains while it builds the AST), so it is built on request only: TIRAMISU_BUILD_DIBARYON=1.
+# Its wrapper keeps the comparison with the authors' C++ restatement behind two switches that are off
+# ("#define RUN_REFERENCE 0", "#define RUN_CHECK 0") and includes that restatement, standard headers and all, inside
+# an extern "C" block: the switches are flipped on the way into the compiler (the text goes through a pipe; nothing of
+# the reference is written anywhere) and the standard headers are included ahead of the file.
+DIBARYON = ["benchmarks/tensors/dibaryon/gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
+
+
+def build_dibaryon(rel):
+    import subprocess
+    name = os.path.basename(rel)
+    source = os.path.join(REFERENCE, rel)
+    bdir = os.path.join(HERE, "build")
+    work = os.path.join(bdir, name)
+    os.makedirs(work, exist_ok=True)
+    generator = [f for f in os.listdir(source) if f.endswith("_generator.cpp")][0]
+    wrapper = [f for f in os.listdir(source) if f.endswith("_wrapper.cpp")][0]
+    build.build_program(os.path.join(source, generator), directory=work, shim_headers=True)
+    objects = [os.path.join(work, f) for f in os.listdir(work) if f.endswith(".o")]
+    entry = os.path.join(bdir, "entry.h")
+    with open(entry, "w") as f:
+        f.write('extern "C" int tiramisu_wrapper_main(int, char **);\n')
+    text = open(os.path.join(source, wrapper)).read()
+    for switch in ("RUN_REFERENCE", "RUN_CHECK"):
+        if "#define %s 0" % switch not in text:
+            raise RuntimeError("%s: no '#define %s 0' to flip" % (wrapper, switch))
+        text = text.replace("#define %s 0" % switch, "#define %s 1" % switch)
+    ahead = []
+    for h in ("complex", "vector", "fstream", "string", "map", "iostream", "stdio.h", "stdlib.h", "math.h", "time.h", "chrono", "algorithm"):
+        ahead += ["-include", h]
+    cmd = ["g++", "-std=c++17", "-O2", "-w", "-fPIC", "-shared", "-I" + build.INCLUDE, "-I" + os.path.join(build.INCLUDE, "tiramisu", "shim"),
+           "-I" + source] + ahead + ["-include", entry, "-Dmain=tiramisu_wrapper_main", "-o", library(name), "-x", "c++", "-", "-x", "none"] + objects + \
+          ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)]
+    r = subprocess.run(cmd, input=text, text=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+    if r.returncode != 0:
+        raise RuntimeError("wrapper of %s failed to compile:\n%s" % (name, r.stdout[-3000:]))
+
+
 # Benchmark generators whose wrapper needs CUDA, cuBLAS or cuDNN headers: the tests drive the
 # generated function themselves.  Each program writes its object into its working directory and
 # (all but the first LSTM) times its kernels through an external get_time(): timer_hook.c.
@@ -300,6 +340,11 @@ def build_all(verbose=False):
         if verbose:
             print("[reference programs]", rel, flush=True)
         build_baryon(rel)
+    if os.environ.get("TIRAMISU_BUILD_DIBARYON") == "1":
+        for rel in DIBARYON:
+            if verbose:
+                print("[reference programs]", rel, "(about ten minutes)", flush=True)
+            build_dibaryon(rel)
     if verbose:
         print("[reference programs] benchmarks/DNN/blocks/LSTM/gpu_lib/generator.cpp (double precision)", flush=True)
     build_lstm_gpu_lib_f64()

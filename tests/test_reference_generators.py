@@ -200,6 +200,7 @@ def test_reference_gpu_test_passes(name):
     assert lib.tiramisu_wrapper_main(0, None) == 0
 
 
+DIBARYON = ["gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
 BARYON = ["gpu_tiramisu_make_fused_baryon_blocks_correlator", "gpu_tiramisu_make_fused_identical_baryon_blocks_correlator",
           "gpu_single_tiramisu_make_fused_identical_baryon_blocks_correlator"]
 
@@ -227,6 +228,29 @@ def test_reference_baryon_correlator_passes_its_own_check(name):
     lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
     print("running", name, flush=True)
     assert lib.tiramisu_wrapper_main(0, None) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", DIBARYON)
+def test_reference_dibaryon_correlator_passes_its_own_check(name):
+    """benchmarks/tensors/dibaryon/gpu_single_...: generator unchanged; the wrapper with its two switches
+    (RUN_REFERENCE, RUN_CHECK) on, so that it runs the authors' C++ restatement and compares every correlator entry
+    with the generated function's (ten kernels; kernels inside host loops take the loops' iterators as parameters
+    in a program with 64-bit loop iterators).  Built on request only (TIRAMISU_BUILD_DIBARYON=1: about ten minutes)."""
+    if not os.path.exists(library(name)):
+        pytest.skip("built on request only: TIRAMISU_BUILD_DIBARYON=1 python tests/reference_programs/build_reference_programs.py")
+    runtime.wrappers()
+    lib = ctypes.CDLL(library(name))
+    lib.tiramisu_wrapper_main.restype = ctypes.c_int
+    lib.tiramisu_wrapper_main.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    print("running", name, flush=True)
+    here = os.getcwd()
+    work = os.path.join(HERE, "reference_programs", "build", name)
+    os.chdir(work)                      # the wrapper writes performance_CPU.csv where it runs
+    try:
+        assert lib.tiramisu_wrapper_main(0, None) == 0
+    finally:
+        os.chdir(here)
 
 
 TUNED_SGEMM = {"sgemm_generator1": "generic", "sgemm_generator2": "generic", "sgemm_generator3": "mfma-contraction"}
