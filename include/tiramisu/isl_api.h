@@ -32,6 +32,11 @@ typedef struct isl_ast_node_list isl_ast_node_list;
 typedef struct isl_ast_expr isl_ast_expr;
 typedef struct isl_constraint isl_constraint;
 typedef struct isl_map_list isl_map_list;
+typedef struct isl_schedule isl_schedule;
+typedef struct isl_schedule_node isl_schedule_node;
+typedef struct isl_union_set_list isl_union_set_list;
+typedef struct isl_union_pw_aff isl_union_pw_aff;
+typedef struct isl_multi_union_pw_aff isl_multi_union_pw_aff;
 
 typedef int isl_size;
 typedef enum { isl_bool_error = -1, isl_bool_false = 0, isl_bool_true = 1 } isl_bool;
@@ -168,6 +173,12 @@ char *isl_union_map_to_str(isl_union_map *umap);
 isl_map *isl_map_from_union_map(isl_union_map *umap);
 isl_union_map *isl_union_map_intersect_domain(isl_union_map *umap, isl_union_set *uset);
 isl_union_set *isl_union_set_from_set(isl_set *set);
+isl_union_set *isl_union_set_union(isl_union_set *a, isl_union_set *b);
+isl_union_set *isl_union_map_domain(isl_union_map *umap);
+isl_map_list *isl_union_map_get_map_list(isl_union_map *umap);
+isl_size isl_map_list_n_map(isl_map_list *list);
+isl_map *isl_map_list_get_map(isl_map_list *list, int index);
+isl_map_list *isl_map_list_free(isl_map_list *list);
 isl_bool isl_union_map_is_equal(isl_union_map *a, isl_union_map *b);
 
 /* dataflow analysis: the last write (must source) that every read (sink) sees under a schedule */
@@ -227,6 +238,24 @@ isl_union_map *isl_ast_build_get_schedule(isl_ast_build *build);
 isl_ast_expr *isl_ast_build_access_from_pw_multi_aff(isl_ast_build *build, isl_pw_multi_aff *pma);
 isl_ast_expr *isl_ast_build_call_from_pw_multi_aff(isl_ast_build *build, isl_pw_multi_aff *pma);
 isl_ast_expr *isl_ast_build_expr_from_pw_aff(isl_ast_build *build, isl_pw_aff *pa);
+
+// schedule trees (the second way into the AST generator)
+isl_schedule *isl_schedule_from_domain(isl_union_set *domain);
+isl_schedule *isl_schedule_free(isl_schedule *schedule);
+isl_schedule *isl_schedule_copy(isl_schedule *schedule);
+isl_schedule_node *isl_schedule_get_root(isl_schedule *schedule);
+isl_schedule *isl_schedule_node_get_schedule(isl_schedule_node *node);
+isl_schedule_node *isl_schedule_node_free(isl_schedule_node *node);
+isl_schedule_node *isl_schedule_node_child(isl_schedule_node *node, int pos);
+isl_schedule_node *isl_schedule_node_parent(isl_schedule_node *node);
+isl_schedule_node *isl_schedule_node_insert_sequence(isl_schedule_node *node, isl_union_set_list *filters);
+isl_schedule_node *isl_schedule_node_insert_partial_schedule(isl_schedule_node *node, isl_multi_union_pw_aff *schedule);
+isl_union_set_list *isl_union_set_list_alloc(isl_ctx *ctx, int n);
+isl_union_set_list *isl_union_set_list_add(isl_union_set_list *list, isl_union_set *el);
+isl_union_pw_aff *isl_union_pw_aff_from_pw_aff(isl_pw_aff *pa);
+isl_union_pw_aff *isl_union_pw_aff_union_add(isl_union_pw_aff *a, isl_union_pw_aff *b);
+isl_multi_union_pw_aff *isl_multi_union_pw_aff_from_union_pw_aff(isl_union_pw_aff *upa);
+isl_ast_node *isl_ast_build_node_from_schedule(isl_ast_build *build, isl_schedule *schedule);
 
 enum isl_ast_node_type isl_ast_node_get_type(isl_ast_node *node);
 isl_ast_expr *isl_ast_node_for_get_iterator(isl_ast_node *node);

@@ -385,6 +385,69 @@ void apply_tags(function *f, const node_ptr &root) {
 
 }  // namespace
 
+namespace {
+
+// The schedule as a tree (option ast_from_schedule_tree).  The reference hands isl one flat map from statement
+// instances to time vectors (tiramisu_function.cpp: gen_isl_ast, isl_ast_build_node_from_schedule_map), and isl then
+// finds out, level by level, which statements' domains follow which -- pairwise, an emptiness test each: with the
+// hundreds of statements of a tensor-contraction program three quarters of the generation time.  But the time vectors
+// say it outright: positions 0, 2, 4, ... hold the statement's place among its siblings (constants), positions 1, 3, ...
+// the loops.  So: a sequence node over the groups of equal constant for an even position (none when all agree), a band
+// of one member for an odd position, and so on down.  The AST is the same; isl is told the order instead of deriving it.
+struct scheduled_statement { isl_map *schedule; isl_pw_multi_aff *time; };
+
+isl_schedule_node *place(isl_ctx *ctx, isl_schedule_node *node, const std::vector<scheduled_statement *> &group, int p, int dims) {
+    if (p >= dims) return node;
+    if (p % 2 == 0) {
+        std::map<long, std::vector<scheduled_statement *>> by_place;
+        for (auto s : group) {
+            isl_val *v = isl_map_plain_get_val_if_fixed(s->schedule, isl_dim_out, p);
+            if (!v || isl_val_is_int(v) != isl_bool_true) { isl_val_free(v); return nullptr; }
+            by_place[isl_val_get_num_si(v)].push_back(s);
+            isl_val_free(v);
+        }
+        if (by_place.size() == 1) return place(ctx, node, group, p + 1, dims);
+        isl_union_set_list *filters = isl_union_set_list_alloc(ctx, (int)by_place.size());
+        for (auto &g : by_place) {
+            isl_union_set *members = nullptr;
+            for (auto s : g.second) {
+                isl_union_set *d = isl_union_set_from_set(isl_map_domain(isl_map_copy(s->schedule)));
+                members = members ? isl_union_set_union(members, d) : d;
+            }
+            filters = isl_union_set_list_add(filters, members);
+        }
+        node = isl_schedule_node_insert_sequence(node, filters);
+        int child = 0;
+        for (auto &g : by_place) {
+            node = isl_schedule_node_child(isl_schedule_node_child(node, child++), 0);
+            node = place(ctx, node, g.second, p + 1, dims);
+            if (!node) return nullptr;
+            node = isl_schedule_node_parent(isl_schedule_node_parent(node));
+        }
+        return node;
+    }
+    // A statement whose coordinate here is a constant while its siblings' are loops (a copy left unordered against
+    // a loop nest: same place, no loop of its own) would be scanned inside those loops under a guard; the flat form
+    // separates it out, which is what the emitters need (no copy inside a kernel).  Such schedules are left to it.
+    int constant = 0;
+    for (auto s : group) {
+        isl_val *v = isl_map_plain_get_val_if_fixed(s->schedule, isl_dim_out, p);
+        if (v && isl_val_is_int(v) == isl_bool_true) constant++;
+        isl_val_free(v);
+    }
+    if (constant != 0 && constant != (int)group.size()) return nullptr;
+    isl_union_pw_aff *when = nullptr;
+    for (auto s : group) {
+        isl_union_pw_aff *u = isl_union_pw_aff_from_pw_aff(isl_pw_multi_aff_get_pw_aff(s->time, p));
+        when = when ? isl_union_pw_aff_union_add(when, u) : u;
+    }
+    node = isl_schedule_node_insert_partial_schedule(node, isl_multi_union_pw_aff_from_union_pw_aff(when));
+    node = place(ctx, isl_schedule_node_child(node, 0), group, p + 1, dims);
+    return node ? isl_schedule_node_parent(node) : nullptr;
+}
+
+}  // namespace
+
 void function::gen_isl_ast() {
     for (auto c : body)
         if (!c->get_time_space_domain()) { gen_time_space_domain(); break; }
@@ -405,18 +468,88 @@ void function::gen_isl_ast() {
     }
     if (!umap) ERROR("function " + name + " has nothing to schedule", true);
 
+    // "1": build the AST from the schedule as a tree where the schedule has that layout; "check": build it both ways,
+    // keep the flat form's and report whether the two programs read the same
+    const char *tree_option = backend_option("TIRAMISU_AST_FROM_SCHEDULE_TREE");
+    const std::string tree_mode = tree_option ? tree_option : "0";
+    isl_schedule *tree = nullptr;
+    if (tree_mode != "0") {
+        std::vector<scheduled_statement> statements;
+        int dims = -1;
+        bool uniform = true;
+        isl_map_list *maps = isl_union_map_get_map_list(umap);
+        for (int i = 0; i < isl_map_list_n_map(maps); i++) {
+            isl_map *m = isl_map_list_get_map(maps, i);
+            const int nd = isl_map_dim(m, isl_dim_out);
+            if (dims >= 0 && nd != dims) uniform = false;
+            dims = nd;
+            statements.push_back({m, isl_pw_multi_aff_from_map(isl_map_copy(m))});
+        }
+        isl_map_list_free(maps);
+        if (uniform && !statements.empty()) {
+            std::vector<scheduled_statement *> all;
+            for (auto &s : statements) all.push_back(&s);
+            isl_schedule *start = isl_schedule_from_domain(isl_union_map_domain(isl_union_map_copy(umap)));
+            isl_schedule_node *root = isl_schedule_get_root(start);
+            isl_schedule_free(start);
+            isl_schedule_node *done = place(ctx, isl_schedule_node_child(root, 0), all, 0, dims);
+            if (done) {
+                tree = isl_schedule_node_get_schedule(done);
+                isl_schedule_node_free(done);
+            }
+        }
+        for (auto &s : statements) { isl_map_free(s.schedule); isl_pw_multi_aff_free(s.time); }
+        if (!tree && debug_level() >= 1) std::cout << "schedule of " << name << " is left to the flat form" << std::endl;
+    }
+    auto build_ast = [&](lowering &lw, bool from_tree) -> isl_ast_node * {
+        isl_ast_build *build = context_set ? isl_ast_build_from_context(isl_set_copy(context_set)) : isl_ast_build_alloc(ctx);
+        build = isl_ast_build_set_at_each_domain(build, &at_each_domain, &lw);
+        isl_ast_node *result;
+        if (from_tree) {
+            // loops take the names they have in the flat form, where every position of the time vector has a name
+            // and the loops sit at the odd ones: c1, c3, ...
+            int dims = 0;
+            isl_map_list *maps = isl_union_map_get_map_list(umap);
+            if (isl_map_list_n_map(maps) > 0) { isl_map *m = isl_map_list_get_map(maps, 0); dims = isl_map_dim(m, isl_dim_out); isl_map_free(m); }
+            isl_map_list_free(maps);
+            isl_id_list *names = isl_id_list_alloc(ctx, dims / 2 + 1);
+            for (int p = 1; p < dims; p += 2) names = isl_id_list_add(names, isl_id_alloc(ctx, ("c" + std::to_string(p)).c_str(), nullptr));
+            build = isl_ast_build_set_iterators(build, names);
+            result = isl_ast_build_node_from_schedule(build, isl_schedule_copy(tree));
+        } else {
+            result = isl_ast_build_node_from_schedule_map(build, isl_union_map_copy(umap));
+        }
+        isl_ast_build_free(build);
+        return result;
+    };
+
     lowering lw;
     lw.f = this;
-    isl_ast_build *build = context_set ? isl_ast_build_from_context(isl_set_copy(context_set)) : isl_ast_build_alloc(ctx);
-    build = isl_ast_build_set_at_each_domain(build, &at_each_domain, &lw);
-    ast = isl_ast_build_node_from_schedule_map(build, umap);
-    isl_ast_build_free(build);
+    const bool use_tree = tree && tree_mode == "1";
+    ast = build_ast(lw, use_tree);
     if (!ast) ERROR("isl failed to generate an AST for " + name, true);
 
     lowered.reset(new lir::program());
     lowered->fct = this;
     lowered->root = convert(lw, ast);
     apply_tags(this, lowered->root);
+    if (tree && tree_mode == "check") {
+        lowering other;
+        other.f = this;
+        isl_ast_node *second = build_ast(other, true);
+        if (!second) ERROR("isl failed to generate an AST for " + name + " from the schedule tree", true);
+        node_ptr root2 = convert(other, second);
+        apply_tags(this, root2);
+        isl_ast_node_free(second);
+        const std::string a = lir::dump(lowered->root), b = lir::dump(root2);
+        if (a != b) std::cerr << "---- from the schedule map\n" << a << "---- from the schedule tree\n" << b
+                              << "schedule tree check: " << name << " gives another program text than its schedule map" << std::endl;
+        else std::cerr << "schedule tree check: " << name << " gives the same program both ways" << std::endl;
+    } else if (tree_mode == "check") {
+        std::cerr << "schedule tree check: " << name << " is left to the flat form" << std::endl;
+    }
+    if (tree) isl_schedule_free(tree);
+    isl_union_map_free(umap);
 
     // Function-wide constants: literal-indexed reads of argument buffers, or plain expressions.
     for (auto c : invariants) {
