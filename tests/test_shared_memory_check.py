@@ -74,6 +74,43 @@ def test_reference_sgemm_generators_pass_the_check(tmp_path, stem):
     assert "__shared__" in text and "__syncthreads" in text
 
 
+STUBS = {"HIPCC_PATH": "/bin/true", "TIRAMISU_HOST_CXX": "/bin/true"}      # the check runs before any code is emitted
+
+
+@pytest.mark.parametrize("gen", ["gen_convolutiongpu_tiramisu", "gen_heat2dgpu_tiramisu", "gen_tutorial_04gpu2"])
+def test_reference_programs_with_run_time_sizes_are_analysed_and_pass(tmp_path, gen):
+    """benchmarks/halide/convolutiongpu_tiramisu.cpp (an 18 x 18 LDS tile filled by four guarded copies),
+    heat2dgpu_tiramisu.cpp and tutorial_04gpu2: image sizes known only at run time, so the thread loops' bounds are
+    min(15, N - 16 block - 1) and the halo copies' guards mix thread and size terms; the check takes the constant
+    side of such bounds and the decidable side of such guards, analyses every access and finds nothing."""
+    path = os.path.join(ROOT, "tests", "reference_programs", "build", gen)
+    if not os.path.exists(path):
+        pytest.skip("the reference's generators are built only where its sources are")
+    r = run_generator(path, tmp_path, env=dict(STUBS, TIRAMISU_HIP_CHECK_SHARED_MEMORY="1"))
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "LDS race check" not in r.stdout
+
+
+def test_the_reference_hand_staged_lstm_has_races(tmp_path):
+    """benchmarks/DNN/blocks/LSTM/gpu/generator.cpp:212-236 orders, inside the loop over 16-wide slices, the product
+    that reads the LDS tiles, one sync, the stores of the next slice into the tiles -- and then the next round's
+    product with nothing in between (and for the second product: stores, sync, product, next round's stores).  The
+    check names all four: a write of one round against the reads of the next on both tiles of the first product,
+    reads against the next round's writes on both tiles of the second."""
+    path = os.path.join(ROOT, "tests", "reference_programs", "build", "lstm_gpu", "gen")
+    if not os.path.exists(path):
+        pytest.skip("the reference's generators are built only where its sources are")
+    r = run_generator(path, tmp_path, env=dict(STUBS, TIRAMISU_HIP_CHECK_SHARED_MEMORY="warn"))
+    assert r.returncode == 0, r.stdout[-2000:]
+    found = [l for l in r.stdout.split("\n") if l.startswith("LDS race check: no sync between")]
+    assert len(found) == 4, r.stdout[-3000:]
+    for tile, first in (("b_m1_R_shr", "writes"), ("b_m1_h_shr", "writes"), ("b_m2_W_shr", "reads"), ("b_m2_h_shr", "reads")):
+        assert any((first + " " + tile) in l.split('" and "')[0] and tile in l.split('" and "')[1] for l in found), tile
+    # with "1" the same findings stop code generation
+    r = run_generator(path, tmp_path, env=dict(STUBS, TIRAMISU_HIP_CHECK_SHARED_MEMORY="1"))
+    assert r.returncode != 0 and "not separated by a sync" in r.stdout
+
+
 @pytest.mark.gpu
 def test_gpu_kernels_with_hand_declared_lds_match_numpy(programs_dir):
     from gpu_util import DeviceArray

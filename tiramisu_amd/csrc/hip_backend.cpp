@@ -146,6 +146,15 @@ struct generic_kernel_gen {
         const op_t op = e.get_op_type();
         if (op == o_access || op == o_call || op == o_address_of || op == o_lin_index || op == o_buffer) return false;
         const int n = e.get_n_arg();
+        if ((op == o_logical_and || op == o_logical_or) && n == 2) {
+            // one side may be known only at run time: false && x is false, true || x is true
+            const bool has_a = evaluate(e.get_operand(0), env, a), has_b = evaluate(e.get_operand(1), env, b);
+            const long decides = op == o_logical_and ? 0 : 1;
+            if ((has_a && (a != 0) == decides) || (has_b && (b != 0) == decides)) { out = decides; return true; }
+            if (!has_a || !has_b) return false;
+            out = op == o_logical_and ? (a && b) : (a || b);
+            return true;
+        }
         if (n >= 1 && !evaluate(e.get_operand(0), env, a)) return false;
         if (op == o_select || op == o_cond) {           // only the branch taken must evaluate
             return n == 3 && evaluate(e.get_operand(a ? 1 : 2), env, out);
@@ -177,6 +186,20 @@ struct generic_kernel_gen {
         case o_left_shift: out = a << b; return true;
         default: return false;
         }
+    }
+    // A loop bound for the enumeration: its value, or -- for min(a, b) as an upper bound and max(a, b) as a lower one,
+    // the shape of a partial tile's bound -- the side that has a value.  That may run through more iterations than
+    // the loop has (threads that a guard keeps out), which can add findings but cannot hide one.
+    static bool evaluate_bound(const expr &e, const std::map<std::string, long> &env, bool upper, long &out) {
+        if (evaluate(e, env, out)) return true;
+        if (!e.is_defined() || e.get_expr_type() != e_op) return false;
+        if (e.get_op_type() == o_cast && e.get_n_arg() == 1) return evaluate_bound(e.get_operand(0), env, upper, out);
+        if (e.get_op_type() != (upper ? o_min : o_max) || e.get_n_arg() != 2) return false;
+        long a = 0, b = 0;
+        const bool has_a = evaluate_bound(e.get_operand(0), env, upper, a), has_b = evaluate_bound(e.get_operand(1), env, upper, b);
+        if (!has_a && !has_b) return false;
+        out = has_a && has_b ? (upper ? std::min(a, b) : std::max(a, b)) : has_a ? a : b;
+        return true;
     }
     static bool contains_sync(const node_ptr &n) {
         bool found = false;
@@ -227,7 +250,7 @@ struct generic_kernel_gen {
                 }
                 const node_ptr &l = run_through[d];
                 long first = 0, last = 0, step = 1;
-                if (!evaluate(l->init, at, first) || !evaluate(l->upper, at, last) ||
+                if (!evaluate_bound(l->init, at, false, first) || !evaluate_bound(l->upper, at, true, last) ||
                     (l->increment.is_defined() && !evaluate(l->increment, at, step)) || step <= 0) { acc.known = false; return; }
                 for (long v = first; v <= last && acc.known; v += step) {
                     at[l->iterator] = v;
@@ -288,10 +311,11 @@ struct generic_kernel_gen {
                 return;
             case node_kind::loop: {
                 long first = 0, last = 0, step = 1;
-                const bool bounded = evaluate(n->init, env, first) && evaluate(n->upper, env, last) &&
+                const bool bounded = evaluate_bound(n->init, env, false, first) && evaluate_bound(n->upper, env, true, last) &&
                                      (!n->increment.is_defined() || evaluate(n->increment, env, step)) && step > 0;
                 if (n->gpu_block >= 0) {
-                    if (bounded) env[n->iterator] = first;
+                    // the first workgroup stands for all: only the first value is needed, not how many there are
+                    if (evaluate_bound(n->init, env, false, first)) env[n->iterator] = first;
                     go(n->body);
                     env.erase(n->iterator);
                 } else if (n->gpu_thread >= 0 || !contains_sync(n->body)) {
