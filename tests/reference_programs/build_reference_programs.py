@@ -66,8 +66,7 @@ def build_test(generator_rel, wrapper_rel):
 
 
 # The lattice-QCD correlator benchmarks for the GPU whose code this build generates in seconds (complex fp64
-# arithmetic through utils/complex_util.h, six kernels each; the four dibaryon programs take from ten minutes
-# upwards to generate and are left out).  Each wrapper fills random propagators and wave functions, calls the
+# arithmetic through utils/complex_util.h, six kernels each; the dibaryon programs are further down).  Each wrapper fills random propagators and wave functions, calls the
 # generated function and the plain C++ restatement its authors wrote next to it (<...>_ref.cpp, which the wrapper
 # includes), and compares the correlators to a relative 1e-12.  Built like the tests above: generator unchanged,
 # wrapper unchanged, its main() renamed so that a test can call it in-process.
@@ -95,15 +94,17 @@ def build_baryon(rel):
                ["-L" + build.PKG, "-ltiramisu_hip_wrappers", "-Wl,-rpath,$ORIGIN/" + os.path.relpath(build.PKG, bdir)])
 
 
-# One of the four dibaryon correlators (benchmarks/tensors/dibaryon/gpu_*): ten kernels, 1.3 MB of kernel source.
-# Compiling its generator takes four minutes and running it one (almost five with the AST built from the flat
+# Two of the four dibaryon correlators (benchmarks/tensors/dibaryon/gpu_*): ten kernels, 1.3 MB of kernel source each.  (The other
+# two build the same way -- build_dibaryon takes any of them -- but the one tried did not finish within ten minutes on the GPU.)
+# Compiling a generator takes four minutes and running it one (almost five with the AST built from the flat
 # schedule map: three quarters of that inside isl's ordering of the statements' domains), so it is built on request
 # only: TIRAMISU_BUILD_DIBARYON=1.
-# Its wrapper keeps the comparison with the authors' C++ restatement behind two switches that are off
+# Each wrapper keeps the comparison with the authors' C++ restatement behind two switches that are off
 # ("#define RUN_REFERENCE 0", "#define RUN_CHECK 0") and includes that restatement, standard headers and all, inside
 # an extern "C" block: the switches are flipped on the way into the compiler (the text goes through a pipe; nothing of
 # the reference is written anywhere) and the standard headers are included ahead of the file.
-DIBARYON = ["benchmarks/tensors/dibaryon/gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
+DIBARYON = ["benchmarks/tensors/dibaryon/gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator",
+            "benchmarks/tensors/dibaryon/gpu_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
 
 
 def build_dibaryon(rel):

@@ -200,7 +200,7 @@ def test_reference_gpu_test_passes(name):
     assert lib.tiramisu_wrapper_main(0, None) == 0
 
 
-DIBARYON = ["gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
+DIBARYON = ["gpu_single_tiramisu_make_fused_identical_dibaryon_blocks_correlator", "gpu_tiramisu_make_fused_identical_dibaryon_blocks_correlator"]
 BARYON = ["gpu_tiramisu_make_fused_baryon_blocks_correlator", "gpu_tiramisu_make_fused_identical_baryon_blocks_correlator",
           "gpu_single_tiramisu_make_fused_identical_baryon_blocks_correlator"]
 
@@ -236,7 +236,9 @@ def test_reference_dibaryon_correlator_passes_its_own_check(name):
     """benchmarks/tensors/dibaryon/gpu_single_...: generator unchanged; the wrapper with its two switches
     (RUN_REFERENCE, RUN_CHECK) on, so that it runs the authors' C++ restatement and compares every correlator entry
     with the generated function's (ten kernels; kernels inside host loops take the loops' iterators as parameters
-    in a program with 64-bit loop iterators).  Built on request only (TIRAMISU_BUILD_DIBARYON=1: about ten minutes)."""
+    in a program with 64-bit loop iterators; in the second program statements tagged (block, thread) are fused at
+    their second level with statements tagged (block, block, thread, thread), and their accumulations have no
+    thread loop around them).  Built on request only (TIRAMISU_BUILD_DIBARYON=1: about ten minutes each)."""
     if not os.path.exists(library(name)):
         pytest.skip("built on request only: TIRAMISU_BUILD_DIBARYON=1 python tests/reference_programs/build_reference_programs.py")
     runtime.wrappers()

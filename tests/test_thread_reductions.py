@@ -80,9 +80,10 @@ def test_gpu_matches_numpy(programs_dir, name):
 def test_sum_across_wavefronts_under_a_condition_keeps_the_barrier_out(programs_dir):
     """tests/programs/thread_reduction_under_condition.cpp: the 256-thread loop sits under `if (block iterator >= 3)`.
     The lowering across wavefronts ends in a workgroup barrier that every thread must reach, so the emitter must not
-    use it below a condition: the kernel stays as the program states it (no LDS stage, no barrier)."""
+    use it below a condition: the loop stays as the program states it (no LDS stage, no barrier below the condition)."""
     text = open(os.path.join(programs_dir, "build", "row_sums_from_row_3.o.hip")).read()
     kernel = text[text.index('extern "C" __global__'):]
     assert "if ((c1 >= 3))" in kernel
-    assert "block_group_sum" not in kernel and "__syncthreads" not in kernel
+    # (the initialisation above the condition, which no thread loop encloses, runs on the first thread between barriers)
+    assert "block_group_sum" not in kernel and "__syncthreads" not in kernel[kernel.index("if ((c1 >= 3))"):]
     assert "DPP wavefront reductions" not in re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)

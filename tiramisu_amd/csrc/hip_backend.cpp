@@ -94,6 +94,11 @@ struct generic_kernel_gen {
         lir::walk(root, [&](const node_ptr &n) {
             if (n->kind == node_kind::loop) {
                 inner.insert(n->iterator);
+                // Statements fused into one nest may disagree about a loop level: a block dimension for those tagged
+                // (block, block, thread, thread), a thread dimension for those tagged (block, thread).  The loop can be
+                // one thing only: it is a block dimension (which is how it is emitted), and the statements that took
+                // it for their thread loop have no thread loop around them any more (they run once per workgroup, below).
+                if (n->gpu_block >= 0 && n->gpu_thread >= 0) { n->gpu_thread = -1; conflicting_tags = true; }
                 if (n->gpu_block >= 0) loops_per_dim[0][n->gpu_block]++;
                 if (n->gpu_thread >= 0) loops_per_dim[1][n->gpu_thread]++;
             }
@@ -109,6 +114,7 @@ struct generic_kernel_gen {
             std::vector<node_ptr> stack;
             find_reductions(root, stack);
         }
+        if (kernel_has_thread_loops()) mark_once_per_workgroup(root);
         check_shared_memory(root);
     }
 
@@ -298,6 +304,7 @@ struct generic_kernel_gen {
         };
         std::function<void(const node_ptr &)> go = [&](const node_ptr &n) {
             if (!n) return;
+            if (once_per_workgroup.count(n.get())) { pending.clear(); return; }     // one thread, a barrier before and after
             switch (n->kind) {
             case node_kind::block:
                 for (auto &c : without_redundant_barriers(n->children)) go(c);
@@ -409,6 +416,7 @@ struct generic_kernel_gen {
                     const memory_location where = n->lhs->get_location();
                     if (where == memory_location::global || where == memory_location::host || where == memory_location::shared)
                         for (int d = 0; d < 3; d++) {
+                            if (it[d].empty() && loops_per_dim[1][d] > 0) veto = true;    // outside that dimension's thread loops: runs once per workgroup (below)
                             if (it[d].empty()) continue;
                             bool involved = false;
                             for (auto &e : n->lhs_index) involved = involved || lir::mentions(e, it[d]);
@@ -846,7 +854,71 @@ struct generic_kernel_gen {
         return v;
     }
 
+    // ---- statements that no thread loop encloses.  The program means them to run once per iteration of the loops
+    // around them (sequential semantics; on the CPU they do), but every thread of the workgroup reaches them: stores
+    // of the same value are merely repeated, an accumulation (x = x + ...) is wrong -- the reference's CUDA printer
+    // emits them as they stand (tiramisu_codegen_cuda.cpp: a thread loop becomes an index and a guard, what lies
+    // outside it is code of every thread).  Here a statement or loop nest outside all thread loops that writes memory
+    // the other threads see (global, LDS) runs on the workgroup's first thread, between two barriers: what the
+    // thread loops before it wrote is there, and what it writes is there for the thread loops after it.  The barriers
+    // are reached by all threads: nothing thread-dependent encloses such a statement.  Statements that write a
+    // thread's own registers or arrays stay as they are -- every thread needs them.
+    std::set<const node *> once_per_workgroup;       // roots of such subtrees (filled by mark_once_per_workgroup)
+    bool kernel_has_thread_loops() const { return loops_per_dim[1][0] + loops_per_dim[1][1] + loops_per_dim[1][2] > 0; }
+    bool may_run_on_one_thread(const node_ptr &n) const {
+        bool ok = true, writes = false;
+        lir::walk(n, [&](const node_ptr &x) {
+            if (x->kind == node_kind::loop && (x->gpu_thread >= 0 || x->gpu_block >= 0)) ok = false;
+            if (x->kind != node_kind::leaf) return;
+            if (x->lkind == leaf_kind::call) { writes = true; return; }
+            if (x->lkind != leaf_kind::assign || !x->lhs) { ok = false; return; }      // declarations, lets, barriers, copies
+            const memory_location where = x->lhs->get_location();
+            if (where == memory_location::global || where == memory_location::host || where == memory_location::shared) writes = true;
+            else ok = false;
+        });
+        return ok && writes;
+    }
+    void mark_once_per_workgroup(const node_ptr &n) {
+        if (!n || backend_option("TIRAMISU_HIP_EVERY_THREAD_RUNS_ALL")) return;
+        if (n->kind == node_kind::loop && n->gpu_thread >= 0) return;               // below a thread loop everything is per thread
+        if (n->kind != node_kind::block && may_run_on_one_thread(n)) { once_per_workgroup.insert(n.get()); return; }
+        for (auto &c : n->children) mark_once_per_workgroup(c);
+        mark_once_per_workgroup(n->body);
+        mark_once_per_workgroup(n->then_body);
+        mark_once_per_workgroup(n->else_body);
+    }
+    void emit_on_first_thread(const std::vector<node_ptr> &nodes, int ind) {
+        std::string first;
+        for (int d = 0; d < 3; d++)
+            if (loops_per_dim[1][d] > 0) first += std::string(first.empty() ? "" : " && ") + "threadIdx." + "xyz"[d] + " == 0";
+        body << pad(ind) << "__syncthreads();\n";
+        body << pad(ind) << "if (" << first << ") {   // once per workgroup: no thread loop around these statements\n";
+        for (auto &c : nodes) emit_node(c, ind + 1);
+        body << pad(ind) << "}\n";
+        body << pad(ind) << "__syncthreads();\n";
+        statements_on_first_thread = true;
+    }
+    bool statements_on_first_thread = false;
+    bool conflicting_tags = false;
+
     void emit(const node_ptr &n, int ind) {
+        if (!n) return;
+        if (n->kind == node_kind::block) {
+            // neighbours that run once share one pair of barriers
+            std::vector<node_ptr> run;
+            for (auto &c : without_redundant_barriers(n->children)) {
+                if (once_per_workgroup.count(c.get())) { run.push_back(c); continue; }
+                if (!run.empty()) { emit_on_first_thread(run, ind); run.clear(); }
+                emit(c, ind);
+            }
+            if (!run.empty()) emit_on_first_thread(run, ind);
+            return;
+        }
+        if (once_per_workgroup.count(n.get())) { emit_on_first_thread({n}, ind); return; }
+        emit_node(n, ind);
+    }
+
+    void emit_node(const node_ptr &n, int ind) {
         if (!n) return;
         switch (n->kind) {
         case node_kind::block:
@@ -1055,6 +1127,8 @@ static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const
     if (g.wave_reductions)
         k.how += ", " + std::to_string(g.wave_reductions) + " sum(s) across the threads of a loop lowered to DPP wavefront reductions" +
                  (g.needs_reduction_scratch ? " (wavefront totals combined through LDS)" : "");
+    if (g.conflicting_tags) k.how += ", a loop tagged as a block dimension by some statements and as a thread dimension by others is a block dimension";
+    if (g.statements_on_first_thread) k.how += ", statements outside the thread loops run on the workgroup's first thread between barriers";
     k.name = "_kernel_" + std::to_string(ctx.next_kernel_id());
     function *f = ctx.f;
 
