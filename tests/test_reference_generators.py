@@ -241,6 +241,8 @@ def test_reference_dibaryon_correlator_passes_its_own_check(name):
     thread loop around them).  Built on request only (TIRAMISU_BUILD_DIBARYON=1: about ten minutes each)."""
     if not os.path.exists(library(name)):
         pytest.skip("built on request only: TIRAMISU_BUILD_DIBARYON=1 python tests/reference_programs/build_reference_programs.py")
+    if os.environ.get("TIRAMISU_RUN_DIBARYON") != "1":
+        pytest.skip("a minute and a half each, most of it the wrapper's own set-up on the host: run with TIRAMISU_RUN_DIBARYON=1")
     runtime.wrappers()
     lib = ctypes.CDLL(library(name))
     lib.tiramisu_wrapper_main.restype = ctypes.c_int
