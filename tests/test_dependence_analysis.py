@@ -104,3 +104,18 @@ def test_codegen_refuses_a_race_when_asked_to_check(tmp_path):
     assert r.returncode != 0
     assert "S: loop j (level 1, mapped to threadIdx) carries a dependence" in r.stdout
     assert not os.path.exists(tmp_path / "build" / "scan_rows_refused.o")
+
+
+def test_the_check_of_mapped_loops_has_a_time_limit(tmp_path):
+    """The analysis is one isl dataflow computation over the whole function and has no natural bound; it runs in a child
+    process under hip_check_time_limit seconds (default 600).  With a limit of one second the LSTM program's check is
+    stopped, says so, and code generation goes on (device and host compilers stubbed out here)."""
+    gen = os.path.join(os.path.dirname(BUILD), "..", "..", "tiramisu_amd", "programs", "build", "gen_lstm")
+    gen = os.path.abspath(gen)
+    assert os.path.exists(gen), "run __graft_entry__.build() first"
+    os.makedirs(tmp_path / "build")
+    env = dict(os.environ, TIRAMISU_HIP_CHECK_MAPPED_LOOPS="1", TIRAMISU_HIP_CHECK_TIME_LIMIT="1", HIPCC_PATH="/bin/true", TIRAMISU_HOST_CXX="/bin/true")
+    r = subprocess.run([gen], cwd=tmp_path, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "the dependence analysis of lstm_4x64x512x100 did not finish within 1 s and was stopped" in r.stdout
+    assert os.path.exists(tmp_path / "build" / "lstm_4x64x512x100.o.hip")

@@ -3,6 +3,9 @@
 // time-space vector [dup, s0, d0, s1, d1, ..., d(n-1), sn] (static ordering dimensions s_k
 // interleaved with dynamic loop dimensions d_k), as in the reference
 // (src/tiramisu_core.cpp:2041-2081, :7640-7662); every command is a rewrite of the range.
+#include <csignal>
+#include <sys/wait.h>
+#include <unistd.h>
 #include <tiramisu/block.h>
 #include <tiramisu/core.h>
 
@@ -427,7 +430,50 @@ void function::codegen(const std::vector<buffer *> &arguments, const std::string
     set_arguments(arguments);
     gen_time_space_domain();
     if (arch == hardware_architecture_t::arch_amd_gpu && backend_option("TIRAMISU_HIP_CHECK_MAPPED_LOOPS")) {
-        const std::vector<std::string> races = gpu_mapped_loops_that_carry_dependences();
+        // The analysis is one isl dataflow computation over the whole function and has no natural bound (a tensor
+        // contraction with hundreds of statements: more than 40 minutes), so it runs in a child process with a time
+        // limit (option hip_check_time_limit, seconds, default 600; 0: in this process, without one).  A check that
+        // does not finish says so and stops nothing.
+        const char *limit_text = backend_option("TIRAMISU_HIP_CHECK_TIME_LIMIT");
+        const int limit = limit_text ? std::atoi(limit_text) : 600;
+        std::vector<std::string> races;
+        bool finished = true;
+        if (limit <= 0) {
+            races = gpu_mapped_loops_that_carry_dependences();
+        } else {
+            int fd[2];
+            if (pipe(fd) != 0) ERROR("pipe() failed", true);
+            std::cout.flush();
+            std::cerr.flush();
+            const pid_t child = fork();
+            if (child < 0) ERROR("fork() failed", true);
+            if (child == 0) {
+                close(fd[0]);
+                alarm((unsigned)limit);
+                std::string all;
+                for (auto &r : gpu_mapped_loops_that_carry_dependences()) all += r + "\n";
+                size_t off = 0;
+                while (off < all.size()) {
+                    const ssize_t n = write(fd[1], all.data() + off, all.size() - off);
+                    if (n <= 0) break;
+                    off += (size_t)n;
+                }
+                _exit(0);
+            }
+            close(fd[1]);
+            std::string all;
+            char buf[4096];
+            for (ssize_t n; (n = read(fd[0], buf, sizeof buf)) > 0;) all.append(buf, (size_t)n);
+            close(fd[0]);
+            int status = 0;
+            waitpid(child, &status, 0);
+            finished = WIFEXITED(status) && WEXITSTATUS(status) == 0;
+            if (!finished && !(WIFSIGNALED(status) && WTERMSIG(status) == SIGALRM)) ERROR("the check of the GPU mapping ended abnormally", true);
+            for (size_t a = 0, b; (b = all.find('\n', a)) != std::string::npos; a = b + 1) races.push_back(all.substr(a, b - a));
+        }
+        if (!finished)
+            std::cerr << "GPU mapping: the dependence analysis of " << name << " did not finish within " << limit
+                      << " s and was stopped: its mapped loops are not checked (hip_check_time_limit sets the limit)" << std::endl;
         bool refuse = false;
         for (auto &r : races) {
             std::cerr << "GPU mapping: " << r << std::endl;
