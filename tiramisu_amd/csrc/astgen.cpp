@@ -383,6 +383,56 @@ void apply_tags(function *f, const node_ptr &root) {
     });
 }
 
+// isl leaves no loop node where a loop level has a single iteration, so a statement all of whose tagged levels are of
+// that kind (a domain of one point; in general one that fits in a single tile of extent one per tagged dimension)
+// would stay on the host with its GPU buffers -- the reference has the same gap ("TODO check if degenerate",
+// tiramisu_codegen_cuda.cpp:252).  The largest subtrees that consist of such statements alone become the body of a
+// block loop of one iteration, placed inside the loops that lie outside the statements' first tagged level: a kernel
+// of one workgroup.
+// first loop level at which the statement is tagged for the GPU, -1 when it has no such tag
+int first_gpu_level(function *f, const node *leaf) {
+    if (!leaf->comp) return -1;
+    const std::string &cn = leaf->comp->get_name();
+    for (int level = 0; level < 32; level++)
+        if (f->gpu_block_position(cn, level) >= 0 || f->gpu_thread_position(cn, level) >= 0) return level;
+    return -1;
+}
+
+void keep_on_gpu(function *f, node_ptr &n) {
+    if (!n) return;
+    if (n->kind == node_kind::loop && (n->gpu_block >= 0 || n->gpu_thread >= 0)) return;
+    std::vector<node *> leaves;
+    collect_leaves(n, leaves);
+    bool alone = !leaves.empty();
+    int outermost = 32;
+    for (auto l : leaves) {
+        const int first = first_gpu_level(f, l);
+        if (first < 0) alone = false;
+        else outermost = std::min(outermost, first);
+    }
+    // loops outside the statements' first tagged level stay around the kernel (host loops, one launch per iteration)
+    lir::walk(n, [&](const node_ptr &x) {
+        if (x->kind != node_kind::loop) return;
+        if (x->gpu_block >= 0 || x->gpu_thread >= 0 || (x->level >= 0 && x->level < outermost)) alone = false;
+    });
+    if (alone) {
+        node_ptr once = std::make_shared<node>();
+        once->kind = node_kind::loop;
+        once->iterator = "_single_iteration";
+        once->init = expr((int32_t)0);
+        once->upper = expr((int32_t)0);
+        once->increment = expr((int32_t)1);
+        once->gpu_block = 0;
+        once->body = n;
+        n = once;
+        return;
+    }
+    for (auto &c : n->children) keep_on_gpu(f, c);
+    keep_on_gpu(f, n->body);
+    keep_on_gpu(f, n->then_body);
+    keep_on_gpu(f, n->else_body);
+}
+
 }  // namespace
 
 namespace {
@@ -533,6 +583,7 @@ void function::gen_isl_ast() {
     lowered->fct = this;
     lowered->root = convert(lw, ast);
     apply_tags(this, lowered->root);
+    keep_on_gpu(this, lowered->root);
     if (tree && tree_mode == "check") {
         lowering other;
         other.f = this;
@@ -540,6 +591,7 @@ void function::gen_isl_ast() {
         if (!second) ERROR("isl failed to generate an AST for " + name + " from the schedule tree", true);
         node_ptr root2 = convert(other, second);
         apply_tags(this, root2);
+        keep_on_gpu(this, root2);
         isl_ast_node_free(second);
         const std::string a = lir::dump(lowered->root), b = lir::dump(root2);
         if (a != b) std::cerr << "---- from the schedule map\n" << a << "---- from the schedule tree\n" << b
