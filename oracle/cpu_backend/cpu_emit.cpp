@@ -209,7 +209,7 @@ public:
         if (!h) ERROR("cannot write " + src, true);
         h << "// Generated by the CPU back-end restatement (parity oracle). Function: " << f.get_name() << "\n";
         h << "#include <stdint.h>\n#include <stdlib.h>\n#include <string.h>\n#include <math.h>\n";
-        h << halide_buffer_definition() << c_prelude(false) << "\n";
+        h << halide_buffer_definition() << c_prelude(false) << c_prelude_opaque(false, body.str()) << "\n";
         for (auto &d : g.extern_decls) h << d << "\n";
         h << "extern \"C\" int " << f.get_name() << "(";
         for (size_t i = 0; i < args.size(); i++) h << (i ? ", " : "") << "halide_buffer_t *_a" << i;

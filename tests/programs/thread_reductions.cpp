@@ -7,7 +7,13 @@
 //  * gemv_wavefront        y(i) = sum_j A(i,j) x(j), 300 x 1000: four rows per workgroup, the 64 lanes
 //                          of a wavefront share a row (ragged: 1000 = 15 x 64 + 40);
 //  * row_sums_quarter_wave s(i) = 1 + sum_j A(i,j), 128 x 50: 16 lanes per row, four rows per wavefront;
-//  * row_sums_block        s(i) = sum_j A(i,j), 40 x 5000: 256 threads (four wavefronts) per row.
+//  * row_sums_block        s(i) = sum_j A(i,j), 40 x 5000: 256 threads (four wavefronts) per row;
+//  * row_sums_ragged_rows_block  10 x 558, four rows of 256 threads per workgroup: the last workgroup has two rows
+//                          only, and its other 512 threads must still reach the barrier of the sum across wavefronts
+//                          (the row loop is emitted with a predicate instead of a branch);
+//  * row_sums_100_lanes    31 x 450, two rows of 100 threads: the width is rounded up to two wavefronts, the lanes
+//                          beyond the loop's extent add zero (and the last workgroup has one row);
+//  * row_sums_26_of_64_lanes  80 x 26 split by 64: the thread loop has 26 iterations, the sum runs on 32 lanes.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -75,5 +81,8 @@ int main()
     gemv_wavefront();
     row_sums("row_sums_quarter_wave", 128, 50, 16, 16);
     row_sums("row_sums_block", 40, 5000, 1, 256);
+    row_sums("row_sums_ragged_rows_block", 10, 558, 4, 256);
+    row_sums("row_sums_100_lanes", 31, 450, 2, 100);
+    row_sums("row_sums_26_of_64_lanes", 80, 26, 1, 64);
     return 0;
 }

@@ -18,7 +18,11 @@ CASES = {
     "gemv_wavefront": (300, 1000, 0.0, True),
     "row_sums_quarter_wave": (128, 50, 1.0, False),
     "row_sums_block": (40, 5000, 0.0, False),
+    "row_sums_ragged_rows_block": (10, 558, 1.0, False),
+    "row_sums_100_lanes": (31, 450, 1.0, False),
+    "row_sums_26_of_64_lanes": (80, 26, 0.0, False),
 }
+ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes"}
 
 
 def inputs(name, integer, seed):
@@ -44,8 +48,29 @@ def test_lowered_to_wavefront_reductions(programs_dir, name):
     text = open(os.path.join(programs_dir, "build", name + ".o.hip")).read()
     how = re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)
     assert "DPP wavefront reductions" in how
-    assert ("through LDS" in how) == (name == "row_sums_block")
+    assert ("through LDS" in how) == (name in ACROSS_WAVEFRONTS)
     assert "twave::" in text and "_partial0" in text
+
+
+def test_rows_beyond_the_last_tile_carry_a_predicate_and_reach_the_barrier(programs_dir):
+    """Four rows of 256 threads per workgroup, 10 rows: the row loop's guard must not enclose the sum across
+    wavefronts (its barrier is for every thread); the statements run under a predicate instead."""
+    text = open(os.path.join(programs_dir, "build", "row_sums_ragged_rows_block.o.hip")).read()
+    kernel = text[text.index('extern "C" __global__'):]
+    assert "const bool _live_c3 = " in kernel
+    at = kernel.index("block_group_sum<256>")
+    before = kernel[:at]
+    assert before.count("{") - before.count("}") == 4        # kernel, block loop, row loop, the sum's own scope: no `if` open
+    assert "if (threadIdx.x == 255 && _live_c3)" in kernel
+
+
+def test_a_width_between_the_supported_ones_is_rounded_up(programs_dir):
+    for name, width, last in (("row_sums_100_lanes", "block_group_sum<128>", 99), ("row_sums_26_of_64_lanes", "wave_group_sum<32>", 25)):
+        text = open(os.path.join(programs_dir, "build", name + ".o.hip")).read()
+        assert width in text
+        assert re.search(r"c5 >= 0 && c5 <= %d\)" % last, text), name       # the lanes beyond the loop's extent add nothing
+        host = open(os.path.join(programs_dir, "build", name + ".o.host.cpp")).read()
+        assert re.search(r"_block\[3\] = \{\(uint32_t\)\((128|32)\)", host)
 
 
 @pytest.mark.parametrize("name", sorted(CASES))
@@ -87,3 +112,16 @@ def test_sum_across_wavefronts_under_a_condition_keeps_the_barrier_out(programs_
     # (the initialisation above the condition, which no thread loop encloses, runs on the first thread between barriers)
     assert "block_group_sum" not in kernel and "__syncthreads" not in kernel[kernel.index("if ((c1 >= 3))"):]
     assert "DPP wavefront reductions" not in re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)
+
+
+def test_a_sum_left_as_scheduled_is_reported(programs_dir, tmp_path):
+    """... and the generator says that the threads of that loop race (the reference emits such sums silently,
+    tiramisu_codegen_cuda.cpp:549-707)."""
+    import subprocess
+    os.makedirs(os.path.join(str(tmp_path), "build"))
+    env = dict(os.environ, HIPCC_PATH="/bin/true", TIRAMISU_HOST_CXX="/bin/true")
+    r = subprocess.run([os.path.join(programs_dir, "build", "gen_thread_reduction_under_condition")], cwd=str(tmp_path), env=env,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    assert "GPU mapping: the sum s over thread loop c3 of row_sums_from_row_3 is emitted as scheduled, its threads race on" in r.stdout, r.stdout
+    assert "under a condition" in r.stdout

@@ -120,6 +120,13 @@ std::string c_printer::print(const expr &e) const {
     const bool narrow = t == p_uint8 || t == p_int8 || t == p_uint16 || t == p_int16;
     auto keep = [&](const std::string &v) { return narrow ? "((" + primitive_c_name(t) + ")" + v + ")" : v; };
     auto bin = [&](const char *sym) { return "(" + P(0) + " " + sym + " " + P(1) + ")"; };
+    // hipcc 7.2 for gfx950 has been seen to compute (int8_t)((int8_t)(a * b) / 2) wrongly (x + 3 instead of x / 2 for
+    // most inputs; gcc and the host side of the same clang are right): the truncation of a signed narrow product is
+    // folded into a following operation that depends on its sign.  The products of signed 8- and 16-bit values, and
+    // the left operands of their /, % and >>, therefore pass through t_opaque(): on the device an empty asm statement
+    // that hands the sign-extended value back as one the optimiser knows nothing about, on the host the identity.
+    const bool narrow_signed = t == p_int8 || t == p_int16;
+    auto bin_opaque_left = [&](const char *sym) { return "(t_opaque(" + P(0) + ") " + sym + " " + P(1) + ")"; };
     if (const char *m = math_name(o)) {
         std::string fn = m;
         if (t == p_float32 || t == p_bfloat16) fn += "f";
@@ -134,9 +141,9 @@ std::string c_printer::print(const expr &e) const {
         return "((" + primitive_c_name(t) + ")(" + P(0) + "))";
     case o_add: return keep(bin("+"));
     case o_sub: return keep(bin("-"));
-    case o_mul: return keep(bin("*"));
-    case o_div: return keep(bin("/"));
-    case o_mod: return is_float_type(t) ? "fmod(" + P(0) + ", " + P(1) + ")" : keep(bin("%"));
+    case o_mul: return narrow_signed ? "t_opaque(" + keep(bin("*")) + ")" : keep(bin("*"));
+    case o_div: return keep(narrow_signed ? bin_opaque_left("/") : bin("/"));
+    case o_mod: return is_float_type(t) ? "fmod(" + P(0) + ", " + P(1) + ")" : keep(narrow_signed ? bin_opaque_left("%") : bin("%"));
     case o_floordiv: return "t_floordiv(" + P(0) + ", " + P(1) + ")";
     case o_floormod: return "t_floormod(" + P(0) + ", " + P(1) + ")";
     case o_logical_and: return bin("&&");
@@ -149,7 +156,7 @@ std::string c_printer::print(const expr &e) const {
     case o_gt: return bin(">");
     case o_max: return "t_max(" + P(0) + ", " + P(1) + ")";
     case o_min: return "t_min(" + P(0) + ", " + P(1) + ")";
-    case o_right_shift: return keep(bin(">>"));
+    case o_right_shift: return keep(narrow_signed ? bin_opaque_left(">>") : bin(">>"));
     case o_left_shift: return keep(bin("<<"));
     case o_select: case o_cond: return "(" + P(0) + " ? " + P(1) + " : " + P(2) + ")";
     case o_lerp: return "t_lerp(" + P(0) + ", " + P(1) + ", " + P(2) + ")";
@@ -219,6 +226,14 @@ std::string c_prelude(bool device) {
           "if ((x.u & 0x7fffffffu) > 0x7f800000u) return (tiramisu_bf16_t)((x.u >> 16) | 0x40); "
           "uint32_t r = 0x7fffu + ((x.u >> 16) & 1u); return (tiramisu_bf16_t)((x.u + r) >> 16); }\n";
     return os.str();
+}
+
+// t_opaque (see c_printer::print), added to a generated file whose code uses it
+std::string c_prelude_opaque(bool device, const std::string &code) {
+    if (code.find("t_opaque(") == std::string::npos) return "";
+    if (device)
+        return "template <typename T> __device__ __forceinline__ T t_opaque(T v) { int32_t w = v; asm(\"\" : \"+v\"(w)); return (T)w; }\n";
+    return "template <typename T> static inline T t_opaque(T v) { return v; }\n";
 }
 
 std::string halide_buffer_definition() {

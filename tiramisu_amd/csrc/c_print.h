@@ -41,6 +41,7 @@ struct c_printer {
 /** Helper functions (floor division, min/max, bf16 conversion) that printed code relies on;
   * \p device selects __device__ qualifiers. */
 std::string c_prelude(bool device);
+std::string c_prelude_opaque(bool device, const std::string &code);
 /** Layout-compatible definition of halide_buffer_t for generated host code. */
 std::string halide_buffer_definition();
 

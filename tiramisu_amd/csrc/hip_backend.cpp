@@ -94,6 +94,7 @@ struct generic_kernel_gen {
         lir::walk(root, [&](const node_ptr &n) {
             if (n->kind == node_kind::loop) {
                 inner.insert(n->iterator);
+                loops_by_iterator[n->iterator].push_back(n);
                 // Statements fused into one nest may disagree about a loop level: a block dimension for those tagged
                 // (block, block, thread, thread), a thread dimension for those tagged (block, thread).  The loop can be
                 // one thing only: it is a block dimension (which is how it is emitted), and the statements that took
@@ -641,7 +642,7 @@ struct generic_kernel_gen {
     // a sum across the lanes of the wavefront with DPP row shifts and broadcasts (across wavefronts
     // through LDS when the loop is wider than a wavefront), and one read-modify-write of X[e] by the last
     // thread of the loop.
-    struct thread_reduction { node_ptr leaf; expr term; int width; };
+    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; };   // widened: width exceeds the loop's extent
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
     int conds_above = 0;          // conditions between the kernel's root and the node that find_reductions is visiting
@@ -692,51 +693,133 @@ struct generic_kernel_gen {
                 R = stack[d];
                 at = d;
             }
-        if (!R || loops_per_dim[1][0] != 1) return;
+        if (!R) return;
+        // From here on the statement is known to be a sum that all threads of loop R add to one element.  Where it
+        // is not lowered it is emitted as scheduled, like the reference does (tiramisu_codegen_cuda.cpp:549-707):
+        // the threads race and the result is wrong, so say so.
+        auto left_as_scheduled = [&](const std::string &why) {
+            std::cerr << "GPU mapping: the sum " << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
+                      << " is emitted as scheduled, its threads race on " << leaf->lhs->get_name() << " (" << why << ")" << std::endl;
+        };
+        if (loops_per_dim[1][0] != 1) return left_as_scheduled("another loop of the kernel is mapped to threadIdx.x as well");
         // inside it: this statement only, under serial loops whose iterators the element does not involve either
         for (size_t d = at + 1; d < stack.size(); d++)
-            if (stack[d]->gpu_thread >= 0 || stack[d]->gpu_block >= 0 || element_involves(stack[d]->iterator)) return;
+            if (stack[d]->gpu_thread >= 0 || stack[d]->gpu_block >= 0 || element_involves(stack[d]->iterator))
+                return left_as_scheduled("a loop inside the thread loop is mapped too, or selects the element");
         int leaves_inside = 0;
         lir::walk(R, [&](const node_ptr &x) { if (x->kind == node_kind::leaf) leaves_inside++; });
-        if (leaves_inside != 1) return;
-        // width of the loop = blockDim.x: a power of two up to a wavefront, or whole wavefronts
+        if (leaves_inside != 1) return left_as_scheduled("the thread loop holds other statements");
+        // width of the loop = blockDim.x: a power of two up to a wavefront, or whole wavefronts; an extent in between
+        // is rounded up (the lanes beyond the loop's last iteration are masked by the loop's guard and add zero)
         bool guard;
         expr first;
         const expr ext = lir::simplify(host_extent(R, first, guard));
-        if (!ext.is_integer_literal()) return;
-        const long w = ext.get_int_val();
-        const bool in_wave = w >= 2 && w <= 64 && (w & (w - 1)) == 0, waves = w >= 128 && w <= 1024 && w % 64 == 0;
-        if (!in_wave && !waves) return;
+        if (!ext.is_integer_literal()) return left_as_scheduled("the extent of the thread loop is not a constant");
+        const long extent = ext.get_int_val();
+        if (extent < 2 || extent > 1024) return left_as_scheduled("the extent of the thread loop is " + std::to_string(extent));
+        long w = extent;
+        if (w <= 64) while (w & (w - 1)) w++;
+        else w = (w + 63) / 64 * 64;
+        long other_threads = 1;
+        for (size_t d = 0; d < at; d++)
+            if (stack[d]->gpu_thread >= 0) {
+                bool g;
+                expr f0;
+                const expr e = lir::simplify(host_extent(stack[d], f0, g));
+                if (e.is_integer_literal()) other_threads *= e.get_int_val();
+            }
+        if (w != extent && w * other_threads > 1024)
+            return left_as_scheduled("rounded up to " + std::to_string(w) + " lanes the workgroup would exceed 1024 threads");
+        const bool waves = w > 64;
         if (waves) {
             // the barrier of the LDS stage must be reached by every thread: no guarded mapped loop around it,
             // no serial loop and no condition (a separated remainder, a hoisted predicate: it may depend on a
             // thread iterator) between the kernel entry and the loop.  (Adding the wavefronts' totals with
             // atomics instead would need no barrier, but nothing would then order them after an initialisation of
             // the element that other wavefronts of the workgroup execute: the barrier is what does that.)
-            if (conds_above > 0) return;
+            if (conds_above > 0) return left_as_scheduled("wider than a wavefront and under a condition: the barrier of the sum across wavefronts would not be reached by every thread");
+            std::vector<const node *> guarded;
             for (size_t d = 0; d < at; d++) {
                 bool g;
                 expr f0;
-                if (stack[d]->gpu_thread < 0 && stack[d]->gpu_block < 0) return;
+                if (stack[d]->gpu_thread < 0 && stack[d]->gpu_block < 0)
+                    return left_as_scheduled("wider than a wavefront and inside a serial loop");
                 host_extent(stack[d], f0, g);
-                const int dim = stack[d]->gpu_block >= 0 ? stack[d]->gpu_block : stack[d]->gpu_thread;
-                if (g || loops_per_dim[stack[d]->gpu_block >= 0 ? 0 : 1][dim] > 1) return;
+                if (stack[d]->gpu_block >= 0) {
+                    // the guard of a block loop is the same for the whole workgroup, unless a thread loop lies outside it
+                    for (size_t o = 0; o < d; o++)
+                        if (stack[o]->gpu_thread >= 0) return left_as_scheduled("wider than a wavefront and inside a block loop that a thread loop encloses");
+                    continue;
+                }
+                if (!g && loops_per_dim[1][stack[d]->gpu_thread] <= 1) continue;
+                // A thread loop with a partial last tile: its threads beyond the tile must still reach the barrier.  The
+                // loop is emitted with a predicate instead of a branch (live_predicates); that cannot hold statements
+                // that declare something for later ones, or a barrier of the program's own.
+                bool plain = true;
+                lir::walk(stack[d]->body, [&](const node_ptr &x) {
+                    if (x->kind == node_kind::cond) plain = false;
+                    if (x->kind == node_kind::leaf && (x->lkind != leaf_kind::assign || !x->lhs)) plain = false;
+                });
+                if (!plain)
+                    return left_as_scheduled("wider than a wavefront and inside a mapped loop with a partial last tile that also holds declarations, barriers or conditions");
+                guarded.push_back(stack[d].get());
             }
+            for (auto g : guarded) predicated_loops.insert(g);
         }
-        reductions[R.get()] = {leaf, term, (int)w};
+        reductions[R.get()] = {leaf, term, (int)w, w != extent};
+    }
+
+    // Thread loops with a partial last tile around a sum across wavefronts: the threads beyond the tile do not branch
+    // around the loop's body but carry a predicate (_live_<iterator>), under which the ordinary statements run; the sum
+    // itself runs for all of them, the dead ones adding zero and skipping the store.
+    std::set<const node *> predicated_loops;
+    std::vector<std::string> live_predicates;
+    std::string all_live() const {
+        std::string c;
+        for (auto &p : live_predicates) c += (c.empty() ? "" : " && ") + p;
+        return c;
+    }
+    bool holds_wide_reduction(const node_ptr &n) const {
+        bool found = false;
+        lir::walk(n, [&](const node_ptr &x) {
+            auto r = reductions.find(x.get());
+            if (r != reductions.end() && r->second.width > 64) found = true;
+        });
+        return found;
+    }
+    void emit_predicated(const node_ptr &n, int ind) {
+        if (!n) return;
+        if (n->kind == node_kind::block) {
+            for (auto &c : n->children) emit_predicated(c, ind);
+            return;
+        }
+        if (n->kind == node_kind::loop && holds_wide_reduction(n)) {
+            emit_loop(n, ind);
+            return;
+        }
+        body << pad(ind) << "if (" << all_live() << ") {\n";
+        emit(n, ind + 1);
+        body << pad(ind) << "}\n";
     }
 
     void emit_thread_reduction(const node_ptr &n, const thread_reduction &r, int ind) {
         bool guard;
         expr first;
-        block_ext[0].push_back(host_extent(n, first, guard));
+        const expr extent = host_extent(n, first, guard);
+        block_ext[0].push_back(r.widened ? expr((int32_t)r.width) : extent);
+        if (r.widened) guard = true;
         const std::string acc = "_partial" + std::to_string(reduction_count++);
         body << pad(ind) << "{\n";
         body << pad(ind + 1) << "float " << acc << " = 0.0f;   // this thread's share of the sum\n";
         body << pad(ind + 1) << "{\n";
         body << pad(ind + 2) << "const int32_t " << n->iterator << " = (int32_t)threadIdx.x + " << dev.print(first) << ";\n";
-        if (guard)
-            body << pad(ind + 2) << "if (" << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+        const std::string live = all_live();
+        if (!live.empty() && !guard) {
+            guard = true;
+            body << pad(ind + 2) << "if (" << live << ") {\n";
+        } else if (guard) {
+            body << pad(ind + 2) << "if (" << (live.empty() ? "" : live + " && ") << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator << " <= " << dev.print(n->upper) << ") {\n";
+        }
         pending_partial = acc;
         pending_leaf = r.leaf.get();
         pending_term = r.term;
@@ -751,7 +834,7 @@ struct generic_kernel_gen {
             body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", _reduction_scratch, "
                  << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
         }
-        body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << ") "
+        body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << (live.empty() ? "" : " && " + live) << ") "
              << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, p_float32) << "\n";
         body << pad(ind) << "}\n";
         add_include_once(ctx, "#include \"wave_reduce.hip.h\"");
@@ -776,10 +859,71 @@ struct generic_kernel_gen {
             }
         };
         split(bound);
-        if (parts.empty()) ERROR("GPU-mapped loop " + what + " has no kernel-invariant bound", true);
+        if (parts.empty()) {
+            // every argument varies inside the kernel (a triangular domain: the bound of one mapped loop is a function
+            // of another's iterator): the launch covers what the bound can reach over the ranges of those iterators
+            expr r;
+            if (!over_the_ranges(bound, combiner == o_min, r)) ERROR("GPU-mapped loop " + what + " has no kernel-invariant bound", true);
+            return lir::simplify(r);
+        }
         expr r = parts[0];
         for (size_t i = 1; i < parts.size(); i++) r = expr(combiner, r, parts[i]);
         return r;
+    }
+
+    // A kernel-invariant upper (or lower) bound of an expression of in-kernel loop iterators: each iterator ranges
+    // over what the host sees of its loop, sums, differences, products with and quotients by literals and min / max
+    // are followed; false for anything else.
+    std::map<std::string, std::vector<node_ptr>> loops_by_iterator;
+    bool over_the_ranges(const expr &e, bool upper, expr &out) {
+        if (!depends_on(e, inner)) { out = e; return true; }
+        if (e.get_expr_type() == e_var) {
+            auto it = loops_by_iterator.find(e.get_name());
+            if (it == loops_by_iterator.end()) return false;
+            bool have = false;
+            for (auto &n : it->second) {
+                expr first; bool guard;
+                const expr ext = host_extent(n, first, guard);
+                const expr v = upper ? lir::simplify(first + ext - 1) : first;
+                out = have ? expr(upper ? o_max : o_min, out, v) : v;
+                have = true;
+            }
+            return have;
+        }
+        if (e.get_expr_type() != e_op) return false;
+        auto literal = [](const expr &x, int64_t &v) {
+            const expr c = lir::simplify(x);
+            if (!c.is_integer_literal()) return false;
+            v = c.get_int_val();
+            return true;
+        };
+        expr a, b;
+        int64_t c;
+        switch (e.get_op_type()) {
+        case o_add:
+            if (!over_the_ranges(e.get_operand(0), upper, a) || !over_the_ranges(e.get_operand(1), upper, b)) return false;
+            out = a + b; return true;
+        case o_sub:
+            if (!over_the_ranges(e.get_operand(0), upper, a) || !over_the_ranges(e.get_operand(1), !upper, b)) return false;
+            out = a - b; return true;
+        case o_mul:
+            for (int side = 0; side < 2; side++)
+                if (literal(e.get_operand(side), c)) {
+                    if (!over_the_ranges(e.get_operand(1 - side), c >= 0 ? upper : !upper, a)) return false;
+                    out = e.get_operand(side) * a; return true;
+                }
+            return false;
+        case o_div: case o_floordiv:
+            if (!literal(e.get_operand(1), c) || c <= 0 || !over_the_ranges(e.get_operand(0), upper, a)) return false;
+            out = expr(e.get_op_type(), a, e.get_operand(1)); return true;
+        case o_min: case o_max:
+            if (!over_the_ranges(e.get_operand(0), upper, a) || !over_the_ranges(e.get_operand(1), upper, b)) return false;
+            out = expr(e.get_op_type(), a, b); return true;
+        case o_cast:
+            if (!over_the_ranges(e.get_operand(0), upper, a)) return false;
+            out = cast(e.get_data_type(), a); return true;
+        default: return false;
+        }
     }
 
     // Extent and first value of a mapped loop as seen from the host.  Bounds that vary inside the
@@ -943,6 +1087,24 @@ struct generic_kernel_gen {
         auto red = reductions.find(n.get());
         if (red != reductions.end()) {
             emit_thread_reduction(n, red->second, ind);
+            return;
+        }
+        if (is_thread && (predicated_loops.count(n.get()) || (!live_predicates.empty() && holds_wide_reduction(n)))) {
+            const int dim = n->gpu_thread;
+            bool guard;
+            expr first;
+            block_ext[dim].push_back(host_extent(n, first, guard));
+            if (loops_per_dim[1][dim] > 1 || predicated_loops.count(n.get())) guard = true;
+            body << pad(ind) << "{\n";
+            body << pad(ind + 1) << "const int32_t " << n->iterator << " = (int32_t)threadIdx." << "xyz"[dim] << " + " << dev.print(first) << ";\n";
+            if (guard) {
+                body << pad(ind + 1) << "const bool _live_" << n->iterator << " = " << n->iterator << " >= " << dev.print(n->init) << " && " << n->iterator
+                     << " <= " << dev.print(n->upper) << ";   // a predicate, not a branch: the sum below has a barrier that every thread must reach\n";
+                live_predicates.push_back("_live_" + n->iterator);
+            }
+            emit_predicated(n->body, ind + 1);
+            if (guard) live_predicates.pop_back();
+            body << pad(ind) << "}\n";
             return;
         }
         if (retile.on && (is_block || is_thread)) {
@@ -1772,7 +1934,9 @@ public:
             k << "// Generated by the Tiramisu HIP back-end for gfx950.  Function: " << f.get_name() << "\n";
             k << "#include <hip/hip_runtime.h>\n#include <stdint.h>\n";
             k << ctx.includes;
-            k << c_prelude(true) << "\n";
+            std::string all_kernels;
+            for (auto &kr : ctx.kernels) all_kernels += kr.source;
+            k << c_prelude(true) << c_prelude_opaque(true, all_kernels) << "\n";
             for (auto &nm : ctx.constant_buffers) {
                 const buffer *b = f.get_buffers().at(nm);
                 long cnt = 1;
@@ -1808,7 +1972,7 @@ public:
             h << "// Generated by the Tiramisu HIP back-end: host glue of function " << f.get_name() << "\n";
             h << "#include <stdint.h>\n#include <stdlib.h>\n#include <string.h>\n#include <math.h>\n#include <map>\n";
             h << "#include <tiramisu_hip_wrappers.h>\n";
-            h << halide_buffer_definition() << c_prelude(false) << "\n";
+            h << halide_buffer_definition() << c_prelude(false) << c_prelude_opaque(false, body.str()) << "\n";
             for (auto &d : hg.extern_decls) h << d << "\n";
             if (device_code) {
                 char *abs_path = realpath(hsaco.c_str(), nullptr);
