@@ -13,7 +13,10 @@
 //                          (the row loop is emitted with a predicate instead of a branch);
 //  * row_sums_100_lanes    31 x 450, two rows of 100 threads: the width is rounded up to two wavefronts, the lanes
 //                          beyond the loop's extent add zero (and the last workgroup has one row);
-//  * row_sums_26_of_64_lanes  80 x 26 split by 64: the thread loop has 26 iterations, the sum runs on 32 lanes.
+//  * row_sums_26_of_64_lanes  80 x 26 split by 64: the thread loop has 26 iterations, the sum runs on 32 lanes;
+//  * row_sums_int32_wave, row_sums_int32_block  the same sums on int32 data (50 x 45 on 16 lanes, four rows per
+//                          workgroup; 33 x 700 on 128 lanes, two rows per workgroup): the lane shifts move 32-bit
+//                          patterns, and a lane without a neighbour adds the all-zero pattern.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -48,13 +51,13 @@ static void gemv_wavefront()
 #endif
 }
 
-static void row_sums(const std::string &name, int M, int N, int rows_per_block, int lanes)
+static void row_sums(const std::string &name, int M, int N, int rows_per_block, int lanes, primitive_t type = p_float32)
 {
     tiramisu::init(name);
     var i("i", 0, M), j("j", 0, N), i0("i0"), i1("i1"), j0("j0"), j1("j1");
-    input A("A", {i, j}, p_float32);
-    computation s_init("s_init", {i}, expr((float)(rows_per_block > 1 ? 1 : 0)));
-    computation s("s", {i, j}, p_float32);
+    input A("A", {i, j}, type);
+    computation s_init("s_init", {i}, cast(type, expr((float)(rows_per_block > 1 ? 1 : 0))));
+    computation s("s", {i, j}, type);
     s.store_in(s_init.get_buffer(), {i});
     s.set_expression(A(i, j) + s(i, 0));     // the element on the right of the sum
     s.split(j, lanes, j0, j1);
@@ -84,5 +87,7 @@ int main()
     row_sums("row_sums_ragged_rows_block", 10, 558, 4, 256);
     row_sums("row_sums_100_lanes", 31, 450, 2, 100);
     row_sums("row_sums_26_of_64_lanes", 80, 26, 1, 64);
+    row_sums("row_sums_int32_wave", 50, 45, 4, 16, p_int32);
+    row_sums("row_sums_int32_block", 33, 700, 2, 128, p_int32);
     return 0;
 }

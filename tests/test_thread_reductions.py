@@ -21,8 +21,11 @@ CASES = {
     "row_sums_ragged_rows_block": (10, 558, 1.0, False),
     "row_sums_100_lanes": (31, 450, 1.0, False),
     "row_sums_26_of_64_lanes": (80, 26, 0.0, False),
+    "row_sums_int32_wave": (50, 45, 1, False),
+    "row_sums_int32_block": (33, 700, 1, False),
 }
-ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes"}
+ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block"}
+INT32 = {"row_sums_int32_wave", "row_sums_int32_block"}
 
 
 def inputs(name, integer, seed):
@@ -30,6 +33,9 @@ def inputs(name, integer, seed):
     rng = np.random.RandomState(seed)
     draw = (lambda shape: (rng.randint(0, 10, shape) - 5).astype(np.float32)) if integer else \
         (lambda shape: rng.uniform(-1, 1, shape).astype(np.float32))
+    if name in INT32:
+        A = rng.randint(-2 ** 20, 2 ** 20, (M, N)).astype(np.int32)
+        return A, None, init + A.sum(axis=1, dtype=np.int64)
     A = draw((M, N))
     x = draw((N,)) if vec else None
     expected = init + (A.astype(np.float64) @ x.astype(np.float64) if vec else A.astype(np.float64).sum(axis=1))
@@ -76,10 +82,10 @@ def test_a_width_between_the_supported_ones_is_rounded_up(programs_dir):
 @pytest.mark.parametrize("name", sorted(CASES))
 def test_cpu_generated_code_matches_numpy(programs_dir, name):
     A, x, expected = inputs(name, True, 1)
-    out = np.full((A.shape[0],), -7.0, np.float32)
+    out = np.full((A.shape[0],), -7, A.dtype)
     cpu = runtime.Program(oracle_build.cpu_program_library(programs_dir, name), name, needs_gpu_runtime=False)
     call(cpu, A, x, out)
-    assert np.array_equal(out, expected.astype(np.float32))
+    assert np.array_equal(out, expected.astype(A.dtype))
 
 
 @pytest.mark.gpu
@@ -87,9 +93,9 @@ def test_cpu_generated_code_matches_numpy(programs_dir, name):
 def test_gpu_matches_numpy(programs_dir, name):
     from gpu_util import DeviceArray, assert_fp32_parity
     prog = runtime.load(programs_dir, name)
-    for integer in (True, False):
+    for integer in (True,) if name in INT32 else (True, False):
         A, x, expected = inputs(name, integer, 2 + integer)
-        out = np.full((A.shape[0],), -7.0, np.float32)
+        out = np.full((A.shape[0],), -7, A.dtype)
         dev = [DeviceArray(a) for a in ([A, out] if x is None else [A, x, out])]
         print("running", name, "integer" if integer else "uniform", flush=True)
         prog(*[d.buffer() for d in dev])
@@ -97,7 +103,7 @@ def test_gpu_matches_numpy(programs_dir, name):
         for d in dev:
             d.free()
         if integer:
-            assert np.array_equal(got, expected.astype(np.float32))
+            assert np.array_equal(got, expected.astype(A.dtype))
         else:
             assert_fp32_parity(got, expected, name + " vs float64 numpy", 1e-4)
 

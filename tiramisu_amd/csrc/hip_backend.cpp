@@ -642,7 +642,7 @@ struct generic_kernel_gen {
     // a sum across the lanes of the wavefront with DPP row shifts and broadcasts (across wavefronts
     // through LDS when the loop is wider than a wavefront), and one read-modify-write of X[e] by the last
     // thread of the loop.
-    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; };   // widened: width exceeds the loop's extent
+    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type; };   // widened: width exceeds the loop's extent
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
     int conds_above = 0;          // conditions between the kernel's root and the node that find_reductions is visiting
@@ -659,7 +659,7 @@ struct generic_kernel_gen {
         if (!n) return;
         if (n->kind == node_kind::loop) stack.push_back(n);
         if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && !n->predicate.is_defined() && n->lets.empty() &&
-            n->rhs.is_defined() && n->rhs.get_data_type() == p_float32 && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
+            n->rhs.is_defined() && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
             consider_reduction(n, stack);
         for (auto &c : n->children) find_reductions(c, stack);
         find_reductions(n->body, stack);
@@ -701,6 +701,9 @@ struct generic_kernel_gen {
             std::cerr << "GPU mapping: the sum " << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
                       << " is emitted as scheduled, its threads race on " << leaf->lhs->get_name() << " (" << why << ")" << std::endl;
         };
+        const primitive_t type = leaf->rhs.get_data_type();
+        if (type != p_float32 && type != p_int32 && type != p_uint32)
+            return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: float, int32_t and uint32_t are");
         if (loops_per_dim[1][0] != 1) return left_as_scheduled("another loop of the kernel is mapped to threadIdx.x as well");
         // inside it: this statement only, under serial loops whose iterators the element does not involve either
         for (size_t d = at + 1; d < stack.size(); d++)
@@ -766,7 +769,7 @@ struct generic_kernel_gen {
             }
             for (auto g : guarded) predicated_loops.insert(g);
         }
-        reductions[R.get()] = {leaf, term, (int)w, w != extent};
+        reductions[R.get()] = {leaf, term, (int)w, w != extent, type};
     }
 
     // Thread loops with a partial last tile around a sum across wavefronts: the threads beyond the tile do not branch
@@ -810,7 +813,8 @@ struct generic_kernel_gen {
         if (r.widened) guard = true;
         const std::string acc = "_partial" + std::to_string(reduction_count++);
         body << pad(ind) << "{\n";
-        body << pad(ind + 1) << "float " << acc << " = 0.0f;   // this thread's share of the sum\n";
+        const std::string ctype = primitive_c_name(r.type);
+        body << pad(ind + 1) << ctype << " " << acc << " = 0;   // this thread's share of the sum\n";
         body << pad(ind + 1) << "{\n";
         body << pad(ind + 2) << "const int32_t " << n->iterator << " = (int32_t)threadIdx.x + " << dev.print(first) << ";\n";
         const std::string live = all_live();
@@ -831,11 +835,11 @@ struct generic_kernel_gen {
             body << pad(ind + 1) << acc << " = twave::wave_group_sum<" << r.width << ">(" << acc << ");\n";
         } else {
             needs_reduction_scratch = true;
-            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", _reduction_scratch, "
+            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", " << (r.type == p_float32 ? "" : "(" + ctype + " *)") << "_reduction_scratch, "
                  << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
         }
         body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << (live.empty() ? "" : " && " + live) << ") "
-             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, p_float32) << "\n";
+             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, r.type) << "\n";
         body << pad(ind) << "}\n";
         add_include_once(ctx, "#include \"wave_reduce.hip.h\"");
         wave_reductions++;

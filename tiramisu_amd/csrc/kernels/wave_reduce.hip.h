@@ -17,13 +17,15 @@
 
 namespace twave {
 
-template <int CTRL, int ROW_MASK, bool ZERO_FILL>
-__device__ __forceinline__ float dpp_term(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, ZERO_FILL));
+// T: float, int32_t or uint32_t (a lane without a neighbour adds the all-zero pattern, which is 0 in each of them)
+template <int CTRL, int ROW_MASK, bool ZERO_FILL, class T>
+__device__ __forceinline__ T dpp_term(T v) {
+    static_assert(sizeof(T) == 4, "DPP moves 32-bit lanes");
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, ZERO_FILL));
 }
 
-template <int W>
-__device__ __forceinline__ float wave_group_sum(float v) {
+template <int W, class T>
+__device__ __forceinline__ T wave_group_sum(T v) {
     static_assert(W >= 2 && W <= 64 && (W & (W - 1)) == 0, "group width must be a power of two up to the wavefront size");
     if (W >= 2) v += dpp_term<0x111, 0xf, true>(v);    // row_shr:1
     if (W >= 4) v += dpp_term<0x112, 0xf, true>(v);    // row_shr:2
@@ -35,13 +37,13 @@ __device__ __forceinline__ float wave_group_sum(float v) {
 }
 
 // `scratch` holds one float per wavefront of the workgroup; `linear` is the thread's linear id.
-template <int W>
-__device__ __forceinline__ float block_group_sum(float v, float *scratch, int linear) {
+template <int W, class T>
+__device__ __forceinline__ T block_group_sum(T v, T *scratch, int linear) {
     static_assert(W % 64 == 0 && W >= 128 && W <= 1024, "group width must be whole wavefronts");
     v = wave_group_sum<64>(v);
     if ((linear & 63) == 63) scratch[linear >> 6] = v;
     __syncthreads();
-    float total = 0.f;
+    T total = 0;
     if ((linear % W) == W - 1) {
         const int last = linear >> 6;
 #pragma unroll
