@@ -1,8 +1,8 @@
 // A sum over a loop of 256 GPU threads that sits under a condition: rows 3 .. 39 of s(i) = sum_j A(i, j) are summed,
 // rows 0 .. 2 only initialised, both statements in one block loop -- so the generated kernel tests the block
 // iterator before the thread loop.  The lowering of such a sum across wavefronts ends in a workgroup barrier,
-// which every thread must reach: the back-end may use it only when nothing conditional lies between the kernel's
-// entry and the loop, and leaves this loop as the program states it.
+// which every thread must reach: a condition on block iterators alone is the same for the whole workgroup, so the
+// sum is lowered below it (a condition that names a thread iterator would keep the loop as the program states it).
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;

@@ -108,26 +108,46 @@ def test_gpu_matches_numpy(programs_dir, name):
             assert_fp32_parity(got, expected, name + " vs float64 numpy", 1e-4)
 
 
-def test_sum_across_wavefronts_under_a_condition_keeps_the_barrier_out(programs_dir):
+def test_sum_across_wavefronts_under_a_condition_on_the_block_iterator(programs_dir):
     """tests/programs/thread_reduction_under_condition.cpp: the 256-thread loop sits under `if (block iterator >= 3)`.
-    The lowering across wavefronts ends in a workgroup barrier that every thread must reach, so the emitter must not
-    use it below a condition: the loop stays as the program states it (no LDS stage, no barrier below the condition)."""
+    The lowering across wavefronts ends in a workgroup barrier that every thread must reach; this condition is the
+    same for all threads of a workgroup, so the sum is lowered below it."""
     text = open(os.path.join(programs_dir, "build", "row_sums_from_row_3.o.hip")).read()
     kernel = text[text.index('extern "C" __global__'):]
     assert "if ((c1 >= 3))" in kernel
-    # (the initialisation above the condition, which no thread loop encloses, runs on the first thread between barriers)
-    assert "block_group_sum" not in kernel and "__syncthreads" not in kernel[kernel.index("if ((c1 >= 3))"):]
-    assert "DPP wavefront reductions" not in re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)
+    assert "block_group_sum<256>" in kernel[kernel.index("if ((c1 >= 3))"):]
+    assert "DPP wavefront reductions" in re.search(r"^// _kernel_\d+: (.*)$", text, re.M).group(1)
 
 
-def test_a_sum_left_as_scheduled_is_reported(programs_dir, tmp_path):
-    """... and the generator says that the threads of that loop race (the reference emits such sums silently,
-    tiramisu_codegen_cuda.cpp:549-707)."""
+@pytest.mark.gpu
+def test_gpu_sum_under_a_condition_on_the_block_iterator(programs_dir):
+    from gpu_util import DeviceArray
+    rng = np.random.RandomState(40)
+    A = (rng.randint(0, 10, (40, 5000)) - 5).astype(np.float32)
+    expected = A.astype(np.float64).sum(axis=1).astype(np.float32)
+    expected[:3] = 0
+    dev = [DeviceArray(A), DeviceArray(np.full(40, -7.0, np.float32))]
+    print("row_sums_from_row_3", flush=True)
+    runtime.load(programs_dir, "row_sums_from_row_3")(*[d.buffer() for d in dev])
+    got = dev[1].download()
+    for d in dev:
+        d.free()
+    assert np.array_equal(got, expected)
+
+
+def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
+    """tests/programs/thread_reduction_left_as_scheduled.cpp: a float64 sum on the lanes, and an update that lies inside
+    one of the kernel's two thread loops only.  The reference emits such code silently
+    (tiramisu_codegen_cuda.cpp:549-707); this back-end generates it as scheduled too and says what will happen."""
     import subprocess
     os.makedirs(os.path.join(str(tmp_path), "build"))
     env = dict(os.environ, HIPCC_PATH="/bin/true", TIRAMISU_HOST_CXX="/bin/true")
-    r = subprocess.run([os.path.join(programs_dir, "build", "gen_thread_reduction_under_condition")], cwd=str(tmp_path), env=env,
+    r = subprocess.run([os.path.join(programs_dir, "build", "gen_thread_reduction_left_as_scheduled")], cwd=str(tmp_path), env=env,
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
-    assert "GPU mapping: the sum s over thread loop c3 of row_sums_from_row_3 is emitted as scheduled, its threads race on" in r.stdout, r.stdout
-    assert "under a condition" in r.stdout
+    assert ("GPU mapping: the sum s over thread loop c3 of row_sums_float64 is emitted as scheduled, its threads race on _s_init_b1 "
+            "(sums of double are not lowered: float, int32_t and uint32_t are)") in r.stdout, r.stdout
+    assert ("GPU mapping: bump of update_inside_one_thread_loop_only updates _s_init_b1 from its own value inside some of the "
+            "kernel's thread loops only: every thread along dimension x repeats the update") in r.stdout, r.stdout
+    # the lowered sum of the second program is not reported
+    assert "the sum s over thread loop c5 of update_inside_one_thread_loop_only" not in r.stdout

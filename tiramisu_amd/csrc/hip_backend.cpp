@@ -645,7 +645,7 @@ struct generic_kernel_gen {
     struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type; };   // widened: width exceeds the loop's extent
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
-    int conds_above = 0;          // conditions between the kernel's root and the node that find_reductions is visiting
+    std::vector<expr> conds_above;     // conditions between the kernel's root and the node that find_reductions is visiting
 
     static bool is_same_element(const expr &e, const buffer *b, const std::vector<expr> &idx) {
         if (e.get_expr_type() != e_op || e.get_op_type() != o_access || e.get_name() != b->get_name() || e.get_access().size() != idx.size())
@@ -661,13 +661,35 @@ struct generic_kernel_gen {
         if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && !n->predicate.is_defined() && n->lets.empty() &&
             n->rhs.is_defined() && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
             consider_reduction(n, stack);
+        if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && n->rhs.is_defined()) repeated_along_a_thread_dimension(n, stack);
         for (auto &c : n->children) find_reductions(c, stack);
         find_reductions(n->body, stack);
-        if (n->kind == node_kind::cond) conds_above++;
+        if (n->kind == node_kind::cond) conds_above.push_back(n->condition);
         find_reductions(n->then_body, stack);
         find_reductions(n->else_body, stack);
-        if (n->kind == node_kind::cond) conds_above--;
+        if (n->kind == node_kind::cond) conds_above.pop_back();
         if (n->kind == node_kind::loop) stack.pop_back();
+    }
+
+    // An update of an element from its own value (x = x + ..., x = f(x)) that lies inside the thread loops of some of
+    // the kernel's thread dimensions but not of all: the threads along the missing dimensions all execute it, so it is
+    // applied that many times (a plain store of one value is merely repeated).  The reference emits the same
+    // (tiramisu_codegen_cuda.cpp:549-707); say so.  Statements outside all thread loops run on one thread instead.
+    void repeated_along_a_thread_dimension(const node_ptr &leaf, const std::vector<node_ptr> &stack) {
+        const memory_location where = leaf->lhs->get_location();
+        if (where != memory_location::global && where != memory_location::shared) return;
+        int inside = 0, used = 0;
+        for (auto &l : stack) if (l->gpu_thread >= 0) inside |= 1 << l->gpu_thread;
+        for (int d = 0; d < 3; d++) if (loops_per_dim[1][d] > 0) used |= 1 << d;
+        if (inside == 0 || inside == used) return;
+        bool reads_itself = false;
+        leaf->rhs.visit([&](const expr &x) { if (is_same_element(x, leaf->lhs, leaf->lhs_index)) reads_itself = true; });
+        if (!reads_itself) return;
+        std::string missing;
+        for (int d = 0; d < 3; d++) if ((used & ~inside) & (1 << d)) missing += std::string(missing.empty() ? "" : ", ") + "xyz"[d];
+        std::cerr << "GPU mapping: " << leaf->comp->get_name() << " of " << f->get_name() << " updates " << leaf->lhs->get_name()
+                  << " from its own value inside some of the kernel's thread loops only: every thread along dimension " << missing
+                  << " repeats the update" << std::endl;
     }
 
     void consider_reduction(const node_ptr &leaf, const std::vector<node_ptr> &stack) {
@@ -740,7 +762,12 @@ struct generic_kernel_gen {
             // thread iterator) between the kernel entry and the loop.  (Adding the wavefronts' totals with
             // atomics instead would need no barrier, but nothing would then order them after an initialisation of
             // the element that other wavefronts of the workgroup execute: the barrier is what does that.)
-            if (conds_above > 0) return left_as_scheduled("wider than a wavefront and under a condition: the barrier of the sum across wavefronts would not be reached by every thread");
+            // a condition on block iterators and kernel parameters alone is the same for the whole workgroup
+            std::set<std::string> varies = inner;
+            for (size_t d = 0; d < at; d++) if (stack[d]->gpu_block >= 0) varies.erase(stack[d]->iterator);
+            for (auto &c : conds_above)
+                if (depends_on(c, varies))
+                    return left_as_scheduled("wider than a wavefront and under a condition that may differ between threads: the barrier of the sum across wavefronts would not be reached by every thread");
             std::vector<const node *> guarded;
             for (size_t d = 0; d < at; d++) {
                 bool g;
