@@ -3,7 +3,8 @@
 //  * row_sums_float64: s(i) = sum_j A(i, j) in float64 on 64 lanes (float, int32_t and uint32_t sums are lowered);
 //  * update_inside_one_thread_loop_only: two rows per workgroup, the row sum on 16 lanes (lowered), and beside its
 //    initialisation a statement bump(i): s(i) = s(i) + 2 that lies inside the loop over rows (threadIdx.y) but outside
-//    the loop over lanes (threadIdx.x): all 16 lanes of a row execute it.
+//    the loop over lanes (threadIdx.x): all 16 lanes of a row execute it;
+//  * row_sums_of_even_columns: the row sum on 64 lanes with a predicate on the statement (j % 2 == 0).
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -57,10 +58,32 @@ static void update_inside_one_thread_loop_only()
     tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/update_inside_one_thread_loop_only.o", true);
 }
 
+static void row_sums_of_even_columns()
+{
+    const int M = 20, N = 300;
+    tiramisu::init("row_sums_of_even_columns");
+    var i("i", 0, M), j("j", 0, N), j0("j0"), j1("j1");
+    input A("A", {i, j}, p_float32);
+    computation s_init("s_init", {i}, expr((float)0));
+    computation s("s", {i, j}, p_float32);
+    s.store_in(s_init.get_buffer(), {i});
+    s.set_expression(A(i, j) + s(i, 0));
+    s.add_predicate(j % 2 == 0);
+    s.split(j, 64, j0, j1);
+    s.interchange(j0, j1);
+    for (buffer *b : {A.get_buffer(), s_init.get_buffer()}) b->tag_gpu_global();
+    s.tag_gpu_block_level(0);
+    s.tag_gpu_thread_level(1);
+    s_init.tag_gpu_block_level(0);
+    s_init.then(s, 0);
+    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/row_sums_of_even_columns.o", true);
+}
+
 int main(int argc, char **argv)
 {
     tiramisu::backend_options_from_command_line(argc, argv);
     row_sums_float64();
     update_inside_one_thread_loop_only();
+    row_sums_of_even_columns();
     return 0;
 }

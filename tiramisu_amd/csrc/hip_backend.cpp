@@ -658,9 +658,9 @@ struct generic_kernel_gen {
     void find_reductions(const node_ptr &n, std::vector<node_ptr> &stack) {
         if (!n) return;
         if (n->kind == node_kind::loop) stack.push_back(n);
-        if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && !n->predicate.is_defined() && n->lets.empty() &&
+        if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs &&
             n->rhs.is_defined() && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
-            consider_reduction(n, stack);
+            consider_reduction(n, stack, !n->predicate.is_defined() && n->lets.empty());
         if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && n->rhs.is_defined()) repeated_along_a_thread_dimension(n, stack);
         for (auto &c : n->children) find_reductions(c, stack);
         find_reductions(n->body, stack);
@@ -692,7 +692,7 @@ struct generic_kernel_gen {
                   << " repeats the update" << std::endl;
     }
 
-    void consider_reduction(const node_ptr &leaf, const std::vector<node_ptr> &stack) {
+    void consider_reduction(const node_ptr &leaf, const std::vector<node_ptr> &stack, bool plain_statement) {
         expr term;
         if (is_same_element(leaf->rhs.get_operand(0), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(1);
         else if (is_same_element(leaf->rhs.get_operand(1), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(0);
@@ -723,6 +723,7 @@ struct generic_kernel_gen {
             std::cerr << "GPU mapping: the sum " << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
                       << " is emitted as scheduled, its threads race on " << leaf->lhs->get_name() << " (" << why << ")" << std::endl;
         };
+        if (!plain_statement) return left_as_scheduled("the statement carries a predicate or scalar definitions");
         const primitive_t type = leaf->rhs.get_data_type();
         if (type != p_float32 && type != p_int32 && type != p_uint32)
             return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: float, int32_t and uint32_t are");
