@@ -16,7 +16,9 @@
 //  * row_sums_26_of_64_lanes  80 x 26 split by 64: the thread loop has 26 iterations, the sum runs on 32 lanes;
 //  * row_sums_int32_wave, row_sums_int32_block  the same sums on int32 data (50 x 45 on 16 lanes, four rows per
 //                          workgroup; 33 x 700 on 128 lanes, two rows per workgroup): the lane shifts move 32-bit
-//                          patterns, and a lane without a neighbour adds the all-zero pattern.
+//                          patterns, and a lane without a neighbour adds the all-zero pattern;
+//  * row_sums_float64_wave, row_sums_int64_block  64-bit sums (37 x 333 on 32 lanes; 21 x 900 on 192 lanes = three
+//                          wavefronts): a value travels between lanes as its two 32-bit halves.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -89,5 +91,7 @@ int main()
     row_sums("row_sums_26_of_64_lanes", 80, 26, 1, 64);
     row_sums("row_sums_int32_wave", 50, 45, 4, 16, p_int32);
     row_sums("row_sums_int32_block", 33, 700, 2, 128, p_int32);
+    row_sums("row_sums_float64_wave", 37, 333, 2, 32, p_float64);
+    row_sums("row_sums_int64_block", 21, 900, 2, 192, p_int64);
     return 0;
 }

@@ -23,9 +23,11 @@ CASES = {
     "row_sums_26_of_64_lanes": (80, 26, 0.0, False),
     "row_sums_int32_wave": (50, 45, 1, False),
     "row_sums_int32_block": (33, 700, 1, False),
+    "row_sums_float64_wave": (37, 333, 1.0, False),
+    "row_sums_int64_block": (21, 900, 1, False),
 }
-ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block"}
-INT32 = {"row_sums_int32_wave", "row_sums_int32_block"}
+ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block", "row_sums_int64_block"}
+INT32 = {"row_sums_int32_wave", "row_sums_int32_block", "row_sums_float64_wave", "row_sums_int64_block"}       # exact sums only
 
 
 def inputs(name, integer, seed):
@@ -34,8 +36,13 @@ def inputs(name, integer, seed):
     draw = (lambda shape: (rng.randint(0, 10, shape) - 5).astype(np.float32)) if integer else \
         (lambda shape: rng.uniform(-1, 1, shape).astype(np.float32))
     if name in INT32:
-        A = rng.randint(-2 ** 20, 2 ** 20, (M, N)).astype(np.int32)
-        return A, None, init + A.sum(axis=1, dtype=np.int64)
+        if name == "row_sums_int64_block":
+            A = rng.randint(-2 ** 50, 2 ** 50, (M, N)).astype(np.int64)
+        elif name == "row_sums_float64_wave":
+            A = rng.randint(-2 ** 40, 2 ** 40, (M, N)).astype(np.float64)         # beyond fp32's 24 bits, exact in fp64
+        else:
+            A = rng.randint(-2 ** 20, 2 ** 20, (M, N)).astype(np.int32)
+        return A, None, init + A.sum(axis=1, dtype=np.float64 if A.dtype == np.float64 else np.int64)
     A = draw((M, N))
     x = draw((N,)) if vec else None
     expected = init + (A.astype(np.float64) @ x.astype(np.float64) if vec else A.astype(np.float64).sum(axis=1))
@@ -136,7 +143,7 @@ def test_gpu_sum_under_a_condition_on_the_block_iterator(programs_dir):
 
 
 def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
-    """tests/programs/thread_reduction_left_as_scheduled.cpp: a float64 sum on the lanes, and an update that lies inside
+    """tests/programs/thread_reduction_left_as_scheduled.cpp: a uint8 sum on the lanes, and an update that lies inside
     one of the kernel's two thread loops only.  The reference emits such code silently
     (tiramisu_codegen_cuda.cpp:549-707); this back-end generates it as scheduled too and says what will happen."""
     import subprocess
@@ -145,8 +152,8 @@ def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
     r = subprocess.run([os.path.join(programs_dir, "build", "gen_thread_reduction_left_as_scheduled")], cwd=str(tmp_path), env=env,
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
-    assert ("GPU mapping: the sum s over thread loop c3 of row_sums_float64 is emitted as scheduled, its threads race on _s_init_b1 "
-            "(sums of double are not lowered: float, int32_t and uint32_t are)") in r.stdout, r.stdout
+    assert ("GPU mapping: the sum s over thread loop c3 of row_sums_uint8 is emitted as scheduled, its threads race on _s_init_b1 "
+            "(sums of uint8_t are not lowered: those of 32- and 64-bit types are)") in r.stdout, r.stdout
     assert ("GPU mapping: bump of update_inside_one_thread_loop_only updates _s_init_b1 from its own value inside some of the "
             "kernel's thread loops only: every thread along dimension x repeats the update") in r.stdout, r.stdout
     assert ("GPU mapping: the sum s over thread loop c3 of row_sums_of_even_columns is emitted as scheduled, its threads race on _s_init_b1 "

@@ -725,8 +725,8 @@ struct generic_kernel_gen {
         };
         if (!plain_statement) return left_as_scheduled("the statement carries a predicate or scalar definitions");
         const primitive_t type = leaf->rhs.get_data_type();
-        if (type != p_float32 && type != p_int32 && type != p_uint32)
-            return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: float, int32_t and uint32_t are");
+        if (primitive_size(type) != 4 && primitive_size(type) != 8)
+            return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: those of 32- and 64-bit types are");
         if (loops_per_dim[1][0] != 1) return left_as_scheduled("another loop of the kernel is mapped to threadIdx.x as well");
         // inside it: this statement only, under serial loops whose iterators the element does not involve either
         for (size_t d = at + 1; d < stack.size(); d++)
@@ -863,7 +863,8 @@ struct generic_kernel_gen {
             body << pad(ind + 1) << acc << " = twave::wave_group_sum<" << r.width << ">(" << acc << ");\n";
         } else {
             needs_reduction_scratch = true;
-            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", " << (r.type == p_float32 ? "" : "(" + ctype + " *)") << "_reduction_scratch, "
+            if (primitive_size(r.type) == 8) wide_reduction_scratch = true;
+            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", " << "(" << ctype << " *)_reduction_scratch, "
                  << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
         }
         body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << (live.empty() ? "" : " && " + live) << ") "
@@ -875,7 +876,7 @@ struct generic_kernel_gen {
     std::string pending_partial;
     const node *pending_leaf = nullptr;
     expr pending_term;
-    bool needs_reduction_scratch = false;
+    bool needs_reduction_scratch = false, wide_reduction_scratch = false;     // wide: a 64-bit sum uses it
     int wave_reductions = 0;
 
     // Kernel-invariant part of a bound that is a min() (upper bounds) or max() (lower bounds) of
@@ -1410,7 +1411,7 @@ static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const
     if (batch && batch_iterator_used)
         os << "    const " << primitive_c_name(global::get_loop_iterator_data_type()) << " " << batch->batch_iterator << " = (int32_t)blockIdx.z + _batch_first;\n";
     for (auto &d : top_decls) os << "    " << d << "\n";
-    if (g.needs_reduction_scratch) os << "    __shared__ float _reduction_scratch[16];\n";
+    if (g.needs_reduction_scratch) os << "    __shared__ " << (g.wide_reduction_scratch ? "double" : "float") << " _reduction_scratch[16];\n";
     if (g.fast_block_dim >= 0) {
         // hardware order l (x fastest) -> XCD l % XCDS, its (l / XCDS)-th workgroup -> tile t of the XCD's share
         const char fast = "xy"[g.fast_block_dim], slow = "xy"[1 - g.fast_block_dim];

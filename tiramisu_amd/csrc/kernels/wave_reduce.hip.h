@@ -17,11 +17,19 @@
 
 namespace twave {
 
-// T: float, int32_t or uint32_t (a lane without a neighbour adds the all-zero pattern, which is 0 in each of them)
+// T: float, double, or a 32- or 64-bit integer (a lane without a neighbour adds the all-zero pattern, which is 0 in each
+// of them); DPP moves 32-bit lanes, so a 64-bit value travels as its two halves.
 template <int CTRL, int ROW_MASK, bool ZERO_FILL, class T>
 __device__ __forceinline__ T dpp_term(T v) {
-    static_assert(sizeof(T) == 4, "DPP moves 32-bit lanes");
-    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, ZERO_FILL));
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit values");
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, ZERO_FILL));
+    } else {
+        const unsigned long long bits = __builtin_bit_cast(unsigned long long, v);
+        const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)bits, CTRL, ROW_MASK, 0xf, ZERO_FILL);
+        const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(bits >> 32), CTRL, ROW_MASK, 0xf, ZERO_FILL);
+        return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | lo);
+    }
 }
 
 template <int W, class T>
