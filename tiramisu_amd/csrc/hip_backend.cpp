@@ -1223,6 +1223,7 @@ struct generic_kernel_gen {
         return 0;
     }
 
+    long shared_bytes = 0;      // of the __shared__ arrays declared so far in this kernel
     std::string declaration(const buffer *b) {
         std::string t = primitive_c_name(b->get_elements_type());
         switch (b->get_location()) {
@@ -1233,6 +1234,7 @@ struct generic_kernel_gen {
                 ERROR("buffer " + b->get_name() + " lives in a GPU kernel and needs constant extents", true);
             long cnt = 1;
             for (auto &d : b->get_dim_sizes()) cnt *= lir::simplify(d).get_int_val();
+            if (b->get_location() == memory_location::shared) shared_bytes += cnt * (long)primitive_size(b->get_elements_type());
             return std::string(b->get_location() == memory_location::shared ? "__shared__ " : "") + t + " " +
                    b->get_name() + "[" + std::to_string(cnt) + "];";
         }
@@ -1398,6 +1400,14 @@ static kernel emit_generic_kernel_impl(context &ctx, const node_ptr &root, const
         long v = strtol(k.block[d].c_str(), &end, 10);
         if (end && *end == 0) threads *= v; else lit = false;
     }
+    // What the hardware will refuse at the launch is refused here, where the program can still be named (the device
+    // compiler accepts both): more than 1024 threads in a workgroup, more than 160 KiB of LDS.
+    if (lit && threads > 1024)
+        ERROR("kernel " + k.name + " of " + f->get_name() + ": a workgroup of " + k.block[0] + " x " + k.block[1] + " x " + k.block[2] + " = " +
+              std::to_string(threads) + " threads; the limit is 1024", true);
+    const long lds = g.shared_bytes + (g.needs_reduction_scratch ? (g.wide_reduction_scratch ? 128 : 64) : 0);
+    if (lds > 160 * 1024)
+        ERROR("kernel " + k.name + " of " + f->get_name() + ": " + std::to_string(lds) + " bytes of shared memory; a workgroup has 163840", true);
     os << "extern \"C\" __global__ void ";
     if (lit) os << "__launch_bounds__(" << threads << ") ";
     os << k.name << "(";
