@@ -1,6 +1,6 @@
 // NO_CPU_VARIANT (the point is what the generator says about the GPU code; nothing here is run)
 // Sums on GPU threads that the back-end does not lower, and says so on stderr instead of emitting the race silently:
-//  * row_sums_uint8: s(i) = sum_j A(i, j) in uint8 on 64 lanes (sums of 32- and 64-bit types are lowered);
+//  * row_sums_bf16: s(i) = sum_j A(i, j) stored as bfloat16 on 64 lanes (sums of integers, float and double are lowered);
 //  * update_inside_one_thread_loop_only: two rows per workgroup, the row sum on 16 lanes (lowered), and beside its
 //    initialisation a statement bump(i): s(i) = s(i) + 2 that lies inside the loop over rows (threadIdx.y) but outside
 //    the loop over lanes (threadIdx.x): all 16 lanes of a row execute it;
@@ -9,14 +9,14 @@
 
 using namespace tiramisu;
 
-static void row_sums_uint8()
+static void row_sums_bf16()
 {
     const int M = 20, N = 300;
-    tiramisu::init("row_sums_uint8");
+    tiramisu::init("row_sums_bf16");
     var i("i", 0, M), j("j", 0, N), j0("j0"), j1("j1");
-    input A("A", {i, j}, p_uint8);
-    computation s_init("s_init", {i}, expr((uint8_t)0));
-    computation s("s", {i, j}, p_uint8);
+    input A("A", {i, j}, p_bfloat16);
+    computation s_init("s_init", {i}, cast(p_bfloat16, expr((float)0)));
+    computation s("s", {i, j}, p_bfloat16);
     s.store_in(s_init.get_buffer(), {i});
     s.set_expression(A(i, j) + s(i, 0));
     s.split(j, 64, j0, j1);
@@ -26,7 +26,7 @@ static void row_sums_uint8()
     s.tag_gpu_thread_level(1);
     s_init.tag_gpu_block_level(0);
     s_init.then(s, 0);
-    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/row_sums_uint8.o", true);
+    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/row_sums_bf16.o", true);
 }
 
 static void update_inside_one_thread_loop_only()
@@ -82,7 +82,7 @@ static void row_sums_of_even_columns()
 int main(int argc, char **argv)
 {
     tiramisu::backend_options_from_command_line(argc, argv);
-    row_sums_uint8();
+    row_sums_bf16();
     update_inside_one_thread_loop_only();
     row_sums_of_even_columns();
     return 0;

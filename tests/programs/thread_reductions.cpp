@@ -18,7 +18,9 @@
 //                          workgroup; 33 x 700 on 128 lanes, two rows per workgroup): the lane shifts move 32-bit
 //                          patterns, and a lane without a neighbour adds the all-zero pattern;
 //  * row_sums_float64_wave, row_sums_int64_block  64-bit sums (37 x 333 on 32 lanes; 21 x 900 on 192 lanes = three
-//                          wavefronts): a value travels between lanes as its two 32-bit halves.
+//                          wavefronts): a value travels between lanes as its two 32-bit halves;
+//  * row_sums_uint8_wave, row_sums_int16_block  sums that wrap (45 x 700 uint8 on 64 lanes, 19 x 1300 int16 on 128):
+//                          the partial sums are 32-bit, the final store truncates -- the same value modulo 2^8, 2^16.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -93,5 +95,7 @@ int main()
     row_sums("row_sums_int32_block", 33, 700, 2, 128, p_int32);
     row_sums("row_sums_float64_wave", 37, 333, 2, 32, p_float64);
     row_sums("row_sums_int64_block", 21, 900, 2, 192, p_int64);
+    row_sums("row_sums_uint8_wave", 45, 700, 1, 64, p_uint8);
+    row_sums("row_sums_int16_block", 19, 1300, 2, 128, p_int16);
     return 0;
 }

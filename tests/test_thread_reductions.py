@@ -25,9 +25,11 @@ CASES = {
     "row_sums_int32_block": (33, 700, 1, False),
     "row_sums_float64_wave": (37, 333, 1.0, False),
     "row_sums_int64_block": (21, 900, 1, False),
+    "row_sums_uint8_wave": (45, 700, 0, False),
+    "row_sums_int16_block": (19, 1300, 1, False),
 }
-ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block", "row_sums_int64_block"}
-INT32 = {"row_sums_int32_wave", "row_sums_int32_block", "row_sums_float64_wave", "row_sums_int64_block"}       # exact sums only
+ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block", "row_sums_int64_block", "row_sums_int16_block"}
+INT32 = {"row_sums_int32_wave", "row_sums_int32_block", "row_sums_float64_wave", "row_sums_int64_block", "row_sums_uint8_wave", "row_sums_int16_block"}       # exact sums only
 
 
 def inputs(name, integer, seed):
@@ -36,6 +38,12 @@ def inputs(name, integer, seed):
     draw = (lambda shape: (rng.randint(0, 10, shape) - 5).astype(np.float32)) if integer else \
         (lambda shape: rng.uniform(-1, 1, shape).astype(np.float32))
     if name in INT32:
+        if name == "row_sums_uint8_wave":
+            A = rng.randint(0, 256, (M, N)).astype(np.uint8)
+            return A, None, ((init + A.sum(axis=1, dtype=np.int64)) % 256)
+        if name == "row_sums_int16_block":
+            A = rng.randint(-2 ** 15, 2 ** 15, (M, N)).astype(np.int16)
+            return A, None, (init + A.sum(axis=1, dtype=np.int64)).astype(np.int16)          # wraps
         if name == "row_sums_int64_block":
             A = rng.randint(-2 ** 50, 2 ** 50, (M, N)).astype(np.int64)
         elif name == "row_sums_float64_wave":
@@ -89,7 +97,7 @@ def test_a_width_between_the_supported_ones_is_rounded_up(programs_dir):
 @pytest.mark.parametrize("name", sorted(CASES))
 def test_cpu_generated_code_matches_numpy(programs_dir, name):
     A, x, expected = inputs(name, True, 1)
-    out = np.full((A.shape[0],), -7, A.dtype)
+    out = np.full((A.shape[0],), 7, A.dtype)
     cpu = runtime.Program(oracle_build.cpu_program_library(programs_dir, name), name, needs_gpu_runtime=False)
     call(cpu, A, x, out)
     assert np.array_equal(out, expected.astype(A.dtype))
@@ -102,7 +110,7 @@ def test_gpu_matches_numpy(programs_dir, name):
     prog = runtime.load(programs_dir, name)
     for integer in (True,) if name in INT32 else (True, False):
         A, x, expected = inputs(name, integer, 2 + integer)
-        out = np.full((A.shape[0],), -7, A.dtype)
+        out = np.full((A.shape[0],), 7, A.dtype)
         dev = [DeviceArray(a) for a in ([A, out] if x is None else [A, x, out])]
         print("running", name, "integer" if integer else "uniform", flush=True)
         prog(*[d.buffer() for d in dev])
@@ -143,7 +151,7 @@ def test_gpu_sum_under_a_condition_on_the_block_iterator(programs_dir):
 
 
 def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
-    """tests/programs/thread_reduction_left_as_scheduled.cpp: a uint8 sum on the lanes, and an update that lies inside
+    """tests/programs/thread_reduction_left_as_scheduled.cpp: a bfloat16 sum on the lanes, and an update that lies inside
     one of the kernel's two thread loops only.  The reference emits such code silently
     (tiramisu_codegen_cuda.cpp:549-707); this back-end generates it as scheduled too and says what will happen."""
     import subprocess
@@ -152,8 +160,8 @@ def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
     r = subprocess.run([os.path.join(programs_dir, "build", "gen_thread_reduction_left_as_scheduled")], cwd=str(tmp_path), env=env,
                        stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
-    assert ("GPU mapping: the sum s over thread loop c3 of row_sums_uint8 is emitted as scheduled, its threads race on _s_init_b1 "
-            "(sums of uint8_t are not lowered: those of 32- and 64-bit types are)") in r.stdout, r.stdout
+    assert ("GPU mapping: the sum s over thread loop c3 of row_sums_bf16 is emitted as scheduled, its threads race on _s_init_b1 "
+            "(sums of tiramisu_bf16_t are not lowered: those of integers, float and double are)") in r.stdout, r.stdout
     assert ("GPU mapping: bump of update_inside_one_thread_loop_only updates _s_init_b1 from its own value inside some of the "
             "kernel's thread loops only: every thread along dimension x repeats the update") in r.stdout, r.stdout
     assert ("GPU mapping: the sum s over thread loop c3 of row_sums_of_even_columns is emitted as scheduled, its threads race on _s_init_b1 "

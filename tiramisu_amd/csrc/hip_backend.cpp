@@ -642,7 +642,7 @@ struct generic_kernel_gen {
     // a sum across the lanes of the wavefront with DPP row shifts and broadcasts (across wavefronts
     // through LDS when the loop is wider than a wavefront), and one read-modify-write of X[e] by the last
     // thread of the loop.
-    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type; };   // widened: width exceeds the loop's extent
+    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type, element_type; };   // widened: width exceeds the loop's extent; type: of the partial sums
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
     std::vector<expr> conds_above;     // conditions between the kernel's root and the node that find_reductions is visiting
@@ -725,8 +725,12 @@ struct generic_kernel_gen {
         };
         if (!plain_statement) return left_as_scheduled("the statement carries a predicate or scalar definitions");
         const primitive_t type = leaf->rhs.get_data_type();
-        if (primitive_size(type) != 4 && primitive_size(type) != 8)
-            return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: those of 32- and 64-bit types are");
+        // 8- and 16-bit integers wrap, and the wrap commutes with addition: their partial sums are kept in 32 bits and the
+        // final store truncates
+        primitive_t partial_type = type;
+        if (type == p_int8 || type == p_int16 || type == p_uint8 || type == p_uint16) partial_type = p_uint32;   // unsigned: wraps, never overflows
+        else if (primitive_size(type) != 4 && primitive_size(type) != 8)
+            return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: those of integers, float and double are");
         if (loops_per_dim[1][0] != 1) return left_as_scheduled("another loop of the kernel is mapped to threadIdx.x as well");
         // inside it: this statement only, under serial loops whose iterators the element does not involve either
         for (size_t d = at + 1; d < stack.size(); d++)
@@ -797,7 +801,7 @@ struct generic_kernel_gen {
             }
             for (auto g : guarded) predicated_loops.insert(g);
         }
-        reductions[R.get()] = {leaf, term, (int)w, w != extent, type};
+        reductions[R.get()] = {leaf, term, (int)w, w != extent, partial_type, type};
     }
 
     // Thread loops with a partial last tile around a sum across wavefronts: the threads beyond the tile do not branch
@@ -868,7 +872,7 @@ struct generic_kernel_gen {
                  << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
         }
         body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << (live.empty() ? "" : " && " + live) << ") "
-             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, r.type) << "\n";
+             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, r.element_type) << "\n";
         body << pad(ind) << "}\n";
         add_include_once(ctx, "#include \"wave_reduce.hip.h\"");
         wave_reductions++;
