@@ -20,7 +20,9 @@
 //  * row_sums_float64_wave, row_sums_int64_block  64-bit sums (37 x 333 on 32 lanes; 21 x 900 on 192 lanes = three
 //                          wavefronts): a value travels between lanes as its two 32-bit halves;
 //  * row_sums_uint8_wave, row_sums_int16_block  sums that wrap (45 x 700 uint8 on 64 lanes, 19 x 1300 int16 on 128):
-//                          the partial sums are 32-bit, the final store truncates -- the same value modulo 2^8, 2^16.
+//                          the partial sums are 32-bit, the final store truncates -- the same value modulo 2^8, 2^16;
+//  * row_maxima_wave, row_minima_int32_block, row_maxima_int8_wave  m(i) = max (min) over j of A(i, j): the same
+//                          lowering with another operation; a lane without a neighbour contributes its identity.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -83,6 +85,35 @@ static void row_sums(const std::string &name, int M, int N, int rows_per_block, 
 #endif
 }
 
+// the same with a maximum or a minimum instead of the sum: m(i) = max_j A(i, j), starting from A(i, 0)
+static void row_extremes(const std::string &name, int M, int N, int rows_per_block, int lanes, primitive_t type, op_t op)
+{
+    tiramisu::init(name);
+    var i("i", 0, M), j("j", 0, N), i0("i0"), i1("i1"), j0("j0"), j1("j1");
+    input A("A", {i, j}, type);
+    computation m_init("m_init", {i}, A(i, 0));
+    computation m("m", {i, j}, type);
+    m.store_in(m_init.get_buffer(), {i});
+    m.set_expression(expr(op, m(i, 0), A(i, j)));
+    m.split(j, lanes, j0, j1);
+    m.interchange(j0, j1);
+    m.split(i, rows_per_block, i0, i1);
+    m_init.split(i, rows_per_block, i0, i1);
+#ifndef TIRAMISU_TARGET_CPU
+    for (buffer *b : {A.get_buffer(), m_init.get_buffer()}) b->tag_gpu_global();
+    m.tag_gpu_block_level(0);
+    m.tag_gpu_thread_level(1, 2);
+    m_init.tag_gpu_block_level(0);
+    m_init.tag_gpu_thread_level(1);
+#endif
+    m_init.then(m, i1);
+#ifdef TIRAMISU_TARGET_CPU
+    tiramisu::codegen({A.get_buffer(), m_init.get_buffer()}, "build/" + name + "_cpu.o", false);
+#else
+    tiramisu::codegen({A.get_buffer(), m_init.get_buffer()}, "build/" + name + ".o", true);
+#endif
+}
+
 int main()
 {
     gemv_wavefront();
@@ -97,5 +128,8 @@ int main()
     row_sums("row_sums_int64_block", 21, 900, 2, 192, p_int64);
     row_sums("row_sums_uint8_wave", 45, 700, 1, 64, p_uint8);
     row_sums("row_sums_int16_block", 19, 1300, 2, 128, p_int16);
+    row_extremes("row_maxima_wave", 41, 500, 2, 64, p_float32, o_max);
+    row_extremes("row_minima_int32_block", 10, 900, 4, 256, p_int32, o_min);
+    row_extremes("row_maxima_int8_wave", 30, 333, 4, 16, p_int8, o_max);
     return 0;
 }

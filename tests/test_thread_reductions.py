@@ -27,9 +27,13 @@ CASES = {
     "row_sums_int64_block": (21, 900, 1, False),
     "row_sums_uint8_wave": (45, 700, 0, False),
     "row_sums_int16_block": (19, 1300, 1, False),
+    "row_maxima_wave": (41, 500, None, False),
+    "row_minima_int32_block": (10, 900, None, False),
+    "row_maxima_int8_wave": (30, 333, None, False),
 }
-ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block", "row_sums_int64_block", "row_sums_int16_block"}
-INT32 = {"row_sums_int32_wave", "row_sums_int32_block", "row_sums_float64_wave", "row_sums_int64_block", "row_sums_uint8_wave", "row_sums_int16_block"}       # exact sums only
+EXTREMES = {"row_maxima_wave": (np.float32, np.max), "row_minima_int32_block": (np.int32, np.min), "row_maxima_int8_wave": (np.int8, np.max)}
+ACROSS_WAVEFRONTS = {"row_sums_block", "row_sums_ragged_rows_block", "row_sums_100_lanes", "row_sums_int32_block", "row_sums_int64_block", "row_sums_int16_block", "row_minima_int32_block"}
+INT32 = {"row_sums_int32_wave", "row_sums_int32_block", "row_sums_float64_wave", "row_sums_int64_block", "row_sums_uint8_wave", "row_sums_int16_block", "row_maxima_wave", "row_minima_int32_block", "row_maxima_int8_wave"}       # exact sums only
 
 
 def inputs(name, integer, seed):
@@ -37,6 +41,10 @@ def inputs(name, integer, seed):
     rng = np.random.RandomState(seed)
     draw = (lambda shape: (rng.randint(0, 10, shape) - 5).astype(np.float32)) if integer else \
         (lambda shape: rng.uniform(-1, 1, shape).astype(np.float32))
+    if name in EXTREMES:
+        dtype, pick = EXTREMES[name]
+        A = rng.uniform(-1000, 1000, (M, N)).astype(dtype) if dtype == np.float32 else rng.randint(np.iinfo(dtype).min, np.iinfo(dtype).max + 1, (M, N)).astype(dtype)
+        return A, None, pick(A, axis=1)
     if name in INT32:
         if name == "row_sums_uint8_wave":
             A = rng.randint(0, 256, (M, N)).astype(np.uint8)

@@ -642,7 +642,7 @@ struct generic_kernel_gen {
     // a sum across the lanes of the wavefront with DPP row shifts and broadcasts (across wavefronts
     // through LDS when the loop is wider than a wavefront), and one read-modify-write of X[e] by the last
     // thread of the loop.
-    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type, element_type; };   // widened: width exceeds the loop's extent; type: of the partial sums
+    struct thread_reduction { node_ptr leaf; expr term; int width; bool widened; primitive_t type, element_type; op_t op; };   // widened: width exceeds the loop's extent; type: of the partial sums; op: o_add, o_max or o_min
     std::map<const node *, thread_reduction> reductions;   // keyed by the threadIdx.x loop
     int reduction_count = 0;
     std::vector<expr> conds_above;     // conditions between the kernel's root and the node that find_reductions is visiting
@@ -659,7 +659,8 @@ struct generic_kernel_gen {
         if (!n) return;
         if (n->kind == node_kind::loop) stack.push_back(n);
         if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs &&
-            n->rhs.is_defined() && n->rhs.get_expr_type() == e_op && n->rhs.get_op_type() == o_add)
+            n->rhs.is_defined() && n->rhs.get_expr_type() == e_op &&
+            (n->rhs.get_op_type() == o_add || n->rhs.get_op_type() == o_max || n->rhs.get_op_type() == o_min))
             consider_reduction(n, stack, !n->predicate.is_defined() && n->lets.empty());
         if (n->kind == node_kind::leaf && n->lkind == leaf_kind::assign && n->lhs && n->rhs.is_defined()) repeated_along_a_thread_dimension(n, stack);
         for (auto &c : n->children) find_reductions(c, stack);
@@ -720,7 +721,7 @@ struct generic_kernel_gen {
         // is not lowered it is emitted as scheduled, like the reference does (tiramisu_codegen_cuda.cpp:549-707):
         // the threads race and the result is wrong, so say so.
         auto left_as_scheduled = [&](const std::string &why) {
-            std::cerr << "GPU mapping: the sum " << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
+            std::cerr << "GPU mapping: the " << (leaf->rhs.get_op_type() == o_add ? "sum " : leaf->rhs.get_op_type() == o_max ? "maximum " : "minimum ") << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
                       << " is emitted as scheduled, its threads race on " << leaf->lhs->get_name() << " (" << why << ")" << std::endl;
         };
         if (!plain_statement) return left_as_scheduled("the statement carries a predicate or scalar definitions");
@@ -728,8 +729,15 @@ struct generic_kernel_gen {
         // 8- and 16-bit integers wrap, and the wrap commutes with addition: their partial sums are kept in 32 bits and the
         // final store truncates
         primitive_t partial_type = type;
-        if (type == p_int8 || type == p_int16 || type == p_uint8 || type == p_uint16) partial_type = p_uint32;   // unsigned: wraps, never overflows
-        else if (primitive_size(type) != 4 && primitive_size(type) != 8)
+        const op_t op = leaf->rhs.get_op_type();
+        if (op == o_add) {
+            if (type == p_int8 || type == p_int16 || type == p_uint8 || type == p_uint16) partial_type = p_uint32;   // unsigned: wraps, never overflows
+        } else {
+            // a maximum or minimum: widening keeps the order
+            if (type == p_int8 || type == p_int16) partial_type = p_int32;
+            else if (type == p_uint8 || type == p_uint16) partial_type = p_uint32;
+        }
+        if (primitive_size(partial_type) != 4 && primitive_size(partial_type) != 8)
             return left_as_scheduled("sums of " + primitive_c_name(type) + " are not lowered: those of integers, float and double are");
         if (loops_per_dim[1][0] != 1) return left_as_scheduled("another loop of the kernel is mapped to threadIdx.x as well");
         // inside it: this statement only, under serial loops whose iterators the element does not involve either
@@ -801,7 +809,7 @@ struct generic_kernel_gen {
             }
             for (auto g : guarded) predicated_loops.insert(g);
         }
-        reductions[R.get()] = {leaf, term, (int)w, w != extent, partial_type, type};
+        reductions[R.get()] = {leaf, term, (int)w, w != extent, partial_type, type, op};
     }
 
     // Thread loops with a partial last tile around a sum across wavefronts: the threads beyond the tile do not branch
@@ -846,7 +854,12 @@ struct generic_kernel_gen {
         const std::string acc = "_partial" + std::to_string(reduction_count++);
         body << pad(ind) << "{\n";
         const std::string ctype = primitive_c_name(r.type);
-        body << pad(ind + 1) << ctype << " " << acc << " = 0;   // this thread's share of the sum\n";
+        const std::string opname = r.op == o_max ? "twave::max_op" : r.op == o_min ? "twave::min_op" : "";
+        auto combine = [&](const std::string &a, const std::string &b) {
+            return r.op == o_add ? a + " + " + b : std::string(r.op == o_max ? "t_max" : "t_min") + "((" + ctype + ")(" + a + "), (" + ctype + ")(" + b + "))";
+        };
+        body << pad(ind + 1) << ctype << " " << acc << " = " << (r.op == o_add ? "0" : opname + "::identity<" + ctype + ">()")
+             << ";   // this thread's share of the " << (r.op == o_add ? "sum" : r.op == o_max ? "maximum" : "minimum") << "\n";
         body << pad(ind + 1) << "{\n";
         body << pad(ind + 2) << "const int32_t " << n->iterator << " = (int32_t)threadIdx.x + " << dev.print(first) << ";\n";
         const std::string live = all_live();
@@ -859,24 +872,27 @@ struct generic_kernel_gen {
         pending_partial = acc;
         pending_leaf = r.leaf.get();
         pending_term = r.term;
+        pending_combine = combine;
         emit(n->body, ind + (guard ? 3 : 2));
         pending_leaf = nullptr;
         if (guard) body << pad(ind + 2) << "}\n";
         body << pad(ind + 1) << "}\n";
         if (r.width <= 64) {
-            body << pad(ind + 1) << acc << " = twave::wave_group_sum<" << r.width << ">(" << acc << ");\n";
+            if (r.op == o_add) body << pad(ind + 1) << acc << " = twave::wave_group_sum<" << r.width << ">(" << acc << ");\n";
+            else body << pad(ind + 1) << acc << " = twave::wave_group_reduce<" << r.width << ", " << opname << ">(" << acc << ");\n";
         } else {
             needs_reduction_scratch = true;
             if (primitive_size(r.type) == 8) wide_reduction_scratch = true;
-            body << pad(ind + 1) << acc << " = twave::block_group_sum<" << r.width << ">(" << acc << ", " << "(" << ctype << " *)_reduction_scratch, "
+            body << pad(ind + 1) << acc << " = twave::" << (r.op == o_add ? "block_group_sum<" + std::to_string(r.width) : "block_group_reduce<" + std::to_string(r.width) + ", " + opname) << ">(" << acc << ", " << "(" << ctype << " *)_reduction_scratch, "
                  << "(int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z)));\n";
         }
         body << pad(ind + 1) << "if (threadIdx.x == " << r.width - 1 << (live.empty() ? "" : " && " + live) << ") "
-             << dev.store(r.leaf->lhs, r.leaf->lhs_index, dev.element(r.leaf->lhs, r.leaf->lhs_index) + " + " + acc, r.element_type) << "\n";
+             << dev.store(r.leaf->lhs, r.leaf->lhs_index, combine(dev.element(r.leaf->lhs, r.leaf->lhs_index), acc), r.op == o_add ? r.element_type : r.type) << "\n";
         body << pad(ind) << "}\n";
         add_include_once(ctx, "#include \"wave_reduce.hip.h\"");
         wave_reductions++;
     }
+    std::function<std::string(const std::string &, const std::string &)> pending_combine;
     std::string pending_partial;
     const node *pending_leaf = nullptr;
     expr pending_term;
@@ -1250,7 +1266,7 @@ struct generic_kernel_gen {
 
     void emit_leaf(const node_ptr &n, int ind) {
         if (n.get() == pending_leaf) {
-            body << pad(ind) << pending_partial << " = " << pending_partial << " + " << dev.print(pending_term) << ";\n";
+            body << pad(ind) << pending_partial << " = " << pending_combine(pending_partial, dev.print(pending_term)) << ";\n";
             return;
         }
         switch (n->lkind) {
