@@ -4,7 +4,8 @@
 //  * update_inside_one_thread_loop_only: two rows per workgroup, the row sum on 16 lanes (lowered), and beside its
 //    initialisation a statement bump(i): s(i) = s(i) + 2 that lies inside the loop over rows (threadIdx.y) but outside
 //    the loop over lanes (threadIdx.x): all 16 lanes of a row execute it;
-//  * row_sums_of_even_columns: the row sum on 64 lanes with a predicate on the statement (j % 2 == 0).
+//  * row_sums_of_even_columns: the row sum on 64 lanes with a predicate on the statement (j % 2 == 0);
+//  * tile_sums: s(b) = sum over y, x of A(b, y, x) with both y and x mapped to threads.
 #include <tiramisu/tiramisu.h>
 
 using namespace tiramisu;
@@ -79,11 +80,29 @@ static void row_sums_of_even_columns()
     tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/row_sums_of_even_columns.o", true);
 }
 
+static void tile_sums()
+{
+    tiramisu::init("tile_sums");
+    var b("b", 0, 30), y("y", 0, 8), x("x", 0, 16);
+    input A("A", {b, y, x}, p_float32);
+    computation s_init("s_init", {b}, expr((float)0));
+    computation s("s", {b, y, x}, p_float32);
+    s.store_in(s_init.get_buffer(), {b});
+    s.set_expression(A(b, y, x) + s(b, 0, 0));
+    for (buffer *buf : {A.get_buffer(), s_init.get_buffer()}) buf->tag_gpu_global();
+    s.tag_gpu_block_level(0);
+    s.tag_gpu_thread_level(1, 2);
+    s_init.tag_gpu_block_level(0);
+    s_init.then(s, 0);
+    tiramisu::codegen({A.get_buffer(), s_init.get_buffer()}, "build/tile_sums.o", true);
+}
+
 int main(int argc, char **argv)
 {
     tiramisu::backend_options_from_command_line(argc, argv);
     row_sums_bf16();
     update_inside_one_thread_loop_only();
     row_sums_of_even_columns();
+    tile_sums();
     return 0;
 }

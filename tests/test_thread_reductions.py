@@ -174,5 +174,7 @@ def test_sums_left_as_scheduled_are_reported(programs_dir, tmp_path):
             "kernel's thread loops only: every thread along dimension x repeats the update") in r.stdout, r.stdout
     assert ("GPU mapping: the sum s over thread loop c3 of row_sums_of_even_columns is emitted as scheduled, its threads race on _s_init_b1 "
             "(the statement carries a predicate or scalar definitions)") in r.stdout, r.stdout
+    assert ("GPU mapping: the sum s over thread loop c3 of tile_sums is emitted as scheduled, its threads race on _s_init_b1 "
+            "(it runs over several thread loops, or over one that is not on threadIdx.x)") in r.stdout, r.stdout
     # the lowered sum of the second program is not reported
     assert "the sum s over thread loop c5 of update_inside_one_thread_loop_only" not in r.stdout

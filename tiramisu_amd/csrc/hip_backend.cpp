@@ -694,6 +694,9 @@ struct generic_kernel_gen {
     }
 
     void consider_reduction(const node_ptr &leaf, const std::vector<node_ptr> &stack, bool plain_statement) {
+        // registers and thread-local arrays are a thread's own: nothing is shared, whatever the index says
+        const memory_location where = leaf->lhs->get_location();
+        if (where != memory_location::global && where != memory_location::shared) return;
         expr term;
         if (is_same_element(leaf->rhs.get_operand(0), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(1);
         else if (is_same_element(leaf->rhs.get_operand(1), leaf->lhs, leaf->lhs_index)) term = leaf->rhs.get_operand(0);
@@ -710,11 +713,14 @@ struct generic_kernel_gen {
         // the thread-mapped loops around the statement that its element does not involve
         node_ptr R;
         size_t at = 0;
+        bool not_one_loop_on_x = false;     // the lowering takes one loop, on threadIdx.x (consecutive lanes)
         for (size_t d = 0; d < stack.size(); d++)
             if (stack[d]->gpu_thread >= 0 && !element_involves(stack[d]->iterator)) {
-                if (R || stack[d]->gpu_thread != 0) return;     // one loop, on threadIdx.x (consecutive lanes)
-                R = stack[d];
-                at = d;
+                if (R || stack[d]->gpu_thread != 0) not_one_loop_on_x = true;
+                if (!R) {
+                    R = stack[d];
+                    at = d;
+                }
             }
         if (!R) return;
         // From here on the statement is known to be a sum that all threads of loop R add to one element.  Where it
@@ -724,6 +730,7 @@ struct generic_kernel_gen {
             std::cerr << "GPU mapping: the " << (leaf->rhs.get_op_type() == o_add ? "sum " : leaf->rhs.get_op_type() == o_max ? "maximum " : "minimum ") << leaf->comp->get_name() << " over thread loop " << R->iterator << " of " << f->get_name()
                       << " is emitted as scheduled, its threads race on " << leaf->lhs->get_name() << " (" << why << ")" << std::endl;
         };
+        if (not_one_loop_on_x) return left_as_scheduled("it runs over several thread loops, or over one that is not on threadIdx.x");
         if (!plain_statement) return left_as_scheduled("the statement carries a predicate or scalar definitions");
         const primitive_t type = leaf->rhs.get_data_type();
         // 8- and 16-bit integers wrap, and the wrap commutes with addition: their partial sums are kept in 32 bits and the
